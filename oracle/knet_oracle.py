@@ -1,0 +1,352 @@
+"""ctypes front end of the CPU oracle (``oracle/knet_cpu.c``).
+
+TEST INFRASTRUCTURE: only the tests, the smoke check and the benchmark's CPU
+baseline may import this module.  Arrays are numpy arrays carrying Julia shapes;
+memory order is column-major (``order='F'``) exactly as Knet's ``Array`` path.
+Dimension numbers (``dims``) and labels are 1-based as in the reference.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libknet_oracle.so")
+
+REDUCTION_OPS = ["sum", "prod", "maximum", "minimum", "sumabs", "sumabs2", "maxabs", "minabs", "countnz"]
+
+
+def build(force=False):
+    """Compile the oracle with gcc (``make -C oracle``)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.ko_const.restype = ctypes.c_double
+        _lib.ko_findindices.restype = ctypes.c_long
+        _lib.ko_nll_32.restype = ctypes.c_float
+        _lib.ko_nll_64.restype = ctypes.c_double
+    return _lib
+
+
+def _sfx(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return "32", ctypes.c_float
+    if dtype == np.float64:
+        return "64", ctypes.c_double
+    raise TypeError("oracle supports float32/float64, got %s" % dtype)
+
+
+def _flat(a, dtype=None):
+    a = np.asarray(a, dtype=dtype)
+    return np.ascontiguousarray(a.ravel(order="F"))
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _shape_like(flat, shape):
+    return flat.reshape(shape, order="F")
+
+
+def const(which):
+    return lib().ko_const({"lambda01": 0, "alpha01": 1, "lambdaalpha01": 2}[which])
+
+
+def unary(name, x):
+    s, _ = _sfx(x.dtype)
+    xf = _flat(x)
+    y = np.empty_like(xf)
+    getattr(lib(), "ko_%s_%s" % (name, s))(ctypes.c_long(xf.size), _ptr(xf), _ptr(y))
+    return _shape_like(y, np.shape(x))
+
+
+def back11(name, dy, y):
+    """Two-input gradient ``name(dy, y) -> dx`` (reluback, sigmback, tanhback, eluback, seluback)."""
+    s, _ = _sfx(dy.dtype)
+    assert dy.dtype == y.dtype
+    dyf, yf = _flat(dy), _flat(y)
+    dx = np.empty_like(dyf)
+    getattr(lib(), "ko_%s_%s" % (name, s))(ctypes.c_long(dyf.size), _ptr(dyf), _ptr(yf), _ptr(dx))
+    return _shape_like(dx, np.shape(dy))
+
+
+def back111(name, x, y, dy):
+    """Three-input gradient ``name(x, y, dy) -> dx`` (ops21 family, e.g. ``geluback``)."""
+    s, _ = _sfx(x.dtype)
+    xf, yf, dyf = _flat(x), _flat(y), _flat(dy)
+    dx = np.empty_like(xf)
+    getattr(lib(), "ko_%s_111_%s" % (name, s))(ctypes.c_long(xf.size), _ptr(xf), _ptr(yf), _ptr(dyf), _ptr(dx))
+    return _shape_like(dx, np.shape(x))
+
+
+def relu_kw(x, max_value=np.inf, negative_slope=0.0, threshold=0.0):
+    s, ct = _sfx(x.dtype)
+    xf = _flat(x)
+    y = np.empty_like(xf)
+    getattr(lib(), "ko_relu_1_%s" % s)(ctypes.c_long(xf.size), ct(max_value), ct(negative_slope), ct(threshold), _ptr(xf), _ptr(y))
+    return _shape_like(y, np.shape(x))
+
+
+def reluback_kw(x, y, dy, max_value=np.inf, negative_slope=0.0, threshold=0.0):
+    s, ct = _sfx(x.dtype)
+    xf, yf, dyf = _flat(x), _flat(y), _flat(dy)
+    dx = np.empty_like(xf)
+    getattr(lib(), "ko_reluback_1_%s" % s)(ctypes.c_long(xf.size), ct(max_value), ct(negative_slope), ct(threshold),
+                                           _ptr(xf), _ptr(yf), _ptr(dyf), _ptr(dx))
+    return _shape_like(dx, np.shape(x))
+
+
+def _norm_dims(dims, nd):
+    if dims is None or dims == ":":
+        return list(range(1, nd + 1))
+    if isinstance(dims, (int, np.integer)):
+        dims = [int(dims)]
+    return sorted(set(int(d) for d in dims))
+
+
+def reduce(op, x, dims=None):
+    """``op(x; dims)`` keeping singleton dims (``dims=None`` reduces everything to a scalar)."""
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    nd = max(x.ndim, 1)
+    shape = x.shape if x.ndim else (1,)
+    dl = _norm_dims(dims, nd)
+    mask = (ctypes.c_int * nd)(*[1 if (k + 1) in dl else 0 for k in range(nd)])
+    cdims = (ctypes.c_long * nd)(*shape)
+    yshape = tuple(1 if (k + 1) in dl else shape[k] for k in range(nd))
+    xf = _flat(x)
+    y = np.empty(int(np.prod(yshape)), dtype=x.dtype)
+    getattr(lib(), "ko_reduce_%s" % s)(ctypes.c_int(REDUCTION_OPS.index(op)), ctypes.c_int(nd), cdims, mask, _ptr(xf), _ptr(y))
+    if dims is None or dims == ":":
+        return y[0]
+    return _shape_like(y, yshape)
+
+
+def _view3(shape, dims):
+    """(inner, d, outer) for a softmax along the contiguous group of 1-based ``dims``."""
+    nd = len(shape)
+    dl = _norm_dims(dims, nd)
+    if dl != list(range(dl[0], dl[-1] + 1)):
+        raise ValueError("oracle softmax needs adjacent dims, got %r" % (dims,))
+    inner = int(np.prod(shape[: dl[0] - 1], dtype=np.int64))
+    d = int(np.prod(shape[dl[0] - 1: dl[-1]], dtype=np.int64))
+    outer = int(np.prod(shape[dl[-1]:], dtype=np.int64))
+    return inner, d, outer
+
+
+def _softmax_fwd(name, x, dims):
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    inner, d, outer = _view3(x.shape, dims)
+    xf = _flat(x)
+    y = np.empty_like(xf)
+    getattr(lib(), "ko_%s_%s" % (name, s))(ctypes.c_long(inner), ctypes.c_long(d), ctypes.c_long(outer), _ptr(xf), _ptr(y))
+    return _shape_like(y, x.shape)
+
+
+def logsoftmax(x, dims=None):
+    return _softmax_fwd("logsoftmax", x, dims)
+
+
+def softmax(x, dims=None):
+    return _softmax_fwd("softmax", x, dims)
+
+
+def _softmax_bwd(name, y, dy, dims):
+    y = np.asarray(y)
+    s, _ = _sfx(y.dtype)
+    inner, d, outer = _view3(y.shape, dims)
+    yf, dyf = _flat(y), _flat(dy, y.dtype)
+    dx = np.empty_like(yf)
+    getattr(lib(), "ko_%s_%s" % (name, s))(ctypes.c_long(inner), ctypes.c_long(d), ctypes.c_long(outer), _ptr(yf), _ptr(dyf), _ptr(dx))
+    return _shape_like(dx, y.shape)
+
+
+def logsoftmaxback(y, dy, dims=None):
+    return _softmax_bwd("logsoftmaxback", y, dy, dims)
+
+
+def softmaxback(y, dy, dims=None):
+    return _softmax_bwd("softmaxback", y, dy, dims)
+
+
+def logsumexp(x, dims=None):
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    inner, d, outer = _view3(x.shape, dims)
+    dl = _norm_dims(dims, x.ndim)
+    yshape = tuple(1 if (k + 1) in dl else x.shape[k] for k in range(x.ndim))
+    xf = _flat(x)
+    y = np.empty(inner * outer, dtype=x.dtype)
+    getattr(lib(), "ko_logsumexp_%s" % s)(ctypes.c_long(inner), ctypes.c_long(d), ctypes.c_long(outer), _ptr(xf), _ptr(y))
+    return _shape_like(y, yshape)
+
+
+def logsumexpback(x, y, dy, dims=None):
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    inner, d, outer = _view3(x.shape, dims)
+    xf, yf, dyf = _flat(x), _flat(y, x.dtype), _flat(dy, x.dtype)
+    dx = np.empty_like(xf)
+    getattr(lib(), "ko_logsumexpback_%s" % s)(ctypes.c_long(inner), ctypes.c_long(d), ctypes.c_long(outer), _ptr(xf), _ptr(yf), _ptr(dyf), _ptr(dx))
+    return _shape_like(dx, x.shape)
+
+
+def findindices(scores_shape, labels, dims=1):
+    """1-based linear indices of the labelled entries (label 0 skipped)."""
+    labels = _flat(labels, np.int32)
+    y1 = int(scores_shape[0]) if dims == 1 else int(np.prod(scores_shape[:-1], dtype=np.int64))
+    total = int(np.prod(scores_shape, dtype=np.int64))
+    y2 = total // y1 if y1 else 0
+    out = np.empty(max(labels.size, 1), dtype=np.int64)
+    n = lib().ko_findindices(ctypes.c_long(y1), ctypes.c_long(y2), _ptr(labels), ctypes.c_long(labels.size), ctypes.c_int(dims), _ptr(out))
+    if n == -1:
+        raise ValueError("DimensionMismatch")
+    if n == -2:
+        raise ValueError("findindices only supports dims = 1 or 2")
+    return out[:n].copy()
+
+
+def nll(scores, labels, dims=1, average=True):
+    scores = np.asarray(scores)
+    s, _ = _sfx(scores.dtype)
+    y1, y2 = scores.shape
+    sf, lf = _flat(scores), _flat(labels, np.int32)
+    cnt = ctypes.c_long(0)
+    v = getattr(lib(), "ko_nll_%s" % s)(ctypes.c_long(y1), ctypes.c_long(y2), _ptr(sf), _ptr(lf), ctypes.c_int(dims), ctypes.byref(cnt))
+    v = scores.dtype.type(v)
+    if average:
+        return v
+    return scores.dtype.type(v * scores.dtype.type(cnt.value)), cnt.value
+
+
+def nll_back(scores, labels, dims=1):
+    scores = np.asarray(scores)
+    s, _ = _sfx(scores.dtype)
+    y1, y2 = scores.shape
+    sf, lf = _flat(scores), _flat(labels, np.int32)
+    dx = np.empty_like(sf)
+    getattr(lib(), "ko_nll_back_%s" % s)(ctypes.c_long(y1), ctypes.c_long(y2), _ptr(sf), _ptr(lf), ctypes.c_int(dims), _ptr(dx))
+    return _shape_like(dx, scores.shape)
+
+
+def getents(x, ents):
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    xf, ef = _flat(x), _flat(ents, np.int32)
+    y = np.empty(ef.size, dtype=x.dtype)
+    getattr(lib(), "ko_getents_%s" % s)(ctypes.c_long(ef.size), _ptr(ef), _ptr(xf), _ptr(y))
+    return y
+
+
+def addents(x, ents, y):
+    """Returns a copy of ``x`` with ``y`` scatter-added at the 1-based linear indices ``ents``."""
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    xf, ef, yf = _flat(x).copy(), _flat(ents, np.int32), _flat(y, x.dtype)
+    getattr(lib(), "ko_addents_%s" % s)(ctypes.c_long(ef.size), _ptr(ef), _ptr(xf), _ptr(yf))
+    return _shape_like(xf, x.shape)
+
+
+def dropout(x, p, u):
+    """``dropout!``: ``u`` is the uniform buffer the reference draws with ``rand!``."""
+    x = np.asarray(x)
+    s, ct = _sfx(x.dtype)
+    xf, y = _flat(x), _flat(u, x.dtype).copy()
+    getattr(lib(), "ko_dropout_%s" % s)(ctypes.c_long(xf.size), ct(p), _ptr(xf), _ptr(y))
+    return _shape_like(y, x.shape)
+
+
+def dropback(p, x, y, dy):
+    y = np.asarray(y)
+    s, ct = _sfx(y.dtype)
+    xf, yf, dyf = _flat(x, y.dtype), _flat(y), _flat(dy, y.dtype)
+    dx = np.empty_like(yf)
+    getattr(lib(), "ko_dropback_%s" % s)(ctypes.c_long(yf.size), ct(p), _ptr(xf), _ptr(yf), _ptr(dyf), _ptr(dx))
+    return _shape_like(dx, y.shape)
+
+
+def add_bias(x, b):
+    """``x .+ b`` where ``b`` has one non-singleton dim (the ``_12`` vector broadcast)."""
+    x, b = np.asarray(x), np.asarray(b)
+    s, _ = _sfx(x.dtype)
+    k = [i for i, d in enumerate(b.shape) if d > 1]
+    k = k[0] if k else 0
+    sb = int(np.prod(x.shape[:k], dtype=np.int64))
+    nb = b.size
+    xf, bf = _flat(x), _flat(b, x.dtype)
+    z = np.empty_like(xf)
+    getattr(lib(), "ko_add_12_%s" % s)(ctypes.c_long(xf.size), _ptr(xf), _ptr(bf), ctypes.c_long(sb), ctypes.c_long(nb), _ptr(z))
+    return _shape_like(z, x.shape)
+
+
+def gemm(A, B, ta=False, tb=False):
+    """Column-major ``op(A)*op(B)`` with wide accumulation."""
+    A, B = np.asarray(A), np.asarray(B)
+    s, _ = _sfx(A.dtype)
+    m = A.shape[1] if ta else A.shape[0]
+    k = A.shape[0] if ta else A.shape[1]
+    n = B.shape[0] if tb else B.shape[1]
+    Af, Bf = _flat(A), _flat(B)
+    C = np.empty(m * n, dtype=A.dtype)
+    getattr(lib(), "ko_gemm_%s" % s)(ctypes.c_int(int(ta)), ctypes.c_int(int(tb)), ctypes.c_long(m), ctypes.c_long(n), ctypes.c_long(k),
+                                     _ptr(Af), ctypes.c_long(A.shape[0]), _ptr(Bf), ctypes.c_long(B.shape[0]), _ptr(C), ctypes.c_long(m))
+    return _shape_like(C, (m, n))
+
+
+def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None):
+    """Reference MLP step: ``x = relu.(w*x .+ b)`` per hidden layer (+ dropout with the given
+    uniform buffers), ``nll`` on the last layer's scores; returns (loss, [dW1, db1, dW2, ...]).
+
+    Follows the model of examples/mnist-mlp/mlp.jl:25-35 and the gradient expressions the
+    reference registers for each primitive (matmul: src/knetarrays/linalg.jl:11-18; bias:
+    ``sum(dy;dims=2)``; relu: ``reluback.(dy,y)``; dropout: ``dropback``; nll: ``ko_nll_back``).
+    """
+    nl = len(weights) // 2
+    acts = [np.asarray(x)]
+    saved = []
+    h = acts[0]
+    for l in range(nl):
+        w, b = weights[2 * l], weights[2 * l + 1]
+        z = add_bias(gemm(w, h), b)
+        if l < nl - 1:
+            y = unary("relu", z)
+            if pdrop > 0:
+                yd = dropout(y, pdrop, uniforms[l])
+                saved.append((h, y, yd))
+                h = yd
+            else:
+                saved.append((h, y, None))
+                h = y
+        else:
+            saved.append((h, None, None))
+            h = z
+    loss = nll(h, labels)
+    dz = nll_back(h, labels)
+    grads = [None] * (2 * nl)
+    for l in reversed(range(nl)):
+        hin, y, yd = saved[l]
+        if l < nl - 1:
+            if yd is not None:
+                dz = dropback(pdrop, y, yd, dz)
+            dz = back11("reluback", dz, y)
+        grads[2 * l + 1] = reduce("sum", dz, dims=2)
+        grads[2 * l] = gemm(dz, hin, tb=True)
+        if l > 0:
+            dz = gemm(weights[2 * l], dz, ta=True)
+    return loss, grads
