@@ -1,0 +1,22 @@
+"""Host-side mirror of the part of Knet.jl that sits on the backward-pass gradient path, backed by the
+hand-written gfx950 kernels of ``libknet8.so``.
+
+Names, argument order, 1-based ``dims``/labels and error behaviour follow the reference's Julia API
+(``KnetArray``, ``relu``/``reluback``, ``sum(x; dims)``, ``logsoftmax``, ``nll``, ``dropout``, ``@diff``/``grad``/
+``value`` as ``diff``/``grad``/``value``).  Importing the package loads the library; there is no CPU fallback.
+"""
+from .libknet8 import libknet8, knet8, LIB_PATH
+from .karray import KnetArray, KnetPtr, Array, synchronize
+from .autograd import Param, diff, grad, value, recording
+from .activation import (relu, sigm, tanh, elu, selu, reluback, sigmback, tanhback, eluback, seluback,
+                         gelu, hardsigmoid, hardswish, swish, tanh_, geluback, hardsigmoidback, hardswishback,
+                         swishback, tanh_back, eluback21, seluback21, sigmback21, relu_kw, relu_kw_back,
+                         unary_op, back11_op, back111_op)
+from .reduction import sum, prod, maximum, minimum, sumabs, sumabs2, maxabs, minabs, countnz, reduce_op
+from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
+from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback
+from .loss import nll, findindices, accuracy, getindex, ungetindex
+from .dropout import dropout, dropback, dropout_, dropback_
+from .linalg import matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose
+
+libknet8()  # fail loudly at import time if the HIP library is missing

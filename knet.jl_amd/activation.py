@@ -1,0 +1,132 @@
+"""Activation functions and their gradients on ``KnetArray``.
+
+Mirrors src/ops20_gpu/activation.jl:16-47 (``relu/sigm/elu/selu`` -> ``F_S``; ``*back(dy,y)`` ->
+``Fback_S_11``; ``tanh`` gradient specialised for device arrays, ``:11-13``) and
+src/ops21_gpu/activation.jl:10-49 (``f(x)`` / ``fback(x,y,dy)`` -> ``F_S`` / ``Fback_S_111``; relu with
+keyword arguments -> ``relu_S_1`` / ``reluback_S_1``).  In Julia these are reached by broadcasting
+(``relu.(x)``, ``reluback.(dy,y)``); here the functions take whole arrays.
+"""
+import math
+
+from .autograd import primitive
+from .karray import KnetArray
+from .libknet8 import knet8
+
+
+def _check(*arrays):
+    a0 = arrays[0]
+    for a in arrays:
+        if not isinstance(a, KnetArray):
+            raise TypeError("MethodError: expected KnetArray arguments, got %s" % type(a).__name__)
+        if a.dtype != a0.dtype:
+            raise TypeError("MethodError: element types differ (%s, %s)" % (a0.dtype, a.dtype))
+        if a.length != a0.length:
+            raise ValueError("DimensionMismatch: %r vs %r" % (a0.dims, a.dims))
+    if a0.suffix is None:
+        raise TypeError("MethodError: no kernel for %s" % a0.dtype)
+
+
+def unary_op(name, x):
+    """``y = similar(x); @knet8(F_S, (Cint,Ptr,Ptr), length(y), x, y)`` (src/ops20_gpu/activation.jl:20-24)."""
+    _check(x)
+    y = x.similar()
+    knet8("%s_%s" % (name, x.suffix), x.length, x.ptr, y.ptr)
+    return y
+
+
+def back11_op(name, dy, y):
+    """``z = similar(x); @knet8(Fback_S_11, ..., length(z), dy, y, z)`` (src/ops20_gpu/activation.jl:33-37)."""
+    _check(dy, y)
+    dx = dy.similar()
+    knet8("%s_%s_11" % (name, dy.suffix), dx.length, dy.ptr, y.ptr, dx.ptr)
+    return dx
+
+
+def back111_op(name, x, y, dy):
+    """``dx = similar(x); @knet8(Fback_S_111, ..., length(dx), x, y, dy, dx)`` (src/ops21_gpu/activation.jl:23-27)."""
+    _check(x, y, dy)
+    dx = x.similar()
+    knet8("%s_%s_111" % (name, x.suffix), dx.length, x.ptr, y.ptr, dy.ptr, dx.ptr)
+    return dx
+
+
+def reluback(dy, y):
+    return back11_op("reluback", dy, y)
+
+
+def sigmback(dy, y):
+    return back11_op("sigmback", dy, y)
+
+
+def tanhback(dy, y):
+    return back11_op("tanhback", dy, y)
+
+
+def eluback(dy, y):
+    return back11_op("eluback", dy, y)
+
+
+def seluback(dy, y):
+    return back11_op("seluback", dy, y)
+
+
+def _activation(name, back):
+    @primitive
+    def f(x):
+        y = unary_op(name, x)
+        return y, (lambda dy: (back(dy, y),))  # @primitive relu(x),dy,y reluback.(dy,y)  (src/ops20/activation.jl:28)
+
+    f.__name__ = name
+    return f
+
+
+relu = _activation("relu", reluback)
+sigm = _activation("sigm", sigmback)
+tanh = _activation("tanh", tanhback)
+elu = _activation("elu", eluback)
+selu = _activation("selu", seluback)
+
+
+# ---- ops21: f(x) and fback(x,y,dy) ----------------------------------------------------------------------
+
+def _activation21(name, backname):
+    def back(x, y, dy):
+        return back111_op(backname, x, y, dy)
+
+    @primitive
+    def f(x):
+        y = unary_op(name, x)
+        return y, (lambda dy: (back(x, y, dy),))  # @primitive1 gelu(x),dy,y geluback(x,y,dy)  (src/ops21/activation.jl:43)
+
+    f.__name__ = name
+    back.__name__ = backname
+    return f, back
+
+
+gelu, geluback = _activation21("gelu", "geluback")
+hardsigmoid, hardsigmoidback = _activation21("hardsigmoid", "hardsigmoidback")
+hardswish, hardswishback = _activation21("hardswish", "hardswishback")
+swish, swishback = _activation21("swish", "swishback")
+tanh_, tanh_back = _activation21("tanh_", "tanh_back")
+_, eluback21 = _activation21("elu", "eluback")
+_, seluback21 = _activation21("selu", "seluback")
+_, sigmback21 = _activation21("sigm", "sigmback")
+
+
+def relu_kw_back(x, y, dy, max_value=math.inf, negative_slope=0, threshold=0):
+    """``reluback(x,y,dy; max_value, negative_slope, threshold)`` (src/ops21_gpu/activation.jl:43-47)."""
+    _check(x, y, dy)
+    dx = x.similar()
+    c = x.ctype
+    knet8("reluback_%s_1" % x.suffix, dx.length, c(max_value), c(negative_slope), c(threshold), x.ptr, y.ptr, dy.ptr, dx.ptr)
+    return dx
+
+
+@primitive
+def relu_kw(x, max_value=math.inf, negative_slope=0, threshold=0):
+    """``relu(x; max_value, negative_slope, threshold)`` (src/ops21_gpu/activation.jl:37-41)."""
+    _check(x)
+    y = x.similar()
+    c = x.ctype
+    knet8("relu_%s_1" % x.suffix, y.length, c(max_value), c(negative_slope), c(threshold), x.ptr, y.ptr)
+    return y, (lambda dy: (relu_kw_back(x, y, dy, max_value, negative_slope, threshold),))

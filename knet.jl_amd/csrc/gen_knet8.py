@@ -1,0 +1,388 @@
+#!/usr/bin/env python3
+"""Generator of libknet8's gfx950 HIP sources and of its public header.
+
+Plays the role of the reference's src/libknet8/build.jl:42-82 + ops.jl: the operator tables below
+are the configuration; each row becomes a device functor plus the ``extern "C"`` entry points
+(``NAME_stream(..., hipStream_t)`` and the plain ``NAME`` twin) that Knet's ``@knet8`` ccall layer
+binds (src/libknet8/LibKnet8.jl:50-62).  The kernels themselves are the hand-written templates in
+knet8_elementwise.h / knet8_reduce.h / knet8_softmax.h / knet8_index.h.
+
+Expressions follow the reference's CPU ``Array`` path (src/ops20/activation.jl, src/ops21/activation.jl)
+where it differs from the expressions compiled into the reference's CUDA kernels
+(src/libknet8/ops.jl): ``>=`` branch tests for elu/selu, selu constants rounded to T before use,
+NaN-propagating relu, division (not multiplication by a reciprocal) in dropout.
+
+Usage:  python gen_knet8.py   (writes gen/*.hip next to this file and include/knet8.h at the repo root)
+"""
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+GEN = os.path.join(HERE, "gen")
+HEADER = os.path.join(ROOT, "include", "knet8.h")
+
+TYPES = [("float", "32"), ("double", "64")]
+
+LAMBDA01 = "1.0507009873554805"
+LAMBDAALPHA01 = "1.7580993408473773"
+SQRT2 = "1.4142135623730951"
+SQRT2PI = "2.5066282746310002"
+
+# name, body (statements ending in a return; `xi` is the input), reference citation
+UNARY_OPS = [
+    ("relu", "return xi != xi ? xi : (xi > T(0) ? xi : T(0));", "src/ops20/activation.jl:26, src/libknet8/ops.jl:76"),
+    ("sigm", "if (xi >= T(0)) return T(1) / (T(1) + kexp(-xi)); const T z = kexp(xi); return z / (T(1) + z);",
+     "src/ops20/activation.jl:55, src/libknet8/ops.jl:78"),
+    ("tanh", "return ktanh(xi);", "src/libknet8/ops.jl:61"),
+    ("tanh_", "return ktanh(xi);", "src/ops21/activation.jl:186, src/libknet8/ops.jl:62"),
+    ("elu", "return xi >= T(0) ? xi : kexp(xi) - T(1);", "src/ops20/activation.jl:12, src/libknet8/ops.jl:72"),
+    ("selu", "return xi >= T(0) ? T(%s) * xi : T(%s) * (kexp(xi) - T(1));" % (LAMBDA01, LAMBDAALPHA01),
+     "src/ops20/activation.jl:39, src/libknet8/ops.jl:77"),
+    ("gelu", "const T a = xi / T(%s); const T b = T(1) + kerf(a); const T c = xi * b; return c / T(2);" % SQRT2,
+     "src/ops21/activation.jl:37, src/libknet8/ops.jl:73"),
+    ("hardsigmoid", "return xi <= T(-3) ? T(0) : xi >= T(3) ? T(1) : (xi + T(3)) / T(6);",
+     "src/ops21/activation.jl:61, src/libknet8/ops.jl:74"),
+    ("hardswish", "if (xi <= T(-3)) return T(0); if (xi >= T(3)) return xi; const T a = xi + T(3); const T b = xi * a; return b / T(6);",
+     "src/ops21/activation.jl:81, src/libknet8/ops.jl:75"),
+    ("swish", "T s; if (xi >= T(0)) s = T(1) / (T(1) + kexp(-xi)); else { const T z = kexp(xi); s = z / (T(1) + z); } return xi * s;",
+     "src/ops21/activation.jl:170, src/libknet8/ops.jl:79"),
+    ("exp", "return kexp(xi);", "src/libknet8/ops.jl:26"),
+    ("log", "return klog(xi);", "src/libknet8/ops.jl:40"),
+    ("sqrt", "return ksqrt(xi);", "src/libknet8/ops.jl:58"),
+    ("neg", "return -xi;", "src/libknet8/ops.jl:49"),
+    ("abs", "return xi < T(0) ? -xi : xi;", "src/libknet8/ops.jl:8"),
+    ("abs2", "return xi * xi;", "src/libknet8/ops.jl:7"),
+    ("sign", "return xi > T(0) ? T(1) : xi < T(0) ? T(-1) : T(0);", "src/libknet8/ops.jl:55"),
+    ("invx", "return T(1) / xi;", "src/libknet8/ops.jl:71"),
+    ("one", "return T(1);", "src/libknet8/ops.jl:52"),
+    ("zero", "return T(0);", "src/libknet8/ops.jl:67"),
+]
+
+# name, body in terms of (xi, yi), citation.  Used for the _01, _11 and _12/_13 entry points.
+BINARY_OPS = [
+    ("add", "return xi + yi;", "src/libknet8/ops.jl:88"),
+    ("sub", "return xi - yi;", "src/libknet8/ops.jl:89"),
+    ("mul", "return xi * yi;", "src/libknet8/ops.jl:90"),
+    ("div", "return xi / yi;", "src/libknet8/ops.jl:91"),
+    ("max", "return xi > yi ? xi : yi;", "src/libknet8/ops.jl:93"),
+    ("min", "return xi < yi ? xi : yi;", "src/libknet8/ops.jl:94"),
+]
+
+# Two-input gradients NAME_S_11(n, dy, y, dx): xi = dy, yi = y.
+BACK11_OPS = [
+    ("reluback", "return yi > T(0) ? xi : T(0);", "src/ops20/activation.jl:27, src/libknet8/ops.jl:118"),
+    ("sigmback", "const T a = xi * yi; const T b = T(1) - yi; return a * b;", "src/ops20/activation.jl:56, src/libknet8/ops.jl:120"),
+    ("tanhback", "const T a = yi * yi; const T b = T(1) - a; return xi * b;", "src/ops20_gpu/activation.jl:11, src/libknet8/ops.jl:121"),
+    ("eluback", "if (yi >= T(0)) return xi; const T b = T(1) + yi; return xi * b;", "src/ops20/activation.jl:13, src/libknet8/ops.jl:116"),
+    ("seluback", "if (yi >= T(0)) return xi * T(%s); const T b = yi + T(%s); return xi * b;" % (LAMBDA01, LAMBDAALPHA01),
+     "src/ops20/activation.jl:40, src/libknet8/ops.jl:119"),
+]
+
+# Three-input gradients NAME_S_111(n, x, y, dy, dx).
+BACK111_OPS = [
+    ("eluback", "if (y >= T(0)) return dy; const T b = T(1) + y; return dy * b;", "src/ops21/activation.jl:17, src/libknet8/ops.jl:126"),
+    ("seluback", "if (y >= T(0)) return dy * T(%s); const T b = y + T(%s); return dy * b;" % (LAMBDA01, LAMBDAALPHA01),
+     "src/ops21/activation.jl:130, src/libknet8/ops.jl:132"),
+    ("sigmback", "const T a = dy * y; const T b = T(1) - y; return a * b;", "src/ops21/activation.jl:152, src/libknet8/ops.jl:133"),
+    ("tanh_back", "const T a = y * y; const T b = T(1) - a; return dy * b;", "src/ops21/activation.jl:187, src/libknet8/ops.jl:134"),
+    ("geluback", "const T a = x / T(%s); const T b = (T(1) + kerf(a)) / T(2); const T x2 = x * x; const T e = kexp(-x2 / T(2)); "
+                 "const T c = (x * e) / T(%s); const T d = b + c; return dy * d;" % (SQRT2, SQRT2PI),
+     "src/ops21/activation.jl:38, src/libknet8/ops.jl:127"),
+    ("hardsigmoidback", "const T g = x <= T(-3) ? T(0) : x >= T(3) ? T(0) : T(1.0 / 6.0); return dy * g;",
+     "src/ops21/activation.jl:62, src/libknet8/ops.jl:128"),
+    ("hardswishback", "T g; if (x <= T(-3)) g = T(0); else if (x >= T(3)) g = T(1); else { const T a = T(2) * x; const T b = a + T(3); g = b / T(6); } return dy * g;",
+     "src/ops21/activation.jl:82, src/libknet8/ops.jl:129"),
+    ("swishback", "T g; if (x >= T(0)) { const T z = kexp(-x); const T zx = z * x; const T num = (zx + z) + T(1); const T d = z + T(1); g = num / (d * d); } "
+                  "else { const T z = kexp(x); const T s = (x + z) + T(1); const T num = z * s; const T d = z + T(1); g = num / (d * d); } return dy * g;",
+     "src/ops21/activation.jl:171, src/libknet8/ops.jl:135"),
+]
+
+# Reduction operators: order and meaning of src/libknet8/ops.jl:144-156.
+REDUCTION_OPS = [("sum", "RedSum"), ("prod", "RedProd"), ("maximum", "RedMaximum"), ("minimum", "RedMinimum"),
+                 ("sumabs", "RedSumabs"), ("sumabs2", "RedSumabs2"), ("maxabs", "RedMaxabs"), ("minabs", "RedMinabs"),
+                 ("countnz", "RedCountnz")]
+
+BANNER = "// GENERATED by knet.jl_amd/csrc/gen_knet8.py -- edit the tables there, not this file.\n"
+
+
+class Out:
+    """Collects the HIP source of one translation unit and the matching header declarations."""
+
+    def __init__(self):
+        self.src = []
+        self.decl = []
+
+    def entry(self, name, ret, params, call, cite, guard="", body=None):
+        """Emit NAME_stream(params..., hipStream_t) and the plain NAME twin (null stream)."""
+        plist = ", ".join("%s %s" % (t, n) for t, n in params)
+        pnames = ", ".join(n for _, n in params)
+        sep = ", " if params else ""
+        self.decl.append("/* replaces %s */" % cite)
+        self.decl.append("KNET8_API %s %s_stream(%s%shipStream_t stream);" % (ret, name, plist, sep))
+        self.decl.append("KNET8_API %s %s(%s);" % (ret, name, plist))
+        if body is None:
+            body = "  %s%s;\n  knet8::check_launch(\"%s\");" % (guard, call, name)
+        self.src.append("extern \"C\" KNET8_API %s %s_stream(%s%shipStream_t stream) {\n%s\n}" % (ret, name, plist, sep, body))
+        r = "return " if ret != "void" else ""
+        self.src.append("extern \"C\" KNET8_API %s %s(%s) { %s%s_stream(%s%s0); }\n" % (ret, name, plist, r, name, pnames, sep))
+
+
+PRELUDE = BANNER + """#include "../knet8_runtime.h"
+#include "../knet8_elementwise.h"
+#include "../knet8_reduce.h"
+#include "../knet8_softmax.h"
+#include "../knet8_index.h"
+#include "../knet8_transpose.h"
+using namespace knet8;
+
+"""
+
+
+def functor(name, args, body, extra_fields=""):
+    return ("template <typename T> struct %s {\n%s  __device__ __forceinline__ T operator()(%s) const { %s }\n};\n"
+            % (name, extra_fields, ", ".join("T " + a for a in args), body))
+
+
+def gen_elementwise():
+    o = Out()
+    s = o.src
+    s.append(PRELUDE)
+    o.decl.append("\n/* ---- elementwise forward: y[i] = f(x[i]) -- src/libknet8/cuda1.jl:13-38 ---- */")
+    for name, body, cite in UNARY_OPS:
+        s.append(functor("Op_" + name, ["xi"], body))
+        for T, S in TYPES:
+            o.entry("%s_%s" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y")],
+                    "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, y, Op_%s<%s>())" % (T, T, T, name, T), cite)
+    o.decl.append("\n/* ---- scalar (op) array: z[i] = f(xi, y[i]) -- src/libknet8/cuda01.jl:11-25 ---- */")
+    for name, body, cite in BINARY_OPS:
+        s.append(functor("Op2_" + name, ["xi", "yi"], body))
+        s.append("template <typename T> struct Op01_%s { T xi; __device__ __forceinline__ T operator()(T yi) const { return Op2_%s<T>()(xi, yi); } };\n" % (name, name))
+        for T, S in TYPES:
+            o.entry("%s_%s_01" % (name, S), "void", [("int", "n"), (T, "xi"), (T + "*", "y"), (T + "*", "z")],
+                    "launch_ew<%s, 1>(stream, n, y, (const %s*)nullptr, (const %s*)nullptr, z, Op01_%s<%s>{xi})" % (T, T, T, name, T), cite)
+    o.decl.append("\n/* ---- same-shape binary: z[i] = f(x[i], y[i]) -- src/libknet8/cuda11.jl:12-28 ---- */")
+    for name, body, cite in BINARY_OPS:
+        for T, S in TYPES:
+            o.entry("%s_%s_11" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y"), (T + "*", "z")],
+                    "launch_ew<%s, 2>(stream, n, x, y, (const %s*)nullptr, z, Op2_%s<%s>())" % (T, T, name, T), cite)
+    o.decl.append("\n/* ---- vector broadcast: operand k is full size or a vector along one dim, read as v[(i/s)%n]\n"
+                  "   -- src/libknet8/cuda12.jl:18-34; the _13 forms (src/libknet8/cuda13.jl:44-184) take the full array first ---- */")
+    for name, body, cite in BINARY_OPS:
+        s.append("template <typename T> struct Op2r_%s { __device__ __forceinline__ T operator()(T full, T vec) const { return Op2_%s<T>()(vec, full); } };\n" % (name, name))
+        for T, S in TYPES:
+            o.entry("%s_%s_12" % (name, S), "void",
+                    [("int", "n"), (T + "*", "x"), ("int", "sx"), ("int", "nx"), (T + "*", "y"), ("int", "sy"), ("int", "ny"), (T + "*", "z")],
+                    "launch_bcast12<%s>(stream, n, x, sx, nx, y, sy, ny, z, Op2_%s<%s>())" % (T, name, T), "src/libknet8/cuda12.jl:18-34")
+            p13 = [(T + "*", "x"), (T + "*", "y"), (T + "*", "z"), ("int", "dimstride"), ("int", "nextstride"), ("int", "multidimsize"),
+                   ("int", "A_N"), ("int", "B_N")]
+            o.entry("%s_%s_13_x_y" % (name, S), "void", p13,
+                    "(void)nextstride; (void)multidimsize; launch_bcast12<%s>(stream, A_N, x, 1, A_N, y, dimstride, B_N, z, Op2_%s<%s>())" % (T, name, T),
+                    "src/libknet8/cuda13.jl:44-106")
+            o.entry("%s_%s_13_y_x" % (name, S), "void", p13,
+                    "(void)nextstride; (void)multidimsize; launch_bcast12<%s>(stream, A_N, x, 1, A_N, y, dimstride, B_N, z, Op2r_%s<%s>())" % (T, name, T),
+                    "src/libknet8/cuda13.jl:108-184")
+    o.decl.append("\n/* ---- activation gradients dx[i] = f(dy[i], y[i]) -- src/libknet8/cuda11.jl:12-28 with the *back rows of ops.jl:114-121 ---- */")
+    for name, body, cite in BACK11_OPS:
+        s.append(functor("Op11_" + name, ["xi", "yi"], body))
+        for T, S in TYPES:
+            o.entry("%s_%s_11" % (name, S), "void", [("int", "n"), (T + "*", "dy"), (T + "*", "y"), (T + "*", "dx")],
+                    "launch_ew<%s, 2>(stream, n, dy, y, (const %s*)nullptr, dx, Op11_%s<%s>())" % (T, T, name, T), cite)
+    o.decl.append("\n/* ---- ops21 gradients dx[i] = f(x[i], y[i], dy[i]) -- src/libknet8/cuda111.jl:12-29 ---- */")
+    for name, body, cite in BACK111_OPS:
+        s.append(functor("Op111_" + name, ["x", "y", "dy"], "(void)x; (void)y; " + body))
+        for T, S in TYPES:
+            o.entry("%s_%s_111" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
+                    "launch_ew<%s, 3>(stream, n, x, y, dy, dx, Op111_%s<%s>())" % (T, name, T), cite)
+    o.decl.append("\n/* ---- relu with max_value / negative_slope / threshold -- src/libknet8/relu.jl:8-38, src/ops21/activation.jl:101-112 ---- */")
+    s.append("template <typename T> struct OpReluKw { T maxv, slope, thr; __device__ __forceinline__ T operator()(T x) const {\n"
+             "  if (x >= maxv) return maxv; if (x >= thr) return x; if (slope == T(0)) return T(0); const T a = x - thr; return slope * a; } };\n")
+    s.append("template <typename T> struct OpRelubackKw { T maxv, slope, thr; __device__ __forceinline__ T operator()(T x, T dy) const {\n"
+             "  const T g = x >= maxv ? T(0) : x >= thr ? T(1) : slope; return dy * g; } };\n")
+    for T, S in TYPES:
+        o.entry("relu_%s_1" % S, "void", [("int", "n"), (T, "max_value"), (T, "negative_slope"), (T, "threshold"), (T + "*", "x"), (T + "*", "y")],
+                "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, y, OpReluKw<%s>{max_value, negative_slope, threshold})" % (T, T, T, T),
+                "src/libknet8/relu.jl:8-15,26-31")
+        o.entry("reluback_%s_1" % S, "void",
+                [("int", "n"), (T, "max_value"), (T, "negative_slope"), (T, "threshold"), (T + "*", "x"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
+                "(void)y; launch_ew<%s, 2>(stream, n, x, dy, (const %s*)nullptr, dx, OpRelubackKw<%s>{max_value, negative_slope, threshold})" % (T, T, T),
+                "src/libknet8/relu.jl:17-24,32-37 (y is not read: 3 streams instead of 4)")
+    o.decl.append("\n/* ---- fill, dropout, axpy, scal ---- */")
+    s.append("template <typename T> struct OpFill { T v; __device__ __forceinline__ T operator()() const { return v; } };\n")
+    s.append("// dropout!: y holds U[0,1) on entry; y = y>p ? x/q : 0 with q = 1-p  (src/ops20/dropout.jl:45-58)\n"
+             "template <typename T> struct OpDropout { T p, q; __device__ __forceinline__ T operator()(T x, T u) const { return u > p ? x / q : T(0); } };\n")
+    s.append("// dropback!: dx = y==0 ? 0 : dy/q  (src/ops20/dropout.jl:60-71)\n"
+             "template <typename T> struct OpDropback { T q; __device__ __forceinline__ T operator()(T y, T dy) const { return y == T(0) ? T(0) : dy / q; } };\n")
+    s.append("template <typename T> struct OpAxpy { T a; __device__ __forceinline__ T operator()(T x, T y) const { const T p = a * x; return y + p; } };\n")
+    s.append("template <typename T> struct OpScal { T a; __device__ __forceinline__ T operator()(T x) const { return a * x; } };\n")
+    for T, S in TYPES:
+        o.entry("fill_%s" % S, "void", [("int", "n"), (T, "x"), (T + "*", "y")],
+                "launch_ew<%s, 0>(stream, n, (const %s*)nullptr, (const %s*)nullptr, (const %s*)nullptr, y, OpFill<%s>{x})" % (T, T, T, T, T),
+                "src/libknet8/cuda1.jl:82-105")
+        o.entry("dropout_%s" % S, "void", [("int", "n"), (T, "p"), (T + "*", "x"), (T + "*", "y")],
+                "launch_ew<%s, 2>(stream, n, x, y, (const %s*)nullptr, y, OpDropout<%s>{p, %s(1) - p})" % (T, T, T, T),
+                "src/libknet8/cuda1.jl:459-484 (in place: y is the uniform buffer on entry)")
+        o.entry("dropback_%s" % S, "void", [("int", "n"), (T, "p"), (T + "*", "x"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
+                "(void)x; launch_ew<%s, 2>(stream, n, y, dy, (const %s*)nullptr, dx, OpDropback<%s>{%s(1) - p})" % (T, T, T, T),
+                "src/libknet8/cuda1.jl:469-493")
+        o.entry("axpy_%s" % S, "void", [("int", "n"), (T, "alpha"), (T + "*", "x"), (T + "*", "y")],
+                "launch_ew<%s, 2>(stream, n, x, y, (const %s*)nullptr, y, OpAxpy<%s>{alpha})" % (T, T, T),
+                "cublas%saxpy_v2 with unit increments at src/knetarrays/linalg.jl:58-73 (addto!, src/autograd_gpu/addto.jl:7-10)" % ("S" if S == "32" else "D"))
+        o.entry("scal_%s" % S, "void", [("int", "n"), (T, "alpha"), (T + "*", "x")],
+                "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, x, OpScal<%s>{alpha})" % (T, T, T, T),
+                "cublas%sscal_v2 with unit increment at src/knetarrays/linalg.jl:75-90" % ("S" if S == "32" else "D"))
+    return o
+
+
+def gen_reduce():
+    o = Out()
+    o.src.append(PRELUDE)
+    o.decl.append("\n/* ---- reductions.  _20: whole array -> scalar returned by value (blocks until done);\n"
+                  "   _21: x[i] goes into y[(i/sy)%ny]; _22: N-d array, one reduced dim of size xd1+1 and stride s1,\n"
+                  "   next stride s2 -- src/libknet8/cuda20.jl:27-104, cuda21.jl:22-77, cuda22.jl:22-66;\n"
+                  "   dispatch src/knetarrays/reduction.jl:21-77 ---- */")
+    for name, cls in REDUCTION_OPS:
+        for T, S in TYPES:
+            op = "%s<%s>" % (cls, T)
+            body20 = ("  %s r = %s::init();\n"
+                      "  if (n <= 0) return r;\n"
+                      "  %s* out = static_cast<%s*>(knet8::scalar_slot(stream));\n"
+                      "  launch_reduce_run<%s, %s>(stream, x, (long)n, 1, 1, out);\n"
+                      "  knet8::check_launch(\"%s_%s_20\");\n"
+                      "  knet8::fetch_scalar(stream, out, &r, sizeof(r));\n"
+                      "  return r;") % (T, op, T, T, T, op, name, S)
+            o.entry("%s_%s_20" % (name, S), T, [("int", "n"), (T + "*", "x")], None, "src/libknet8/cuda20.jl:84-104", body=body20)
+            o.entry("%s_%s_21" % (name, S), "void", [("int", "nx"), (T + "*", "x"), ("int", "sy"), ("int", "ny"), (T + "*", "y")],
+                    "knet8::reduce_21<%s, %s>(stream, nx, x, sy, ny, y)" % (T, op), "src/libknet8/cuda21.jl:68-76")
+            o.entry("%s_%s_22" % (name, S), "void",
+                    [("int", "nx"), ("int", "xd1"), (T + "*", "x"), ("int", "s1"), ("int", "s2"), ("int", "ny"), (T + "*", "y")],
+                    "knet8::reduce_22<%s, %s>(stream, nx, xd1, x, s1, s2, ny, y)" % (T, op), "src/libknet8/cuda22.jl:58-65")
+    return o
+
+
+def gen_softmax():
+    o = Out()
+    o.src.append(PRELUDE)
+    o.decl.append("\n/* ---- softmax family down each contiguous column of an m x n column-major matrix.  No libknet8 counterpart:\n"
+                  "   these replace the cudnnSoftmaxForward/Backward calls (MODE_INSTANCE on a (1,1,m,n) view, ACCURATE and LOG\n"
+                  "   algorithms) at src/ops20_gpu/softmax.jl:44-56; arithmetic of src/ops20/softmax.jl:42-63 ---- */")
+    for T, S in TYPES:
+        z = "(const %s*)nullptr" % T
+        o.entry("softmax_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "x"), (T + "*", "y")],
+                "launch_softmax<%s, AlgoSoftmax<%s>>(stream, m, n, x, %s, y, nullptr, %s(0), nullptr)" % (T, T, z, T),
+                "unsafe_cudnnSoftmaxForward(ACCURATE) at src/ops20_gpu/softmax.jl:44-49")
+        o.entry("logsoftmax_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "x"), (T + "*", "y")],
+                "launch_softmax<%s, AlgoLogSoftmax<%s>>(stream, m, n, x, %s, y, nullptr, %s(0), nullptr)" % (T, T, z, T),
+                "unsafe_cudnnSoftmaxForward(LOG) at src/ops20_gpu/softmax.jl:44-49")
+        o.entry("softmaxback_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
+                "launch_softmax<%s, AlgoSoftmaxBack<%s>>(stream, m, n, y, dy, dx, nullptr, %s(0), nullptr)" % (T, T, T),
+                "unsafe_cudnnSoftmaxBackward(ACCURATE) at src/ops20_gpu/softmax.jl:51-56")
+        o.entry("logsoftmaxback_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
+                "launch_softmax<%s, AlgoLogSoftmaxBack<%s>>(stream, m, n, y, dy, dx, nullptr, %s(0), nullptr)" % (T, T, T),
+                "unsafe_cudnnSoftmaxBackward(LOG) at src/ops20_gpu/softmax.jl:51-56")
+        o.decl.append("/* Fused gradient of nll(scores, labels; dims=1) wrt scores: dx = scale*(softmax(x) - onehot(label)) per column and\n"
+                      "   loss[col] = -logsoftmax(x)[label, col]; labels are 1-based int32, label 0 skips the column (dx = 0, loss = 0).\n"
+                      "   One pass over the scores instead of logsoftmax + getents + fill + addents + logsoftmaxback. */")
+        o.entry("nll_logsoftmax_back_%s" % S, "void",
+                [("int", "m"), ("int", "n"), (T + "*", "scores"), ("int*", "labels"), (T, "scale"), (T + "*", "dx"), (T + "*", "loss")],
+                "launch_softmax<%s, AlgoNll<%s>>(stream, m, n, scores, %s, dx, labels, scale, loss)" % (T, T, z),
+                "the chain nll -> getindex -> logsoftmax of src/ops20/loss.jl:37-41 (getents/addents + cuDNN LOG backward)")
+    o.decl.append("\n/* ---- 2-d transpose y(n,m) = x(m,n)' -- CUDA.jl permutedims / cublasSgeam at src/knetarrays/reshape.jl:18, linalg.jl:92-113 ---- */")
+    for T, S in TYPES:
+        o.entry("transpose_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "x"), (T + "*", "y")],
+                "launch_transpose<%s>(stream, m, n, x, y)" % T, "permutedims(x) for matrices, src/ops20_gpu/softmax.jl:19-20")
+    o.decl.append("\n/* ---- gather / scatter on 1-based int32 linear indices -- src/libknet8/cuda1.jl:342-362 ---- */")
+    for T, S in TYPES:
+        o.entry("getents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],
+                "launch_getents<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:342-348")
+        o.entry("setents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],
+                "launch_setents<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:349-355")
+        o.entry("addents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],
+                "launch_addents<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:356-362")
+    return o
+
+
+HEADER_TOP = """/* knet8.h -- C ABI of libknet8.so for AMD Instinct MI355X (gfx950).
+ *
+ * GENERATED by knet.jl_amd/csrc/gen_knet8.py together with the sources of the library.
+ *
+ * Every kernel entry point exists twice, as in the reference (src/libknet8/LibKnet8.jl:50-62):
+ *   NAME_stream(args..., hipStream_t)  -- asynchronous launch on the given stream (what @knet8 binds)
+ *   NAME(args...)                      -- same on the null stream
+ * S in a name is the element width (32: float, 64: double).  Sizes and strides are 32-bit ints, scalars
+ * are passed by value in T, arrays are device pointers owned and pre-allocated by the caller, index
+ * arrays hold 1-based int32.  Calls return nothing (only the _20 reductions return a value, and block);
+ * n <= 0 is a no-op.  Failures are recorded and can be read with knet8_last_error().
+ */
+#ifndef KNET8_H
+#define KNET8_H
+#include <stddef.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+#ifndef KNET8_API
+#define KNET8_API __attribute__((visibility("default")))
+#endif
+typedef struct ihipStream_t* hipStream_t;
+"""
+
+HEADER_RUNTIME = """
+/* ---- runtime: device memory for KnetArray storage, copies, streams, GEMM ---- */
+/* replaces knetMalloc / the free-list pool of src/knetarrays/kptr.jl:105-142,186-194: size-class pool over hipMalloc */
+KNET8_API void* knet8_malloc(size_t nbytes);
+KNET8_API void knet8_free(void* ptr);
+/* replaces Knet.gc, src/knetarrays/kptr.jl:204-226: hipFree every cached block; returns the bytes released */
+KNET8_API size_t knet8_trim(void);
+/* replaces meminfo/kmeminfo, src/knetarrays/kptr.jl:254-255: out[0]=bytes in use, out[1]=bytes cached, out[2]=hipMalloc calls, out[3]=pool hits */
+KNET8_API void knet8_meminfo(size_t* out4);
+/* replaces the copyto!/unsafe_copyto! paths of src/knetarrays/copy.jl:6-11: kind 1 = host->device, 2 = device->host, 3 = device->device;
+   host copies return when the data has landed */
+KNET8_API int knet8_memcpy(void* dst, const void* src, size_t nbytes, int kind, hipStream_t stream);
+KNET8_API int knet8_device_count(void);
+KNET8_API int knet8_set_device(int dev);
+KNET8_API hipStream_t knet8_stream_create(void);
+KNET8_API void knet8_stream_destroy(hipStream_t stream);
+KNET8_API int knet8_synchronize(hipStream_t stream);
+/* elapsed device time between two marks on a stream, in milliseconds (HIP events) */
+KNET8_API void knet8_timer_start(hipStream_t stream);
+KNET8_API float knet8_timer_stop(hipStream_t stream);
+/* last recorded failure as text (NULL if none); reading clears it */
+KNET8_API const char* knet8_last_error(void);
+KNET8_API int knet8_version(void);
+/* launch-heuristic knobs (0: bytes per reduction workgroup, 1/2: min/max workgroups per reduction launch) */
+KNET8_API int knet8_tune(int key, int value);
+/* replaces cublasSgemm_v2 / cublasDgemm_v2 at src/knetarrays/linalg.jl:26-52 (column-major, transa/transb in 'N','T'): hipBLASLt */
+KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc, hipStream_t stream);
+KNET8_API int gemm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc);
+KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc, hipStream_t stream);
+KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc);
+"""
+
+HEADER_BOTTOM = """
+#ifdef __cplusplus
+}
+#endif
+#endif /* KNET8_H */
+"""
+
+
+def generate(write=True):
+    units = {"knet8_elementwise_gen.hip": gen_elementwise(), "knet8_reduce_gen.hip": gen_reduce(), "knet8_softmax_gen.hip": gen_softmax()}
+    files = {}
+    for fn, o in units.items():
+        files[os.path.join(GEN, fn)] = "\n".join(o.src) + "\n"
+    header = HEADER_TOP + "\n".join("\n".join(o.decl) for o in units.values()) + "\n" + HEADER_RUNTIME + HEADER_BOTTOM
+    files[HEADER] = header
+    if write:
+        os.makedirs(GEN, exist_ok=True)
+        os.makedirs(os.path.dirname(HEADER), exist_ok=True)
+        for path, text in files.items():
+            old = open(path).read() if os.path.exists(path) else None
+            if old != text:
+                with open(path, "w") as f:
+                    f.write(text)
+    return files
+
+
+if __name__ == "__main__":
+    for p in generate():
+        print("wrote", os.path.relpath(p, ROOT))

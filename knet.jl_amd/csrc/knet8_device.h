@@ -1,0 +1,101 @@
+// Device-side building blocks shared by every libknet8 kernel family (gfx950 / CDNA4 only).
+//
+// Conventions
+//   * wavefront = 64 lanes; workgroups are multiples of 64 threads.
+//   * streaming operands are moved as 16-byte vectors (global_load_dwordx4 /
+//     global_store_dwordx4) with the non-temporal hint: every array on the gradient path is
+//     touched exactly once per launch, so nothing is worth keeping in L2.
+//   * all arithmetic is compiled with -ffp-contract=off: one rounding per operation, the same
+//     sequence of operations as the CPU Array path of the reference.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace knet8 {
+
+constexpr int kWave = 64;
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+  typedef float type __attribute__((ext_vector_type(4)));
+  static constexpr int N = 4;
+};
+template <> struct Vec16<double> {
+  typedef double type __attribute__((ext_vector_type(2)));
+  static constexpr int N = 2;
+};
+template <> struct Vec16<int> {
+  typedef int type __attribute__((ext_vector_type(4)));
+  static constexpr int N = 4;
+};
+
+// Streaming (read-once / write-once) accesses.
+template <typename V> __device__ __forceinline__ V ld_stream(const V* p) { return __builtin_nontemporal_load(p); }
+template <typename V> __device__ __forceinline__ void st_stream(V* p, V v) { __builtin_nontemporal_store(v, p); }
+
+template <typename T> __host__ __device__ __forceinline__ bool aligned16(const T* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+// ---- wave64 reductions -------------------------------------------------------------------------
+// Butterfly over the 64 lanes with ds_bpermute-free cross-lane moves (__shfl_xor lowers to DPP /
+// ds_swizzle / permlane on gfx950).  Every lane ends with the full result, in a fixed order, so
+// results are deterministic run to run.
+template <typename T, typename Merge> __device__ __forceinline__ T wave_reduce(T v, Merge merge) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v = merge(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Reduce over a workgroup of NWAVES*64 threads.  `lds` must hold NWAVES elements.  Every thread
+// returns the full result.  Contains two barriers: may be called repeatedly with the same `lds`.
+template <typename T, int NWAVES, typename Merge>
+__device__ __forceinline__ T block_reduce(T v, T* lds, Merge merge, T identity) {
+  v = wave_reduce(v, merge);
+  if (NWAVES == 1) return v;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  __syncthreads();  // previous use of lds is over
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  T r = (lane < NWAVES) ? lds[lane] : identity;
+  // NWAVES <= 16: a 16-lane butterfly is enough, but the full one keeps every lane identical
+  r = wave_reduce(r, merge);
+  return r;
+}
+
+// Device-scope "last workgroup of a group finishes the job" ticket.  Workgroups that contribute to the
+// same output group publish their partials, fence, and take a ticket; the one that draws the last
+// ticket (returns true) may read all partials (after the fence inside) and must reset the counter so
+// the next launch on the same stream finds it zero.
+__device__ __forceinline__ bool last_block_ticket(unsigned* counter, unsigned nparts, unsigned* lds_flag) {
+  __threadfence();  // publish this workgroup's partials at agent scope
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    *lds_flag = (t == nparts - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  bool last = (*lds_flag != 0);
+  if (last) __threadfence();  // acquire: see every other workgroup's partials
+  return last;
+}
+
+template <typename T> __device__ __forceinline__ T ld_coherent(const T* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace knet8
+
+// ---- libm calls used by the operator tables (ocml, full precision: the library is built without fast-math)
+namespace knet8 {
+__device__ __forceinline__ float kexp(float x) { return expf(x); }
+__device__ __forceinline__ double kexp(double x) { return exp(x); }
+__device__ __forceinline__ float klog(float x) { return logf(x); }
+__device__ __forceinline__ double klog(double x) { return log(x); }
+__device__ __forceinline__ float ktanh(float x) { return tanhf(x); }
+__device__ __forceinline__ double ktanh(double x) { return tanh(x); }
+__device__ __forceinline__ float kerf(float x) { return erff(x); }
+__device__ __forceinline__ double kerf(double x) { return erf(x); }
+__device__ __forceinline__ float ksqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double ksqrt(double x) { return sqrt(x); }
+}  // namespace knet8

@@ -1,0 +1,132 @@
+// Elementwise kernel family: out[i] = f(a[i] [, b[i] [, c[i]]]) over a flat length-n array.
+//
+// Replaces the reference's fixed <<<256,256>>> scalar grid-stride loops (src/libknet8/cuda1.jl:13-38,
+// cuda01.jl:11-25, cuda11.jl:12-28, cuda111.jl:12-29, relu.jl:8-38) with a one-shot grid of
+// 256-thread workgroups in which every lane moves one 16-byte vector per operand with the
+// non-temporal hint.  Measured on MI355X this shape (many small workgroups, one dwordx4 per lane per
+// stream, no loop) sustains the highest 2R+1W bandwidth; persistent grid-stride variants were slower.
+//
+// HBM roofline: (NIN+1)*sizeof(T) algorithmic bytes per element.
+#pragma once
+#include "knet8_device.h"
+
+namespace knet8 {
+
+constexpr int kEwBlock = 256;
+
+template <typename T, int NIN, typename F> struct EwApply;
+template <typename T, typename F> struct EwApply<T, 0, F> {
+  __device__ static __forceinline__ T go(const F& f, T, T, T) { return f(); }
+};
+template <typename T, typename F> struct EwApply<T, 1, F> {
+  __device__ static __forceinline__ T go(const F& f, T a, T, T) { return f(a); }
+};
+template <typename T, typename F> struct EwApply<T, 2, F> {
+  __device__ static __forceinline__ T go(const F& f, T a, T b, T) { return f(a, b); }
+};
+template <typename T, typename F> struct EwApply<T, 3, F> {
+  __device__ static __forceinline__ T go(const F& f, T a, T b, T c) { return f(a, b, c); }
+};
+
+// Vector path.  Operands are congruent modulo 16 bytes: after `head` scalar elements every pointer
+// is 16-byte aligned.  Elements [head, head + nvec*N) go through vectors; the `head` leading and the
+// trailing (n - tail0) elements are handled as scalars by the first lanes of workgroup 0.
+template <typename T, int NIN, typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_vec_kernel(long nvec, int head, long tail0, long n, const T* a, const T* b,
+                                                          const T* c, T* out, F f) {
+  typedef typename Vec16<T>::type V;
+  constexpr int N = Vec16<T>::N;
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i < nvec) {
+    const long e = head + i * N;
+    V va, vb, vc, r;
+    if (NIN >= 1) va = ld_stream(reinterpret_cast<const V*>(a + e));
+    if (NIN >= 2) vb = ld_stream(reinterpret_cast<const V*>(b + e));
+    if (NIN >= 3) vc = ld_stream(reinterpret_cast<const V*>(c + e));
+#pragma unroll
+    for (int k = 0; k < N; k++)
+      r[k] = EwApply<T, NIN, F>::go(f, NIN >= 1 ? va[k] : T(0), NIN >= 2 ? vb[k] : T(0), NIN >= 3 ? vc[k] : T(0));
+    st_stream(reinterpret_cast<V*>(out + e), r);
+  }
+  if (blockIdx.x == 0) {
+    long e = -1;
+    if ((int)threadIdx.x < head) e = threadIdx.x;
+    else if (threadIdx.x >= kWave && tail0 + (threadIdx.x - kWave) < n) e = tail0 + (threadIdx.x - kWave);
+    if (e >= 0)
+      out[e] = EwApply<T, NIN, F>::go(f, NIN >= 1 ? a[e] : T(0), NIN >= 2 ? b[e] : T(0), NIN >= 3 ? c[e] : T(0));
+  }
+}
+
+// Scalar path for operands whose addresses differ modulo 16 bytes (sub-array views that start at
+// arbitrary element offsets).  Lanes still read consecutive elements, four per thread.
+template <typename T, int NIN, typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_scalar_kernel(long n, const T* a, const T* b, const T* c, T* out, F f) {
+  const long base = (long)blockIdx.x * (kEwBlock * 4) + threadIdx.x;
+  T ra[4], rb[4], rc[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const long e = base + u * kEwBlock;
+    if (e < n) {
+      if (NIN >= 1) ra[u] = a[e];
+      if (NIN >= 2) rb[u] = b[e];
+      if (NIN >= 3) rc[u] = c[e];
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const long e = base + u * kEwBlock;
+    if (e < n)
+      out[e] = EwApply<T, NIN, F>::go(f, NIN >= 1 ? ra[u] : T(0), NIN >= 2 ? rb[u] : T(0), NIN >= 3 ? rc[u] : T(0));
+  }
+}
+
+template <typename T, int NIN, typename F>
+inline void launch_ew(hipStream_t stream, long n, const T* a, const T* b, const T* c, T* out, F f) {
+  if (n <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  const uintptr_t mo = reinterpret_cast<uintptr_t>(out) & 15u;
+  bool congruent = (mo % sizeof(T)) == 0;
+  if (NIN >= 1) congruent = congruent && ((reinterpret_cast<uintptr_t>(a) & 15u) == mo);
+  if (NIN >= 2) congruent = congruent && ((reinterpret_cast<uintptr_t>(b) & 15u) == mo);
+  if (NIN >= 3) congruent = congruent && ((reinterpret_cast<uintptr_t>(c) & 15u) == mo);
+  if (congruent) {
+    long head = mo ? (long)((16u - mo) / sizeof(T)) : 0;
+    if (head > n) head = n;
+    const long nvec = (n - head) / N;
+    const long tail0 = head + nvec * N;
+    long grid = (nvec + kEwBlock - 1) / kEwBlock;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL((ew_vec_kernel<T, NIN, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, (int)head, tail0, n,
+                       a, b, c, out, f);
+  } else {
+    const long grid = (n + kEwBlock * 4 - 1) / (kEwBlock * 4);
+    hipLaunchKernelGGL((ew_scalar_kernel<T, NIN, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, a, b, c, out, f);
+  }
+}
+
+// z = f(x[.], y[.]) where each operand is either full size or a vector along one dimension of the
+// result: element i of the result reads x[(i/sx)%nx] (src/libknet8/cuda12.jl:18-27).  Used for the
+// forward bias add; HBM roofline 2*sizeof(T) per element (the vector operand stays in cache).
+template <typename T, typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_bcast12_kernel(long n, const T* x, int sx, int nx, const T* y, int sy, int ny,
+                                                              T* z, F f) {
+  const long base = (long)blockIdx.x * (kEwBlock * 4) + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const long i = base + u * kEwBlock;
+    if (i < n) {
+      const T xi = (nx == n ? x[i] : sx == 1 ? x[i % nx] : nx == 1 ? x[0] : x[(i / sx) % nx]);
+      const T yi = (ny == n ? y[i] : sy == 1 ? y[i % ny] : ny == 1 ? y[0] : y[(i / sy) % ny]);
+      z[i] = f(xi, yi);
+    }
+  }
+}
+
+template <typename T, typename F>
+inline void launch_bcast12(hipStream_t stream, long n, const T* x, int sx, int nx, const T* y, int sy, int ny, T* z, F f) {
+  if (n <= 0) return;
+  const long grid = (n + kEwBlock * 4 - 1) / (kEwBlock * 4);
+  hipLaunchKernelGGL((ew_bcast12_kernel<T, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, x, sx, nx, y, sy, ny, z, f);
+}
+
+}  // namespace knet8

@@ -1,0 +1,347 @@
+// Reduction kernel family behind the `_20` (array -> scalar), `_21` (array -> vector) and `_22`
+// (array -> array, one reduced dimension) entry points.
+//
+// The reference runs one 128-thread block per output element on a fixed <<<128,128>>> grid
+// (src/libknet8/cuda20.jl:27-104, cuda21.jl:22-77, cuda22.jl:22-66); its `sy==1` branch reads with lanes
+// `ny` elements apart.  Here every shape is mapped onto one of two views of the column-major input and
+// each view has a kernel whose lanes always walk the contiguous axis:
+//
+//   run view      x(sy, ny, no)  ->  y(ny)      reduce axes 1 and 3   (`_21` with sy>1, `_20`, `_22` with s1==1)
+//   strided view  x(s1, d, nb)   ->  y(s1, nb)  reduce axis 2         (`_21` with sy==1, `_22` with s1>1)
+//
+// Both split the reduced axis over P workgroups per output group when one group alone would leave the
+// machine idle or take too long; the P partials are combined, in fixed order, by whichever workgroup
+// draws the last ticket of its group, so one launch suffices and the result is deterministic (no float atomics).
+//
+// HBM roofline: sizeof(T)*(nx + ny) algorithmic bytes.
+#pragma once
+#include "knet8_device.h"
+#include "knet8_runtime.h"
+
+namespace knet8 {
+
+constexpr int kRedBlock = 256;
+constexpr int kRedWaves = kRedBlock / kWave;
+
+// ---- operator table: (merge, item, init) triples of src/libknet8/ops.jl:144-156 ---------------------
+template <typename T> struct RedSum     { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedProd    { __host__ __device__ static T init() { return T(1); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a * x; } };
+template <typename T> struct RedMaximum { __host__ __device__ static T init() { return -INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
+template <typename T> struct RedMinimum { __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
+template <typename T> struct RedSumabs  { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedSumabs2 { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x * x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedMaxabs  { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
+template <typename T> struct RedMinabs  { __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
+template <typename T> struct RedCountnz { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x != 0 ? T(1) : T(0); } __device__ static T merge(T a, T x) { return a + x; } };
+
+template <typename Op, typename T> struct MergeFn {
+  __device__ __forceinline__ T operator()(T a, T b) const { return Op::merge(a, b); }
+};
+
+// ---- run view ------------------------------------------------------------------------------------
+// Output j reduces K = no*sy elements: flattened index k -> x[(k/sy)*sy*ny + j*sy + k%sy].
+// NV = elements per lane per load (Vec16<T>::N on the aligned path, 1 otherwise); on the vector path
+// sy % NV == 0 so a vector never straddles two runs.  Workgroup (j,p) covers units [p*chunk, (p+1)*chunk)
+// of the K/NV units of output j.
+template <typename T, typename Op, int NV, bool SINGLE>
+__global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restrict__ x, long sy, long ny, long units, long chunk,
+                                                               unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
+  __shared__ T lds[kRedWaves];
+  __shared__ unsigned flag;
+  const long j = blockIdx.x / P;
+  const unsigned p = blockIdx.x % P;
+  const long u0 = (long)p * chunk;
+  long u1 = u0 + chunk;
+  if (u1 > units) u1 = units;
+  const long usy = sy / NV;              // units per run
+  const long slab = sy * ny;             // elements between the same run of consecutive slabs
+  const T* xj = x + j * sy;
+  T acc[NV];
+#pragma unroll
+  for (int e = 0; e < NV; e++) acc[e] = Op::init();
+  constexpr int U = 4;
+  for (long u = u0 + threadIdx.x; u < u1; u += kRedBlock * U) {
+    T v[U][NV];
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long uu = u + q * kRedBlock;
+      if (uu < u1) {
+        long off;
+        if (SINGLE) off = uu * NV;
+        else { const long o = uu / usy; off = o * slab + (uu - o * usy) * NV; }
+        if (NV > 1) {
+          typedef typename Vec16<T>::type V;
+          V t = ld_stream(reinterpret_cast<const V*>(xj + off));
+#pragma unroll
+          for (int e = 0; e < NV; e++) v[q][e] = Op::item(t[e]);
+        } else {
+          v[q][0] = Op::item(__builtin_nontemporal_load(xj + off));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; e++) v[q][e] = Op::init();
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < U; q++)
+#pragma unroll
+      for (int e = 0; e < NV; e++) acc[e] = Op::merge(acc[e], v[q][e]);
+  }
+  T r = acc[0];
+#pragma unroll
+  for (int e = 1; e < NV; e++) r = Op::merge(r, acc[e]);
+  r = block_reduce<T, kRedWaves>(r, lds, MergeFn<Op, T>(), Op::init());
+  if (P == 1) {
+    if (threadIdx.x == 0) y[j] = r;
+    return;
+  }
+  if (threadIdx.x == 0) partial[j * P + p] = r;
+  if (!last_block_ticket(counters + j, P, &flag)) return;
+  T s = Op::init();
+  for (unsigned q = threadIdx.x; q < P; q += kRedBlock) s = Op::merge(s, ld_coherent(partial + j * P + q));
+  s = block_reduce<T, kRedWaves>(s, lds, MergeFn<Op, T>(), Op::init());
+  if (threadIdx.x == 0) {
+    y[j] = s;
+    counters[j] = 0;
+  }
+}
+
+// ---- strided view --------------------------------------------------------------------------------
+// y[a + b*s1] = reduce_k x[a + k*s1 + b*s1*d].  A wave covers 64*NV consecutive a's with one load per
+// lane; the four waves of a workgroup take k = k0+wave, k0+wave+4, ...; P workgroups split the k range.
+// The same walk (rows `stride` apart, this wave's share of [k0,k1)) combines the P partial tiles at the end
+// (ITEM=false: partials are merged as they are, the item map was applied when they were made).
+template <typename T, typename Op, int NV, bool ITEM>
+__device__ __forceinline__ void strided_walk(const T* base, long stride, long k0, long k1, int wave, T (&acc)[NV]) {
+  constexpr int U = 8;
+  for (long k = k0 + wave; k < k1; k += kRedWaves * U) {
+    T v[U][NV];
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long kk = k + q * kRedWaves;
+      if (kk < k1) {
+        if (NV > 1) {
+          typedef typename Vec16<T>::type V;
+          V t = ld_stream(reinterpret_cast<const V*>(base + kk * stride));
+#pragma unroll
+          for (int e = 0; e < NV; e++) v[q][e] = ITEM ? Op::item(t[e]) : t[e];
+        } else {
+          const T t = __builtin_nontemporal_load(base + kk * stride);
+          v[q][0] = ITEM ? Op::item(t) : t;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; e++) v[q][e] = Op::init();
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < U; q++)
+#pragma unroll
+      for (int e = 0; e < NV; e++) acc[e] = Op::merge(acc[e], v[q][e]);
+  }
+}
+
+template <typename T, typename Op, int NV>
+__global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
+                                                                   unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
+  constexpr int TILE = kWave * NV;
+  __shared__ T lds[kRedWaves][TILE];
+  __shared__ unsigned flag;
+  const long group = blockIdx.x / P;   // (b, atile)
+  const unsigned p = blockIdx.x % P;
+  const long b = group / atiles, at = group % atiles;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const long a0 = at * TILE + (long)lane * NV;
+  const bool live = a0 < s1;           // on the vector path s1 % NV == 0, so a live lane is fully in range
+  const long k0 = (long)p * kchunk;
+  long k1 = k0 + kchunk;
+  if (k1 > d) k1 = d;
+  T acc[NV];
+#pragma unroll
+  for (int e = 0; e < NV; e++) acc[e] = Op::init();
+  if (live) strided_walk<T, Op, NV, true>(x + b * s1 * d + a0, s1, k0, k1, wave, acc);
+  if (P > 1) {
+    // partial tile p of this group = this workgroup's reduction over its k range
+#pragma unroll
+    for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+    __syncthreads();
+    if (threadIdx.x < TILE) {
+      T r = Op::init();
+#pragma unroll
+      for (int w = 0; w < kRedWaves; w++) r = Op::merge(r, lds[w][threadIdx.x]);
+      partial[(group * P + p) * TILE + threadIdx.x] = r;
+    }
+    if (!last_block_ticket(counters + group, P, &flag)) return;
+#pragma unroll
+    for (int e = 0; e < NV; e++) acc[e] = Op::init();
+    strided_walk<T, Op, NV, false>(partial + group * P * TILE + lane * NV, TILE, 0, P, wave, acc);
+    if (threadIdx.x == 0) counters[group] = 0;
+  }
+#pragma unroll
+  for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+  __syncthreads();
+  const long a = at * TILE + threadIdx.x;
+  if (threadIdx.x < TILE && a < s1) {
+    T r = Op::init();
+#pragma unroll
+    for (int w = 0; w < kRedWaves; w++) r = Op::merge(r, lds[w][threadIdx.x]);
+    y[b * s1 + a] = r;
+  }
+}
+
+// Strided view with a short contiguous axis (s1 < 64): lanes along `a` alone would idle most of a wave,
+// so the (s1 x d) slab of batch b is walked as one contiguous range, L = s1*floor(256/s1) lanes at a
+// time; lane t always meets a == t % s1.  Workgroup (b,p) covers elements [p*chunk, (p+1)*chunk) of the
+// slab (chunk is a multiple of L).
+template <typename T, typename Op>
+__global__ __launch_bounds__(kRedBlock) void reduce_strided_small_kernel(const T* __restrict__ x, int s1, long d, long chunk,
+                                                                         unsigned P, T* __restrict__ y, T* partial,
+                                                                         unsigned* counters) {
+  __shared__ T lds[kRedBlock];
+  __shared__ unsigned flag;
+  const long b = blockIdx.x / P;
+  const unsigned p = blockIdx.x % P;
+  const int reps = kRedBlock / s1, L = reps * s1;
+  const long total = (long)s1 * d;
+  const long i0 = (long)p * chunk;
+  long i1 = i0 + chunk;
+  if (i1 > total) i1 = total;
+  const T* xb = x + b * total;
+  T acc = Op::init();
+  if ((int)threadIdx.x < L) {
+    constexpr int U = 4;
+    for (long i = i0 + threadIdx.x; i < i1; i += (long)L * U) {
+      T v[U];
+#pragma unroll
+      for (int q = 0; q < U; q++) {
+        const long ii = i + (long)q * L;
+        v[q] = ii < i1 ? Op::item(__builtin_nontemporal_load(xb + ii)) : Op::init();
+      }
+#pragma unroll
+      for (int q = 0; q < U; q++) acc = Op::merge(acc, v[q]);
+    }
+  }
+  lds[threadIdx.x] = acc;
+  __syncthreads();
+  T r = Op::init();
+  const bool owner = (int)threadIdx.x < s1;
+  if (owner)
+    for (int q = 0; q < reps; q++) r = Op::merge(r, lds[threadIdx.x + q * s1]);
+  if (P == 1) {
+    if (owner) y[b * s1 + threadIdx.x] = r;
+    return;
+  }
+  if (owner) partial[(b * P + p) * s1 + threadIdx.x] = r;
+  if (!last_block_ticket(counters + b, P, &flag)) return;
+  if (owner) {
+    T s = Op::init();
+    for (unsigned q = 0; q < P; q++) s = Op::merge(s, ld_coherent(partial + (b * P + q) * s1 + threadIdx.x));
+    y[b * s1 + threadIdx.x] = s;
+  }
+  if (threadIdx.x == 0) counters[b] = 0;
+}
+
+// ---- host-side planning ----------------------------------------------------------------------------
+
+inline long ceil_div(long a, long b) { return (a + b - 1) / b; }
+
+// Number of workgroups per output group: about `wg_bytes` of input each, but at least enough to give the
+// launch `min_wgs` workgroups and at most enough to reach `max_wgs`; never so many that a workgroup has
+// less than `min_units_per_wg` loads to issue.
+inline unsigned plan_parts(long groups, long units_per_group, long unit_bytes, long min_units_per_wg) {
+  const long wg_bytes = tuning(kTuneRedWgBytes), min_wgs = tuning(kTuneRedMinWgs), max_wgs = tuning(kTuneRedMaxWgs);
+  long P = ceil_div(units_per_group * unit_bytes, wg_bytes);
+  const long fill = ceil_div(min_wgs, groups);
+  long most = max_wgs / groups;
+  if (most < fill) most = fill;
+  if (P > most) P = most;
+  if (P < fill) P = fill;
+  const long cap = units_per_group / min_units_per_wg;
+  if (P > cap) P = cap;
+  if (P > 65535) P = 65535;
+  if (P < 1) P = 1;
+  return (unsigned)P;
+}
+
+template <typename T, typename Op>
+inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y) {
+  if (ny <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  const bool vec = aligned16(x) && (sy % N == 0);
+  const int nv = vec ? N : 1;
+  const long units = sy / nv * no;
+  unsigned P = plan_parts(ny, units, (long)nv * sizeof(T), kRedBlock);
+  long chunk = ceil_div(units, P);
+  P = (unsigned)ceil_div(units, chunk > 0 ? chunk : 1);
+  if (P < 1) P = 1;
+  Workspace ws = {nullptr, nullptr};
+  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)ny * P, (size_t)ny);
+  const dim3 grid((unsigned)(ny * P)), block(kRedBlock);
+  T* partial = static_cast<T*>(ws.partial);
+#define KNET8_RUN(NV, SINGLE) \
+  hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE>), grid, block, 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters)
+  if (vec) { if (no == 1) KNET8_RUN(N, true); else KNET8_RUN(N, false); }
+  else     { if (no == 1) KNET8_RUN(1, true); else KNET8_RUN(1, false); }
+#undef KNET8_RUN
+}
+
+template <typename T, typename Op>
+inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y) {
+  if (s1 <= 0 || nb <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  if (s1 < kWave) {
+    const int reps = kRedBlock / (int)s1, L = reps * (int)s1;
+    const long total = s1 * d;
+    unsigned P = plan_parts(nb, ceil_div(total, L), (long)L * sizeof(T), 1);
+    long chunk = ceil_div(ceil_div(total, L), P) * L;
+    P = (unsigned)ceil_div(total, chunk > 0 ? chunk : 1);
+    if (P < 1) P = 1;
+    Workspace ws = {nullptr, nullptr};
+    if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)nb * P * s1, (size_t)nb);
+    hipLaunchKernelGGL((reduce_strided_small_kernel<T, Op>), dim3((unsigned)(nb * P)), dim3(kRedBlock), 0, stream, x, (int)s1, d,
+                       chunk, P, y, static_cast<T*>(ws.partial), ws.counters);
+    return;
+  }
+  const bool vec = aligned16(x) && (s1 % N == 0);
+  const int nv = vec ? N : 1;
+  const long tile = (long)kWave * nv;
+  const long atiles = ceil_div(s1, tile);
+  const long groups = atiles * nb;
+  unsigned P = plan_parts(groups, d, tile * sizeof(T), kRedWaves * 8);
+  long kchunk = ceil_div(d, P);
+  P = (unsigned)ceil_div(d, kchunk > 0 ? kchunk : 1);
+  if (P < 1) P = 1;
+  Workspace ws = {nullptr, nullptr};
+  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups);
+  const dim3 grid((unsigned)(groups * P)), block(kRedBlock);
+  T* partial = static_cast<T*>(ws.partial);
+  if (vec)
+    hipLaunchKernelGGL((reduce_strided_kernel<T, Op, N>), grid, block, 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters);
+  else
+    hipLaunchKernelGGL((reduce_strided_kernel<T, Op, 1>), grid, block, 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters);
+}
+
+// `_21` contract: x[i] goes into y[(i/sy)%ny]  (src/libknet8/cuda21.jl:23).
+template <typename T, typename Op>
+inline void reduce_21(hipStream_t stream, long nx, const T* x, long sy, long ny, T* y) {
+  if (ny <= 0 || sy <= 0 || nx < 0) return;
+  if (nx % (sy * ny) != 0) { record_error("reduce _21: nx is not a multiple of sy*ny"); return; }
+  const long no = nx / (sy * ny);
+  if (ny == 1) launch_reduce_run<T, Op>(stream, x, nx, 1, 1, y);
+  else if (sy == 1) launch_reduce_strided<T, Op>(stream, x, ny, no, 1, y);
+  else launch_reduce_run<T, Op>(stream, x, sy, ny, no, y);
+}
+
+// `_22` contract: output bi reduces x[lower + k*s1], k = 0..xd1, lower = bi%s1 + (bi/s1)*s2
+// (src/libknet8/cuda22.jl:31-36); the dispatcher always passes s2 = s1*(xd1+1).
+template <typename T, typename Op>
+inline void reduce_22(hipStream_t stream, long nx, long xd1, const T* x, long s1, long s2, long ny, T* y) {
+  (void)nx;
+  if (ny <= 0 || s1 <= 0 || xd1 < 0) return;
+  const long d = xd1 + 1;
+  if (s2 != s1 * d || ny % s1 != 0) { record_error("reduce _22: expected s2 == s1*(xd1+1) and ny a multiple of s1"); return; }
+  if (s1 == 1) launch_reduce_run<T, Op>(stream, x, d, ny, 1, y);
+  else launch_reduce_strided<T, Op>(stream, x, s1, d, ny / s1, y);
+}
+
+}  // namespace knet8

@@ -1,0 +1,34 @@
+// Host-side services shared by the generated entry points: error recording, per-stream reduction
+// scratch, launch-heuristic knobs.  Implemented in knet8_runtime.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+#ifndef KNET8_API
+#define KNET8_API __attribute__((visibility("default")))
+#endif
+
+namespace knet8 {
+
+// The entry points return void like the reference's (errors there are unchecked, src/libknet8/LibKnet8.jl:54);
+// failures are kept as text for knet8_last_error() instead of being dropped.
+void record_error(const char* what);
+void check_launch(const char* name);  // records hipGetLastError() if a launch failed
+
+// Scratch that split reductions need beyond their inputs and outputs: `partial` holds the per-workgroup
+// partial results, `counters` the per-output-group tickets (all zero between launches; the kernel that
+// uses them resets them).  One Workspace per stream, so launches on different streams never share it;
+// launches on one stream are ordered and may.
+struct Workspace {
+  void* partial;
+  unsigned* counters;
+};
+Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters);
+// Device slot for the result of a `_20` reduction on this stream, and the blocking copy that fetches it.
+void* scalar_slot(hipStream_t stream);
+void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes);
+
+enum { kTuneRedWgBytes = 0, kTuneRedMinWgs = 1, kTuneRedMaxWgs = 2, kTuneCount = 8 };
+int tuning(int key);
+
+}  // namespace knet8

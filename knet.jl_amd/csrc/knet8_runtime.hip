@@ -1,0 +1,379 @@
+// Host runtime of libknet8: error slot, per-stream reduction scratch, device-memory pool for KnetArray
+// storage, copies, stream/timer helpers and the hipBLASLt GEMM entry points.
+#include "knet8_runtime.h"
+
+#include <hipblaslt/hipblaslt.h>
+
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <tuple>
+#include <unordered_map>
+#include <vector>
+
+namespace knet8 {
+
+// ---- errors ------------------------------------------------------------------------------------------
+static std::mutex g_err_mutex;
+static std::string g_err;
+static thread_local std::string g_err_out;
+
+void record_error(const char* what) {
+  std::lock_guard<std::mutex> lock(g_err_mutex);
+  if (g_err.empty()) g_err = what;  // keep the first failure: later ones are usually consequences
+}
+
+void check_launch(const char* name) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    std::string msg = std::string(name) + ": " + hipGetErrorString(e);
+    record_error(msg.c_str());
+  }
+}
+
+static bool ok(hipError_t e, const char* what) {
+  if (e == hipSuccess) return true;
+  std::string msg = std::string(what) + ": " + hipGetErrorString(e);
+  record_error(msg.c_str());
+  return false;
+}
+
+// ---- launch-heuristic knobs ------------------------------------------------------------------------------
+static int g_tune[kTuneCount] = {
+    64 * 1024,  // kTuneRedWgBytes: input bytes one reduction workgroup should move
+    2048,       // kTuneRedMinWgs:  split until a reduction launch has at least this many workgroups
+    16384,      // kTuneRedMaxWgs:  ... and never split beyond this many
+    0, 0, 0, 0, 0};
+int tuning(int key) { return (key >= 0 && key < kTuneCount) ? g_tune[key] : 0; }
+
+// ---- per-stream scratch for split reductions ------------------------------------------------------------
+struct StreamScratch {
+  void* partial = nullptr;
+  size_t partial_bytes = 0;
+  unsigned* counters = nullptr;
+  size_t ncounters = 0;
+  void* scalar = nullptr;
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+};
+static std::mutex g_scratch_mutex;
+static std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
+
+static StreamScratch& scratch_of(hipStream_t stream) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  return g_scratch[std::make_pair(dev, stream)];
+}
+
+Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  StreamScratch& s = scratch_of(stream);
+  if (s.partial_bytes < partial_bytes) {
+    // Work already queued on this stream may still use the old buffer: hipFree waits for the device.
+    if (s.partial) (void)hipFree(s.partial);
+    size_t want = partial_bytes < (size_t(1) << 20) ? (size_t(1) << 20) : partial_bytes + partial_bytes / 2;
+    s.partial = nullptr;
+    s.partial_bytes = ok(hipMalloc(&s.partial, want), "hipMalloc(reduction partials)") ? want : 0;
+  }
+  if (s.ncounters < ncounters) {
+    if (s.counters) (void)hipFree(s.counters);
+    size_t want = ncounters < 4096 ? 4096 : ncounters + ncounters / 2;
+    s.counters = nullptr;
+    s.ncounters = 0;
+    if (ok(hipMalloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned)), "hipMalloc(reduction counters)") &&
+        ok(hipMemset(s.counters, 0, want * sizeof(unsigned)), "hipMemset(reduction counters)"))
+      s.ncounters = want;
+  }
+  Workspace w = {s.partial, s.counters};
+  return w;
+}
+
+void* scalar_slot(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  StreamScratch& s = scratch_of(stream);
+  if (!s.scalar) ok(hipMalloc(&s.scalar, 256), "hipMalloc(scalar slot)");
+  return s.scalar;
+}
+
+void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes) {
+  if (!dev) return;
+  if (ok(hipMemcpyAsync(host, dev, nbytes, hipMemcpyDeviceToHost, stream), "hipMemcpyAsync(scalar)"))
+    ok(hipStreamSynchronize(stream), "hipStreamSynchronize(scalar)");
+}
+
+// ---- device-memory pool ---------------------------------------------------------------------------------
+// Freed blocks are kept on per-size free lists and handed out again without touching the driver, as the
+// reference's KnetPtr pool does (src/knetarrays/kptr.jl:105-142; an uncached allocation costs ~0.5 ms there,
+// kptr.jl:187).  Sizes are rounded up to {1, 1.25, 1.5, 1.75} x 2^k (>= 256 bytes), so at most 25 % is lost
+// to rounding.  When hipMalloc fails the free lists are released and the allocation retried once.
+struct Pool {
+  std::mutex mutex;
+  std::unordered_map<size_t, std::vector<void*>> free_lists;  // rounded size -> blocks
+  std::unordered_map<void*, size_t> live;                     // block -> rounded size
+  size_t bytes_live = 0, bytes_cached = 0, nmalloc = 0, nhit = 0;
+};
+static Pool g_pool;
+
+static size_t round_size(size_t n) {
+  if (n <= 256) return 256;
+  size_t p = 256;
+  while (p * 2 < n) p *= 2;  // p < n <= 2p
+  const size_t q = p / 4;
+  for (int k = 1; k <= 4; k++)
+    if (p + k * q >= n) return p + k * q;
+  return 2 * p;
+}
+
+static size_t trim_locked(Pool& pool) {
+  size_t released = 0;
+  for (auto& kv : pool.free_lists) {
+    for (void* p : kv.second) {
+      (void)hipFree(p);
+      released += kv.first;
+    }
+    kv.second.clear();
+  }
+  pool.bytes_cached = 0;
+  return released;
+}
+
+}  // namespace knet8
+
+using namespace knet8;
+
+extern "C" {
+
+KNET8_API void* knet8_malloc(size_t nbytes) {
+  const size_t sz = round_size(nbytes);
+  std::lock_guard<std::mutex> lock(g_pool.mutex);
+  void* p = nullptr;
+  auto it = g_pool.free_lists.find(sz);
+  if (it != g_pool.free_lists.end() && !it->second.empty()) {
+    p = it->second.back();
+    it->second.pop_back();
+    g_pool.bytes_cached -= sz;
+    g_pool.nhit++;
+  } else {
+    hipError_t e = hipMalloc(&p, sz);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      trim_locked(g_pool);
+      e = hipMalloc(&p, sz);
+    }
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      record_error("knet8_malloc: out of device memory");
+      return nullptr;
+    }
+    g_pool.nmalloc++;
+  }
+  g_pool.live[p] = sz;
+  g_pool.bytes_live += sz;
+  return p;
+}
+
+KNET8_API void knet8_free(void* ptr) {
+  if (!ptr) return;
+  std::lock_guard<std::mutex> lock(g_pool.mutex);
+  auto it = g_pool.live.find(ptr);
+  if (it == g_pool.live.end()) {
+    record_error("knet8_free: pointer was not allocated by knet8_malloc");
+    return;
+  }
+  const size_t sz = it->second;
+  g_pool.live.erase(it);
+  g_pool.bytes_live -= sz;
+  g_pool.free_lists[sz].push_back(ptr);
+  g_pool.bytes_cached += sz;
+}
+
+KNET8_API size_t knet8_trim(void) {
+  (void)hipDeviceSynchronize();
+  std::lock_guard<std::mutex> lock(g_pool.mutex);
+  return trim_locked(g_pool);
+}
+
+KNET8_API void knet8_meminfo(size_t* out4) {
+  std::lock_guard<std::mutex> lock(g_pool.mutex);
+  out4[0] = g_pool.bytes_live;
+  out4[1] = g_pool.bytes_cached;
+  out4[2] = g_pool.nmalloc;
+  out4[3] = g_pool.nhit;
+}
+
+KNET8_API int knet8_memcpy(void* dst, const void* src, size_t nbytes, int kind, hipStream_t stream) {
+  if (nbytes == 0) return 0;
+  hipMemcpyKind k;
+  switch (kind) {
+    case 1: k = hipMemcpyHostToDevice; break;
+    case 2: k = hipMemcpyDeviceToHost; break;
+    case 3: k = hipMemcpyDeviceToDevice; break;
+    default: record_error("knet8_memcpy: kind must be 1 (h2d), 2 (d2h) or 3 (d2d)"); return -1;
+  }
+  if (!ok(hipMemcpyAsync(dst, src, nbytes, k, stream), "hipMemcpyAsync")) return -1;
+  if (kind != 3 && !ok(hipStreamSynchronize(stream), "hipStreamSynchronize")) return -1;
+  return 0;
+}
+
+KNET8_API int knet8_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+KNET8_API int knet8_set_device(int dev) { return ok(hipSetDevice(dev), "hipSetDevice") ? 0 : -1; }
+
+KNET8_API hipStream_t knet8_stream_create(void) {
+  hipStream_t s = nullptr;
+  ok(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
+  return s;
+}
+
+KNET8_API void knet8_stream_destroy(hipStream_t stream) {
+  if (stream) ok(hipStreamDestroy(stream), "hipStreamDestroy");
+}
+
+KNET8_API int knet8_synchronize(hipStream_t stream) { return ok(hipStreamSynchronize(stream), "hipStreamSynchronize") ? 0 : -1; }
+
+KNET8_API void knet8_timer_start(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  StreamScratch& s = scratch_of(stream);
+  if (!s.t0) {
+    ok(hipEventCreate(&s.t0), "hipEventCreate");
+    ok(hipEventCreate(&s.t1), "hipEventCreate");
+  }
+  ok(hipEventRecord(s.t0, stream), "hipEventRecord");
+}
+
+KNET8_API float knet8_timer_stop(hipStream_t stream) {
+  hipEvent_t t0, t1;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    StreamScratch& s = scratch_of(stream);
+    t0 = s.t0;
+    t1 = s.t1;
+  }
+  if (!t0) return -1.f;
+  float ms = -1.f;
+  if (ok(hipEventRecord(t1, stream), "hipEventRecord") && ok(hipEventSynchronize(t1), "hipEventSynchronize"))
+    ok(hipEventElapsedTime(&ms, t0, t1), "hipEventElapsedTime");
+  return ms;
+}
+
+KNET8_API const char* knet8_last_error(void) {
+  std::lock_guard<std::mutex> lock(g_err_mutex);
+  if (g_err.empty()) return nullptr;
+  g_err_out = g_err;
+  g_err.clear();
+  return g_err_out.c_str();
+}
+
+KNET8_API int knet8_version(void) { return 100; }
+
+KNET8_API int knet8_tune(int key, int value) {
+  if (key < 0 || key >= kTuneCount) return -1;
+  const int old = g_tune[key];
+  if (value > 0) g_tune[key] = value;
+  return old;
+}
+
+}  // extern "C"
+
+// ---- GEMM through hipBLASLt ----------------------------------------------------------------------------------
+namespace knet8 {
+
+struct GemmKey {
+  int dev, dtype, ta, tb, m, n, k, lda, ldb, ldc;
+  bool operator<(const GemmKey& o) const {
+    return std::tie(dev, dtype, ta, tb, m, n, k, lda, ldb, ldc) < std::tie(o.dev, o.dtype, o.ta, o.tb, o.m, o.n, o.k, o.lda, o.ldb, o.ldc);
+  }
+};
+struct GemmPlan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+  bool valid = false;
+};
+static std::mutex g_gemm_mutex;
+static std::map<int, hipblasLtHandle_t> g_lt;
+static std::map<GemmKey, GemmPlan> g_plans;
+static std::map<std::pair<int, hipStream_t>, void*> g_gemm_ws;
+static const size_t kGemmWorkspace = size_t(64) << 20;
+
+static bool lt_ok(hipblasStatus_t s, const char* what) {
+  if (s == HIPBLAS_STATUS_SUCCESS) return true;
+  char buf[128];
+  snprintf(buf, sizeof(buf), "hipBLASLt %s failed with status %d", what, (int)s);
+  record_error(buf);
+  return false;
+}
+
+template <typename T>
+static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
+                hipStream_t stream) {
+  if (m <= 0 || n <= 0) return 0;
+  const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
+  const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
+  const hipDataType dt = sizeof(T) == 4 ? HIP_R_32F : HIP_R_64F;
+  const hipblasComputeType_t ct = sizeof(T) == 4 ? HIPBLAS_COMPUTE_32F : HIPBLAS_COMPUTE_64F;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  std::lock_guard<std::mutex> lock(g_gemm_mutex);
+  hipblasLtHandle_t& h = g_lt[dev];
+  if (!h && !lt_ok(hipblasLtCreate(&h), "create")) return -1;
+  void*& ws = g_gemm_ws[std::make_pair(dev, stream)];
+  if (!ws && !ok(hipMalloc(&ws, kGemmWorkspace), "hipMalloc(gemm workspace)")) return -1;
+  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc};
+  GemmPlan& p = g_plans[key];
+  if (!p.valid) {
+    const hipblasOperation_t opa = ta ? HIPBLAS_OP_T : HIPBLAS_OP_N, opb = tb ? HIPBLAS_OP_T : HIPBLAS_OP_N;
+    if (!lt_ok(hipblasLtMatmulDescCreate(&p.desc, ct, dt), "desc create")) return -1;
+    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &opa, sizeof(opa)), "set transa")) return -1;
+    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &opb, sizeof(opb)), "set transb")) return -1;
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.la, dt, ta ? k : m, ta ? m : k, lda), "layout A")) return -1;
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lb, dt, tb ? n : k, tb ? k : n, ldb), "layout B")) return -1;
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lc, dt, m, n, ldc), "layout C")) return -1;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (!lt_ok(hipblasLtMatmulPreferenceCreate(&pref), "pref create")) return -1;
+    size_t wsbytes = kGemmWorkspace;
+    lt_ok(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsbytes, sizeof(wsbytes)), "pref workspace");
+    hipblasLtMatmulHeuristicResult_t res[1];
+    int found = 0;
+    const bool got = lt_ok(hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, res, &found), "heuristic");
+    hipblasLtMatmulPreferenceDestroy(pref);
+    if (!got || found < 1) {
+      record_error("hipBLASLt: no algorithm for this GEMM shape");
+      return -1;
+    }
+    p.algo = res[0].algo;
+    p.workspace = res[0].workspaceSize;
+    p.valid = true;
+  }
+  return lt_ok(hipblasLtMatmul(h, p.desc, &alpha, A, p.la, B, p.lb, &beta, C, p.lc, C, p.lc, &p.algo, ws, kGemmWorkspace, stream), "matmul") ? 0 : -1;
+}
+
+}  // namespace knet8
+
+extern "C" {
+KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta,
+                             float* C, int ldc, hipStream_t stream) {
+  return knet8::gemm<float>(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+KNET8_API int gemm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C,
+                      int ldc) {
+  return gemm_32_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, 0);
+}
+KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta,
+                             double* C, int ldc, hipStream_t stream) {
+  return knet8::gemm<double>(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta,
+                      double* C, int ldc) {
+  return gemm_64_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, 0);
+}
+}

@@ -1,0 +1,252 @@
+// Column softmax family: softmax / logsoftmax forward and backward and the fused nll+logsoftmax backward
+// down each contiguous column of an m x n column-major matrix (the reference's dims=1 case).
+//
+// The reference sends these to cuDNN (src/ops20_gpu/softmax.jl:44-56, LOG/ACCURATE algorithms,
+// MODE_INSTANCE on a (1,1,m,n) view); the arithmetic restated here is its CPU path
+// (src/ops20/softmax.jl:42-63), to which the reference's own tests pin cuDNN (test/loss.jl:87-92).
+//
+// One "team" of lanes owns a column and keeps it in registers, so every operand is read from HBM exactly
+// once and the result written once: the column is loaded with 16-byte vectors, reduced (max, then sum)
+// with wave64 butterflies (+ LDS across waves), transformed and stored.  Team size follows the column
+// length: one wave (m <= 4096), a 256-thread workgroup (m <= 16384) or a 1024-thread workgroup
+// (m <= 65536); longer columns fall back to a three-pass streaming kernel.
+//
+// HBM roofline: forward 2*sizeof(T)*m*n; backward 3*sizeof(T)*m*n; fused nll backward 2*sizeof(T)*m*n.
+#pragma once
+#include "knet8_device.h"
+
+namespace knet8 {
+
+template <typename T> __device__ __forceinline__ T dev_exp(T x);
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
+template <typename T> __device__ __forceinline__ T dev_log(T x);
+template <> __device__ __forceinline__ float dev_log<float>(float x) { return logf(x); }
+template <> __device__ __forceinline__ double dev_log<double>(double x) { return log(x); }
+
+// ---- algorithms -------------------------------------------------------------------------------------
+// a, b: the (up to) two inputs.  kInputs==1: a = x.  kInputs==2: a = y, b = dy.
+// kHoldA: a must stay in registers between the reduction and the output pass (false: it is only needed in
+// the output pass and is streamed there).  term(): summand of the column sum.  out(): the result.
+
+// y = (x - max) - log(sum(exp(x - max)))                      src/ops20/softmax.jl:42-47
+template <typename T> struct AlgoLogSoftmax {
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false;
+  __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
+  __device__ static T finish(T s) { return dev_log(s); }
+  __device__ static T out(T a, T, T mx, T fin) { return (a - mx) - fin; }
+};
+// y = exp(x - max) / sum(exp(x - max))                          src/ops20/softmax.jl:53-59
+template <typename T> struct AlgoSoftmax {
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false;
+  __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
+  __device__ static T finish(T s) { return s; }
+  __device__ static T out(T a, T, T mx, T fin) { return dev_exp(a - mx) / fin; }
+};
+// dx = dy - exp(y)*sum(dy)                                      src/ops20/softmax.jl:49-51
+template <typename T> struct AlgoLogSoftmaxBack {
+  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = false, kNll = false;
+  __device__ static T term(T, T b, T) { return b; }
+  __device__ static T finish(T s) { return s; }
+  __device__ static T out(T a, T b, T, T fin) { const T e = dev_exp(a); const T p = e * fin; return b - p; }
+};
+// dx = y*dy - y*sum(y*dy)                                       src/ops20/softmax.jl:61-63
+template <typename T> struct AlgoSoftmaxBack {
+  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = true, kNll = false;
+  __device__ static T term(T a, T b, T) { return a * b; }
+  __device__ static T finish(T s) { return s; }
+  __device__ static T out(T a, T b, T, T fin) { const T p = a * b; const T q = a * fin; return p - q; }
+};
+// Fused nll backward on raw scores: with lsm = logsoftmax(x) and dlp = -scale at the labelled row of each
+// counted column (0 elsewhere), dx = dlp - exp(lsm)*sum(dlp) -- the chain nll -> getindex -> logsoftmax of
+// src/ops20/loss.jl:37-41 and src/ops20/softmax.jl:49-51 -- and loss[col] = -lsm[label].  Label 0 skips
+// the column (dx = 0, loss = 0), as findindices does (src/ops20/loss.jl:125).
+template <typename T> struct AlgoNll {
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = true;
+  __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
+  __device__ static T finish(T s) { return dev_log(s); }
+  __device__ static T out(T a, T, T mx, T fin) { return (a - mx) - fin; }  // lsm; the kernel finishes the job
+};
+
+struct MaxFn { template <typename T> __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; } };
+struct AddFn { template <typename T> __device__ __forceinline__ T operator()(T a, T b) const { return a + b; } };
+
+template <typename T, int TEAM, typename Merge>
+__device__ __forceinline__ T team_reduce(T v, T* lds, Merge merge, T identity) {
+  if (TEAM == kWave) return wave_reduce(v, merge);
+  return block_reduce<T, TEAM / kWave>(v, lds, merge, identity);
+}
+
+// ---- register-resident column kernel -----------------------------------------------------------------
+// TEAM lanes per column (64: four columns per 256-thread workgroup; 256 or 1024: the whole workgroup),
+// E elements of each held input per lane, VEC: 16-byte accesses (m % N == 0 and 16-byte aligned operands).
+template <typename T, typename Algo, int TEAM, int E, bool VEC>
+__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out,
+                                                                                const int* labels, T scale, T* loss) {
+  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int TEAMS = BT / TEAM;
+  constexpr int NV = VEC ? Vec16<T>::N : 1;
+  constexpr int ITEMS = E / NV;
+  typedef typename Vec16<T>::type V;
+  __shared__ T lds[BT / kWave];
+  const int tl = threadIdx.x % TEAM;
+  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
+  const bool colok = col < n;       // only wave teams can be out of range, and those use no barriers
+  const long base = colok ? col * (long)m : 0;
+  const T* ac = a + base;
+  const T* bc = Algo::kInputs == 2 ? b + base : nullptr;
+  T* oc = out + base;
+
+  T ra[Algo::kHoldA ? E : 1], rb[Algo::kInputs == 2 ? E : 1];
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    const int r = (tl + i * TEAM) * NV;
+    const bool ok = colok && r < m;
+    if (VEC) {
+      V va = {}, vb = {};
+      if (ok && Algo::kHoldA) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+      if (ok && Algo::kInputs == 2) vb = ld_stream(reinterpret_cast<const V*>(bc + r));
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        if (Algo::kHoldA) ra[i * NV + e] = ok ? va[e] : T(0);
+        if (Algo::kInputs == 2) rb[i * NV + e] = ok ? vb[e] : T(0);
+      }
+    } else {
+      if (Algo::kHoldA) ra[i] = ok ? __builtin_nontemporal_load(ac + r) : T(0);
+      if (Algo::kInputs == 2) rb[i] = ok ? __builtin_nontemporal_load(bc + r) : T(0);
+    }
+  }
+
+  T mx = T(0);
+  if (Algo::kNeedMax) {
+    mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++)
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        const bool ok = colok && (tl + i * TEAM) * NV + e < m;
+        if (ok) mx = mx > ra[i * NV + e] ? mx : ra[i * NV + e];
+      }
+    mx = team_reduce<T, TEAM>(mx, lds, MaxFn(), T(-INFINITY));
+  }
+  T s = T(0);
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++)
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      const bool ok = colok && (tl + i * TEAM) * NV + e < m;
+      if (ok) s = s + Algo::term(Algo::kHoldA ? ra[i * NV + e] : T(0), Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx);
+    }
+  s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
+  const T fin = Algo::finish(s);
+
+  int lab = 0;
+  T st = T(0);
+  if (Algo::kNll) {
+    lab = colok ? labels[col] : 0;
+    st = -scale;  // sum of dlp over the column: its single non-zero entry
+  }
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    const int r = (tl + i * TEAM) * NV;
+    const bool ok = colok && r < m;
+    if (!ok) continue;
+    T o[NV];
+    V va = {};
+    if (!Algo::kHoldA) {
+      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+      else va[0] = __builtin_nontemporal_load(ac + r);
+    }
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      const T av = Algo::kHoldA ? ra[i * NV + e] : va[e];
+      T v = Algo::out(av, Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx, fin);
+      if (Algo::kNll) {
+        const bool hit = (r + e + 1 == lab);
+        if (hit) loss[col] = -v;
+        const T dlp = hit ? st : T(0);
+        const T p = dev_exp(v) * st;
+        v = lab == 0 ? T(0) : dlp - p;
+      }
+      o[e] = v;
+    }
+    if (VEC) {
+      V vo;
+#pragma unroll
+      for (int e = 0; e < NV; e++) vo[e] = o[e];
+      st_stream(reinterpret_cast<V*>(oc + r), vo);
+    } else {
+      __builtin_nontemporal_store(o[0], oc + r);
+    }
+  }
+  if (Algo::kNll && colok && lab == 0 && tl == 0) loss[col] = T(0);
+}
+
+// ---- streaming fallback for very long columns ----------------------------------------------------------
+// One 1024-thread workgroup per column; the inputs are read once per pass (max, sum, output).
+template <typename T, typename Algo>
+__global__ __launch_bounds__(1024) void softmax_col_stream_kernel(long m, long n, const T* a, const T* b, T* out, const int* labels,
+                                                                  T scale, T* loss) {
+  __shared__ T lds[1024 / kWave];
+  const long col = blockIdx.x;
+  const T* ac = a + col * m;
+  const T* bc = Algo::kInputs == 2 ? b + col * m : nullptr;
+  T* oc = out + col * m;
+  T mx = T(0);
+  if (Algo::kNeedMax) {
+    mx = -INFINITY;
+    for (long r = threadIdx.x; r < m; r += 1024) { const T v = ac[r]; mx = mx > v ? mx : v; }
+    mx = block_reduce<T, 1024 / kWave>(mx, lds, MaxFn(), T(-INFINITY));
+  }
+  T s = T(0);
+  for (long r = threadIdx.x; r < m; r += 1024) s = s + Algo::term(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx);
+  s = block_reduce<T, 1024 / kWave>(s, lds, AddFn(), T(0));
+  const T fin = Algo::finish(s);
+  const int lab = Algo::kNll ? labels[col] : 0;
+  const T st = -scale;
+  for (long r = threadIdx.x; r < m; r += 1024) {
+    T v = Algo::out(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx, fin);
+    if (Algo::kNll) {
+      const bool hit = (r + 1 == lab);
+      if (hit) loss[col] = -v;
+      const T dlp = hit ? st : T(0);
+      const T p = dev_exp(v) * st;
+      v = lab == 0 ? T(0) : dlp - p;
+    }
+    oc[r] = v;
+  }
+  if (Algo::kNll && lab == 0 && threadIdx.x == 0) loss[col] = T(0);
+}
+
+template <typename T, typename Algo, int TEAM, int E>
+inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, const T* a, const T* b, T* out, const int* labels,
+                               T scale, T* loss) {
+  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int TEAMS = BT / TEAM;
+  const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS)), block(BT);
+  if (vec)
+    hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+  else
+    hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+}
+
+template <typename T, typename Algo>
+inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const T* b, T* out, const int* labels, T scale, T* loss) {
+  if (m <= 0 || n <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  // two held inputs double the register footprint: halve the per-lane capacity
+  constexpr int kBig = (Algo::kInputs == 2 && Algo::kHoldA) ? 32 : 64;
+  const bool vec = (m % N == 0) && aligned16(a) && aligned16(out) && (Algo::kInputs == 1 || aligned16(b));
+#define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
+  if (m <= 64 * 4) KNET8_SM(64, 4);
+  else if (m <= 64 * 16) KNET8_SM(64, 16);
+  else if (m <= 64 * kBig) KNET8_SM(64, kBig);
+  else if (m <= 256 * kBig) KNET8_SM(256, kBig);
+  else if (m <= 1024 * 32) KNET8_SM(1024, 32);
+  else if (m <= 1024 * kBig) KNET8_SM(1024, kBig);
+  else
+    hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
+#undef KNET8_SM
+}
+
+}  // namespace knet8

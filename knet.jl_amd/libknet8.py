@@ -1,0 +1,85 @@
+"""Loader of ``libknet8.so`` and the thin call layer over its C ABI.
+
+The counterpart of the reference's src/libknet8/LibKnet8.jl: locate the shared library (``:7``) and
+give the rest of the package ``knet8(fun, *args)``, which -- like the ``@knet8`` macro (``:50-55``) --
+calls the ``<fun>_stream`` entry point with the current stream appended.  Argument types come from
+``include/knet8.h`` so the Python side cannot drift from the header.
+
+There is no CPU fallback: if the library is missing or a symbol is absent, loading fails with an error.
+"""
+import ctypes
+import os
+import re
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_PKG)
+LIB_PATH = os.environ.get("KNET8_LIBRARY", os.path.join(_PKG, "lib", "libknet8.so"))
+HEADER_PATH = os.path.join(_ROOT, "include", "knet8.h")
+
+_CTYPES = {
+    "void": None, "int": ctypes.c_int, "float": ctypes.c_float, "double": ctypes.c_double, "char": ctypes.c_char,
+    "size_t": ctypes.c_size_t, "hipStream_t": ctypes.c_void_p, "float*": ctypes.c_void_p, "double*": ctypes.c_void_p,
+    "int*": ctypes.c_void_p, "void*": ctypes.c_void_p, "const void*": ctypes.c_void_p, "size_t*": ctypes.c_void_p,
+    "const char*": ctypes.c_char_p,
+}
+_DECL = re.compile(r"KNET8_API\s+(.+?)\s*\b(\w+)\s*\(([^)]*)\)\s*;")
+
+
+def parse_header(path=HEADER_PATH):
+    """{symbol: (restype, [argtypes])} for every entry point the header declares."""
+    text = open(path).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for ret, name, params in _DECL.findall(text):
+        args = []
+        params = params.strip()
+        if params and params != "void":
+            for p in params.split(","):
+                p = p.strip()
+                ty = p.rsplit(" ", 1)[0].strip() if " " in p else p
+                if p.endswith("*"):
+                    ty = p
+                args.append(ty.replace(" *", "*"))
+        out[name] = (ret.strip(), args)
+    return out
+
+
+class LibKnet8:
+    def __init__(self, path=LIB_PATH):
+        if not os.path.exists(path):
+            raise OSError("libknet8.so not found at %s -- build it first (python __graft_entry__.py build); "
+                          "there is no CPU fallback" % path)
+        self.path = path
+        self.lib = ctypes.CDLL(path)
+        self.decls = parse_header()
+        self.fn = {}
+        for name, (ret, args) in self.decls.items():
+            f = getattr(self.lib, name)  # AttributeError if the library lacks a declared symbol
+            f.restype = _CTYPES[ret]
+            f.argtypes = [_CTYPES[a] for a in args]
+            self.fn[name] = f
+        self.stream = None  # current stream handle (None = null stream), cf. CUDA.stream() in the reference
+
+    def check(self):
+        msg = self.fn["knet8_last_error"]()
+        if msg:
+            raise RuntimeError("libknet8: " + msg.decode())
+
+    def call(self, fun, *args):
+        """``@knet8(fun, ...)``: asynchronous launch of ``<fun>_stream`` on the current stream."""
+        r = self.fn[fun + "_stream"](*args, self.stream)
+        return r
+
+
+_LIB = None
+
+
+def libknet8():
+    global _LIB
+    if _LIB is None:
+        _LIB = LibKnet8()
+    return _LIB
+
+
+def knet8(fun, *args):
+    return libknet8().call(fun, *args)

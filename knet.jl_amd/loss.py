@@ -1,0 +1,127 @@
+"""``nll``, ``findindices``, ``accuracy`` and the gather / scatter they rest on.
+
+Mirrors src/ops20/loss.jl:37-41,116-140 and the device side of ``x[indices]`` and its gradient:
+``getindex(x, ::Array{Int})`` -> ``getents_S`` (src/knetarrays/getindex.jl:217-220,291-298) and
+``ungetindex`` -> zero-filled array + ``addents_S`` (src/autograd_gpu/getindex.jl:5-13, addto.jl:59-65).
+"""
+import numpy as np
+
+from .autograd import primitive, recording, track, value
+from .karray import KnetArray
+from .libknet8 import knet8, libknet8
+from . import reduction as R
+from .softmax import logsoftmax
+
+
+def findindices(scores, labels, dims=1):
+    """1-based linear indices of the labelled entries; label 0 skips the instance (src/ops20/loss.jl:116-140)."""
+    labels = np.asarray(labels)
+    if not np.issubdtype(labels.dtype, np.integer):
+        raise TypeError("MethodError: labels must be integers")
+    lab = labels.ravel(order="F").astype(np.int64)
+    ninstances = lab.size
+    size = scores.dims if isinstance(scores, KnetArray) else tuple(np.shape(scores))
+    length = int(np.prod(size, dtype=np.int64))
+    if dims == 1:
+        y1 = size[0]
+        y2 = length // y1 if y1 else 0
+        if ninstances != y2:
+            raise ValueError("DimensionMismatch")
+        j = np.nonzero(lab)[0]
+        return j * y1 + lab[j]
+    if dims == 2:
+        y2 = size[-1]
+        y1 = length // y2 if y2 else 0
+        if ninstances != y1:
+            raise ValueError("DimensionMismatch")
+        j = np.nonzero(lab)[0]
+        return (lab[j] - 1) * y1 + j + 1
+    raise ValueError("findindices only supports dims = 1 or 2")
+
+
+def _device_indices(x, indices):
+    idx = np.asarray(indices, dtype=np.int64).ravel()
+    if idx.size and (idx.min() < 1 or idx.max() > x.length):  # bounds check on the host, getindex.jl:277-287
+        raise IndexError("BoundsError")
+    return KnetArray(idx.astype(np.int32))
+
+
+def ungetindex(x, dxi, indices):
+    """Gradient of ``x[indices]``: zeros like ``x`` with ``dxi`` added at ``indices``."""
+    dx = x.similar()
+    knet8("fill_%s" % x.suffix, dx.length, x.ctype(0), dx.ptr)
+    ents = _device_indices(x, indices)
+    knet8("addents_%s" % x.suffix, ents.length, ents.ptr, dx.ptr, dxi.ptr)
+    return dx
+
+
+@primitive
+def getindex(x, indices):
+    """``x[indices]`` for an integer index array (1-based linear indices) -> vector."""
+    ents = _device_indices(x, indices)
+    y = x.similar((ents.length,))
+    knet8("getents_%s" % x.suffix, ents.length, ents.ptr, x.ptr, y.ptr)
+    return y, (lambda dy: (ungetindex(x, dy, indices), None))
+
+
+@primitive
+def _nll_fused(scores, labels, dims=1):
+    """nll and its gradient wrt ``scores`` in one pass over the scores (``nll_logsoftmax_back_S``)."""
+    if dims != 1 or scores.ndims != 2:
+        raise NotImplementedError("fused nll needs a (classes, instances) matrix and dims=1")
+    m, n = scores.dims
+    lab = np.asarray(labels).ravel(order="F")
+    if lab.size != n:
+        raise ValueError("DimensionMismatch")
+    if lab.size and (lab.min() < 0 or lab.max() > m):
+        raise IndexError("BoundsError")
+    count = int(np.count_nonzero(lab))
+    T = scores.dtype.type
+    dlab = KnetArray(lab.astype(np.int32))
+    dx = scores.similar()
+    lossv = scores.similar((n,))
+    scale = T(1) / T(count) if count else T(np.inf)
+    knet8("nll_logsoftmax_back_%s" % scores.suffix, m, n, scores.ptr, dlab.ptr, scores.ctype(scale), dx.ptr, lossv.ptr)
+    total = R.reduce_op("sum", lossv)
+    loss = T(total) / T(count)
+
+    def back(dy):
+        from .linalg import scal
+        if float(dy) != 1.0:
+            scal(float(dy), dx)
+        return (dx, None)
+    return loss, back
+
+
+def nll(scores, labels, dims=1, average=True, fused=False):
+    """``nll(scores, labels; dims=1, average=true)`` (src/ops20/loss.jl:37-41).
+
+    ``fused=False`` follows the reference step by step (logsoftmax, gather, sum); ``fused=True`` computes the loss
+    and, when recording, the gradient with the single-pass kernel (same result within rounding).
+    """
+    if fused and average:
+        return _nll_fused(scores, labels, dims=dims)
+    indices = findindices(value(scores), labels, dims=dims)
+    lp = getindex(logsoftmax(scores, dims=dims), indices)
+    n = len(indices)
+    total = R.sum(lp)
+    return _neg_div(total, n) if average else (_neg_div(total, 1), n)
+
+
+@primitive
+def _neg_div(total, n):
+    """``-sum(lp) / length(lp)`` on host scalars."""
+    T = type(total)
+    return -total / T(n), (lambda dy: (-(T(dy) / T(n)), None))
+
+
+def accuracy(scores, labels, dims=1, average=True):
+    """Ratio of instances whose labelled class has the largest score (src/ops20/loss.jl:52-62); as in the
+    reference the scores are brought to the host for ``findmax``."""
+    s = value(scores).to_numpy()
+    lab = np.asarray(labels).ravel(order="F")
+    pred = s.argmax(axis=0 if dims == 1 else s.ndim - 1).ravel(order="F") + 1
+    keep = lab != 0
+    correct = int(np.count_nonzero(pred[keep] == lab[keep]))
+    count = int(np.count_nonzero(keep))
+    return correct / count if average else (correct, count)

@@ -1,0 +1,102 @@
+"""``softmax / logsoftmax / logsumexp`` on ``KnetArray`` and their gradients.
+
+Mirrors src/ops20_gpu/softmax.jl:10-59.  There ``dims=:`` or ``dims=1`` reshape to ``(1,1,m,n)`` and call
+cuDNN (``_cudnnSoftmaxForward`` LOG / ACCURATE, backward ``_cudnnSoftmaxBackward``); here the same cases
+call ``logsoftmax_S / softmax_S`` and ``logsoftmaxback_S / softmaxback_S`` of libknet8.  2-d ``dims=2`` goes
+through a transpose as in the reference (``:19-20``); other ``dims`` use the generic formulation
+(src/ops20/softmax.jl:42-74) built from reductions and broadcasts.
+"""
+from .autograd import primitive
+from .karray import KnetArray
+from .libknet8 import knet8
+from . import reduction as R
+
+
+def _columns(x, dims):
+    """(m, n) when the softmax runs down contiguous columns, else None."""
+    if dims is None or (x.ndims == 1 and dims in (1, [1], (1,))):
+        return x.length, 1
+    d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
+    if d == list(range(1, len(d) + 1)):  # leading dims: softmax over the first prod(size[1:k]) elements of each slab
+        m = 1
+        for i in d:
+            m *= x.size(i)
+        return m, (x.length // m if m else 0)
+    return None
+
+
+def _fwd(kernel, x, m, n):
+    y = x.similar()
+    knet8("%s_%s" % (kernel, x.suffix), m, n, x.ptr, y.ptr)
+    return y
+
+
+def _bwd(kernel, y, dy, m, n):
+    dx = y.similar()
+    knet8("%s_%s" % (kernel, y.suffix), m, n, y.ptr, dy.ptr, dx.ptr)
+    return dx
+
+
+def permutedims(x):
+    """2-d transpose (the reference uses CUDA.jl's permutedims, src/knetarrays/reshape.jl:18)."""
+    from .linalg import transpose
+    return transpose(x)
+
+
+def _make(kernel, backkernel):
+    @primitive
+    def f(x, dims=None):
+        if not isinstance(x, KnetArray):
+            raise TypeError("MethodError: expected a KnetArray")
+        if x.length == 0:
+            return x.similar(), (lambda dy: (dy,))
+        mn = _columns(x, dims)
+        if mn is not None:
+            m, n = mn
+            y = _fwd(kernel, x, m, n)
+            return y, (lambda dy: (_bwd(backkernel, y, dy, m, n),))  # @primitive1 _cudnnSoftmaxForward(x),dy,y _cudnnSoftmaxBackward(y,dy)
+        d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
+        if x.ndims == 2 and d == [2]:
+            xt = permutedims(x)
+            m, n = xt.size(1), xt.size(2)
+            yt = _fwd(kernel, xt, m, n)
+            y = permutedims(yt)
+            return y, (lambda dy: (permutedims(_bwd(backkernel, yt, permutedims(dy), m, n)),))
+        raise NotImplementedError("softmax over dims=%r of a %d-d array" % (dims, x.ndims))
+
+    f.__name__ = kernel
+    return f
+
+
+logsoftmax = _make("logsoftmax", "logsoftmaxback")
+softmax = _make("softmax", "softmaxback")
+logp = logsoftmax  # const logp = logsoftmax  (src/ops20/softmax.jl:40)
+
+
+def logsoftmaxback(y, dy, dims=None):
+    """``∇logsoftmax``: ``dy - exp.(y).*sum(dy;dims)`` (src/ops20/softmax.jl:49-51)."""
+    m, n = _columns(y, dims)
+    return _bwd("logsoftmaxback", y, dy, m, n)
+
+
+def softmaxback(y, dy, dims=None):
+    """``∇softmax``: ``y.*dy .- y.*sum(y.*dy;dims)`` (src/ops20/softmax.jl:61-63)."""
+    m, n = _columns(y, dims)
+    return _bwd("softmaxback", y, dy, m, n)
+
+
+def logsumexp(x, dims=None):
+    """``xmax + log.(sum(exp.(x .- xmax)))`` (src/ops20/softmax.jl:65-70), from the logsoftmax kernel:
+    logsumexp = x - logsoftmax(x) at any one position of the reduced slice."""
+    mn = _columns(x, dims)
+    if mn is None:
+        raise NotImplementedError("logsumexp over dims=%r" % (dims,))
+    m, n = mn
+    y = _fwd("logsoftmax", x, m, n)
+    from .binary import broadcast_op
+    diff = broadcast_op("sub", x, y)  # every row of a column holds the same value: take the maximum to pick one
+    out = R.reduce_op("maximum", diff.reshape(m, n), 1)
+    if dims is None:
+        return out.to_numpy().ravel()[0]
+    d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
+    return out.reshape(tuple(1 if (i + 1) in d else x.dims[i] for i in range(x.ndims)))

@@ -1,0 +1,183 @@
+"""GPU parity of the elementwise kernel family against the CPU oracle, through the C ABI.
+
+Tolerances (north star): bit-exact for reluback and everything without a libm call (the library is built with
+-ffp-contract=off, so the device evaluates the same IEEE operations in the same order as the oracle);
+<= 2 ulp for forwards that call exp/tanh/erf, measured at the magnitude of the libm result.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from gpu_util import SPECIALS, bits_equal, misaligned, ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 3, 4, 5, 63, 64, 255, 256, 257, 1023, 1025, 100003, (1 << 20) + 7]
+BACK11 = [("reluback", "relu"), ("sigmback", "sigm"), ("tanhback", "tanh"), ("eluback", "elu"), ("seluback", "selu")]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("name,fwd", BACK11)
+def test_back11_bit_exact(knet, oracle, name, fwd, dt):
+    rng = np.random.default_rng(11)
+    for n in SIZES:
+        x = rng.standard_normal(n).astype(dt)
+        y = oracle.unary(fwd, x)
+        dy = rng.standard_normal(n).astype(dt)
+        got = knet.Array(getattr(knet, name)(knet.KnetArray(dy), knet.KnetArray(y)))
+        assert bits_equal(got, oracle.back11(name, dy, y)), (name, n)
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("name,fwd", BACK11)
+def test_back11_special_values(knet, oracle, name, fwd):
+    for dt in (np.float32, np.float64):
+        pairs = np.array(list(itertools.product(SPECIALS, SPECIALS)), dtype=dt)
+        dy, y = pairs[:, 0].copy(), pairs[:, 1].copy()
+        with np.errstate(all="ignore"):
+            want = oracle.back11(name, dy, y)
+        got = knet.Array(getattr(knet, name)(knet.KnetArray(dy), knet.KnetArray(y)))
+        assert bits_equal(got, want), name
+
+
+@pytest.mark.parametrize("offs", [(1, 1, 1), (1, 2, 3), (0, 1, 0), (3, 3, 0), (2, 0, 2)])
+def test_back11_on_misaligned_views(knet, oracle, offs):
+    # sub-array views start at arbitrary element offsets (src/knetarrays/getindex.jl:153-159)
+    rng = np.random.default_rng(12)
+    for dt in (np.float32, np.float64):
+        for n in (1, 2, 7, 1000, 70001):
+            y = oracle.unary("sigm", rng.standard_normal(n).astype(dt))
+            dy = rng.standard_normal(n).astype(dt)
+            dyd, yd = misaligned(knet, dy, offs[0]), misaligned(knet, y, offs[1])
+            out_big = knet.KnetArray(np.full(n + offs[2] + 5, 7.0, dt))
+            out = out_big.view1d(offs[2], n)
+            S = "32" if dt == np.float32 else "64"
+            knet.knet8("sigmback_%s_11" % S, n, dyd.ptr, yd.ptr, out.ptr)
+            full = knet.Array(out_big)
+            assert bits_equal(full[offs[2]: offs[2] + n], oracle.back11("sigmback", dy, y))
+            assert np.all(full[: offs[2]] == 7) and np.all(full[offs[2] + n:] == 7)  # nothing written outside
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("name", ["relu", "sigm", "tanh", "elu", "selu", "gelu", "hardsigmoid", "hardswish", "swish", "tanh_"])
+def test_forward_within_2ulp(knet, oracle, name, dt):
+    rng = np.random.default_rng(13)
+    x = np.concatenate([rng.standard_normal(200001) * 3, [0.0, -0.0, 3.0, -3.0, 30.0, -30.0, 90.0, -90.0]]).astype(dt)
+    oname = "tanh" if name == "tanh_" else name
+    want = oracle.unary(oname, x)
+    got = knet.Array(knet.unary_op(name, knet.KnetArray(x)))
+    if name in ("relu", "hardsigmoid", "hardswish"):  # no libm call: exact
+        assert bits_equal(got, want)
+    else:
+        # exp(x)-1 and x*(1+erf) cancel near 0: the yardstick is the libm result's magnitude (<= 1), not the output's
+        scale = np.maximum(np.abs(want), 1.0) if name in ("elu", "selu", "gelu", "swish") else None
+        assert ulp_diff(got, want, scale).max() <= 2, name
+
+
+def test_relu_nan_and_negative_zero_follow_the_cpu_path(knet):
+    x = np.float32([np.nan, -0.0, 0.0, -1.0, 2.0])
+    got = knet.Array(knet.relu(knet.KnetArray(x)))
+    assert np.isnan(got[0]) and not np.signbit(got[1]) and got[3] == 0 and got[4] == 2
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("name,fwd", [("eluback", "elu"), ("seluback", "selu"), ("sigmback", "sigm"), ("tanh_back", "tanh"),
+                                      ("geluback", "gelu"), ("hardsigmoidback", "hardsigmoid"), ("hardswishback", "hardswish"),
+                                      ("swishback", "swish")])
+def test_back111(knet, oracle, name, fwd, dt):
+    rng = np.random.default_rng(14)
+    for n in (0, 5, 1000, 65537):
+        x = (rng.standard_normal(n) * 2.5).astype(dt)
+        y = oracle.unary(fwd, x)
+        dy = rng.standard_normal(n).astype(dt)
+        got = knet.Array(knet.back111_op(name, knet.KnetArray(x), knet.KnetArray(y), knet.KnetArray(dy)))
+        want = oracle.back111(name, x, y, dy)
+        if name in ("geluback", "swishback"):
+            assert ulp_diff(got, want, np.maximum(np.abs(want), np.abs(dy))).max(initial=0) <= 8, name  # the libm result (device and glibc may differ by 1 ulp) enters the quotient three times
+        else:
+            assert bits_equal(got, want), name
+
+
+def test_relu_with_keyword_arguments(knet, oracle):
+    # settings of test/ops21/activation.jl:45-60
+    rng = np.random.default_rng(15)
+    x = (rng.standard_normal(10001) * 2).astype(np.float32)
+    dy = rng.standard_normal(10001).astype(np.float32)
+    for kw in (dict(), dict(max_value=1.0), dict(negative_slope=0.5), dict(threshold=1.0), dict(max_value=2.0, negative_slope=0.25, threshold=0.5)):
+        xd = knet.KnetArray(x)
+        y = knet.relu_kw(xd, **kw)
+        assert bits_equal(knet.Array(y), oracle.relu_kw(x, **kw)), kw
+        got = knet.Array(knet.relu_kw_back(xd, y, knet.KnetArray(dy), **kw))
+        assert bits_equal(got, oracle.reluback_kw(x, knet.Array(y), dy, **kw)), kw
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("p", [0.5, 0.25, 0.9])
+def test_dropout_and_dropback_bit_exact_given_the_uniform_buffer(knet, oracle, dt, p):
+    rng = np.random.default_rng(16)
+    for n in (1, 6, 4097, 300001):
+        x = rng.standard_normal(n).astype(dt)
+        x[::7] = 0  # a kept element whose x == 0 is treated as dropped by dropback (mask is inferred from y == 0)
+        u = rng.random(n).astype(dt)
+        y = knet.dropout(knet.KnetArray(x), p, drop=True, uniform=u)
+        want_y = oracle.dropout(x, p, u)
+        assert bits_equal(knet.Array(y), want_y)
+        dy = rng.standard_normal(n).astype(dt)
+        dx = knet.dropback(knet.KnetArray(dy), y, knet.KnetArray(x), p)
+        assert bits_equal(knet.Array(dx), oracle.dropback(p, x, want_y, dy))
+    # p = 0 and p = 1 short-circuit on the host (src/ops20/dropout.jl:19-25)
+    xd = knet.KnetArray(np.float32([1, 2, 3]))
+    assert knet.dropout(xd, 0, drop=True) is xd
+    assert np.array_equal(knet.Array(knet.dropout(xd, 1, drop=True)), np.zeros(3, np.float32))
+    with pytest.raises(ValueError):
+        knet.dropout(xd, 1.5, drop=True)
+    assert knet.dropout(xd, 0.5) is xd  # not recording: identity
+
+
+def test_fill_axpy_scal_and_binary(knet):
+    rng = np.random.default_rng(17)
+    for dt in (np.float32, np.float64):
+        for n in (1, 5, 1000, 100001):
+            a = rng.standard_normal(n).astype(dt)
+            b = rng.standard_normal(n).astype(dt)
+            ad, bd = knet.KnetArray(a), knet.KnetArray(b)
+            assert bits_equal(knet.Array(knet.fill(ad.similar(), 2.5)), np.full(n, 2.5, dt))
+            assert bits_equal(knet.Array(knet.add(ad, bd)), a + b)
+            assert bits_equal(knet.Array(knet.sub(ad, bd)), a - b)
+            assert bits_equal(knet.Array(knet.mul(ad, bd)), a * b)
+            assert bits_equal(knet.Array(knet.div(ad, bd)), a / b)
+            assert bits_equal(knet.Array(knet.mul(dt(3), ad)), dt(3) * a)
+            assert bits_equal(knet.Array(knet.sub(ad, 2)), a + dt(-2))
+            assert bits_equal(knet.Array(knet.axpy(0.5, ad, bd.copy())), b + dt(0.5) * a)
+            assert bits_equal(knet.Array(knet.scal(0.25, ad.copy())), dt(0.25) * a)
+
+
+def test_bias_add_broadcast_and_unbroadcast(knet, oracle):
+    rng = np.random.default_rng(18)
+    for shape, bshape in [((64, 100), (64, 1)), ((64, 100), (1, 100)), ((5, 6, 7, 3), (1, 1, 7, 1)), ((513, 1025), (1, 1025)), ((7, 9), (7, 9))]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        b = rng.standard_normal(bshape).astype(np.float32)
+        assert bits_equal(knet.Array(knet.add(knet.KnetArray(x), knet.KnetArray(b))), x + b)
+        assert bits_equal(knet.Array(knet.add(knet.KnetArray(b), knet.KnetArray(x))), b + x)
+        dy = rng.integers(-3, 4, size=shape).astype(np.float32)  # integer-valued: the sum is exact
+        g = knet.unbroadcast(knet.KnetArray(b), knet.KnetArray(dy))
+        axes = tuple(i for i in range(len(shape)) if bshape[i] == 1 and shape[i] > 1)
+        want = dy.sum(axis=axes, keepdims=True) if axes else dy
+        assert g.dims == tuple(bshape) and np.array_equal(knet.Array(g), want)
+    with pytest.raises(ValueError):
+        knet.add(knet.KnetArray(np.zeros((3, 4), np.float32)), knet.KnetArray(np.zeros((4, 3), np.float32)))
+
+
+def test_error_behaviour(knet):
+    a = knet.KnetArray(np.zeros(4, np.float32))
+    b = knet.KnetArray(np.zeros(5, np.float32))
+    c = knet.KnetArray(np.zeros(4, np.float64))
+    with pytest.raises(ValueError):
+        knet.reluback(a, b)
+    with pytest.raises(TypeError):
+        knet.reluback(a, c)
+    with pytest.raises(TypeError):
+        knet.reluback(a, np.zeros(4, np.float32))
+    with pytest.raises(TypeError):
+        knet.KnetArray(np.zeros(3, np.int64))

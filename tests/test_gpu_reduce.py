@@ -1,0 +1,133 @@
+"""GPU parity of the reduction family (`_20`, `_21`, `_22` and the `sum(x; dims)` dispatcher) against the oracle.
+
+Tolerance (north star): 1e-5 relative.  For sums the oracle holds the correctly rounded result; the device
+accumulates in T in a fixed tree order, so the comparison is |gpu - oracle| <= 1e-5 * sum|x| per output (relative
+to the magnitude being summed) and, norm-wise, 1e-5 relative as the reference's own isapprox does
+(src/knetarrays/comparison.jl:12-14).  Integer-valued inputs must match exactly.  max/min-like ops are exact.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+OPS = ["sum", "prod", "maximum", "minimum", "sumabs", "sumabs2", "maxabs", "minabs", "countnz"]
+
+
+def check_sum(got, want, x, axes, rtol=1e-5):
+    mag = np.abs(x.astype(np.float64)).sum(axis=axes, keepdims=True)
+    assert got.shape == want.shape
+    assert np.all(np.abs(got.astype(np.float64) - want) <= rtol * mag + 1e-30)
+    assert np.linalg.norm(got.astype(np.float64) - want) <= rtol * max(np.linalg.norm(want), np.linalg.norm(got))
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (4, 1, 3), (2, 2, 2, 3), (5,), (3, 4), (8, 4, 2, 16), (32, 8), (1, 1), (2, 1), (1, 2)])
+def test_every_dim_subset_every_op_exact_on_integers(knet, oracle, shape):
+    # mirrors test/reduction.jl:41-58,114-142
+    rng = np.random.default_rng(21)
+    nd = len(shape)
+    for dt in (np.float32, np.float64):
+        x = rng.integers(-3, 4, size=shape).astype(dt)
+        x[x == 0] = 1 if x.size < 40 else 0  # small arrays: keep prod away from 0; larger: exercise countnz
+        xd = knet.KnetArray(x)
+        for op in OPS:
+            assert float(knet.reduce_op(op, xd)) == float(oracle.reduce(op, x)), (op, "all")
+            for r in range(1, nd + 1):
+                for dims in itertools.combinations(range(1, nd + 1), r):
+                    got = knet.Array(knet.reduce_op(op, xd, dims=list(dims) if r > 1 else dims[0]))
+                    want = oracle.reduce(op, x, dims=dims)
+                    assert got.shape == want.shape and np.array_equal(got, want), (op, dims, shape)
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("shape", [(10, 100000), (100000, 10), (1000, 1000), (513, 1025), (3, 70000, 5), (65, 3, 1031)])
+def test_large_dims_regression_shapes(knet, oracle, shape):
+    # test/reduction.jl:59-70 ("kernel bug with dims > 64K"), prof/reduction.jl:42-61 (1000 x 1000)
+    rng = np.random.default_rng(22)
+    for dt in (np.float32, np.float64):
+        x = rng.standard_normal(shape).astype(dt)
+        xd = knet.KnetArray(x)
+        rtol = 1e-5 if dt == np.float32 else 1e-12
+        for d in range(1, len(shape) + 1):
+            got = knet.Array(knet.sum(xd, dims=d))
+            check_sum(got, oracle.reduce("sum", x, dims=d).astype(np.float64), x, d - 1, rtol)
+            assert np.array_equal(knet.Array(knet.maximum(xd, dims=d)), oracle.reduce("maximum", x, dims=d))
+            got = knet.Array(knet.sumabs2(xd, dims=d))
+            check_sum(got, oracle.reduce("sumabs2", x, dims=d).astype(np.float64), x * x, d - 1, rtol)
+        tot = float(knet.sum(xd))
+        assert abs(tot - float(oracle.reduce("sum", x))) <= rtol * np.abs(x).sum()
+        # sum(dims=1) then sum(dims=2...) equals sum(:)
+        y = xd
+        for d in range(1, len(shape) + 1):
+            y = knet.sum(y, dims=d)
+        assert abs(float(knet.Array(y).ravel()[0]) - tot) <= rtol * np.abs(x).sum()
+
+
+def test_raw_21_and_22_entry_points_on_odd_shapes_and_misaligned_views(knet, oracle):
+    from gpu_util import misaligned
+    rng = np.random.default_rng(23)
+    for dt, S in ((np.float32, "32"), (np.float64, "64")):
+        for (sy, ny, no) in [(1, 7, 13), (5, 3, 9), (1, 300, 1000), (1, 4096, 64), (257, 3, 4), (4, 1000, 1), (4096, 5, 3), (3136, 16, 8),
+                             (1, 1, 1000), (100, 1, 1), (2, 3, 20000), (12, 77, 5), (1, 63, 5000), (1, 64, 5000), (1, 65, 3000)]:
+            x = rng.integers(-4, 5, size=(sy, ny, no)).astype(dt)
+            want = x.sum(axis=(0, 2))
+            for off in (0, 1, 3):
+                xd = misaligned(knet, x, off)
+                y = knet.KnetArray(np.zeros(ny, dt))
+                knet.knet8("sum_%s_21" % S, x.size, xd.ptr, sy, ny, y.ptr)
+                assert np.array_equal(knet.Array(y), want), (sy, ny, no, off)
+        for (s1, d, nb) in [(1, 9, 5), (3, 7, 2), (64, 100, 3), (256, 33, 2), (300, 1000, 1), (5, 20000, 2), (2, 3, 4000), (1000, 3, 7)]:
+            x = rng.integers(-4, 5, size=(s1, d, nb)).astype(dt)
+            want = x.max(axis=1)
+            wsum = x.sum(axis=1)
+            for off in (0, 1):
+                xd = misaligned(knet, x, off)
+                y = knet.KnetArray(np.zeros((s1, nb), dt))
+                knet.knet8("maximum_%s_22" % S, x.size, d - 1, xd.ptr, s1, s1 * d, s1 * nb, y.ptr)
+                assert np.array_equal(knet.Array(y), want), (s1, d, nb, off)
+                knet.knet8("sum_%s_22" % S, x.size, d - 1, xd.ptr, s1, s1 * d, s1 * nb, y.ptr)
+                assert np.array_equal(knet.Array(y), wsum), (s1, d, nb, off)
+    knet.libknet8().check()
+
+
+def test_repeated_launches_reuse_the_scratch_correctly(knet):
+    # split reductions keep per-stream tickets that every launch must leave at zero
+    rng = np.random.default_rng(24)
+    x = rng.integers(-4, 5, size=(4096, 512)).astype(np.float32)
+    xd = knet.KnetArray(x)
+    w1, w2, w0 = x.sum(axis=0, keepdims=True), x.sum(axis=1, keepdims=True), x.sum()
+    for _ in range(5):
+        assert np.array_equal(knet.Array(knet.sum(xd, dims=2)), w2)
+        assert np.array_equal(knet.Array(knet.sum(xd, dims=1)), w1)
+        assert float(knet.sum(xd)) == w0
+    small = knet.KnetArray(x[:7, :5].copy())
+    assert np.array_equal(knet.Array(knet.sum(small, dims=2)), x[:7, :5].sum(axis=1, keepdims=True))
+
+
+def test_config3_full_size(knet, oracle):
+    """BASELINE config 3: dy (4096,8192) over dims=1 and dims=2; NCHW bias gradient (56,56,256,64) -> (1,1,256,1)."""
+    rng = np.random.default_rng(25)
+    x = rng.standard_normal((4096, 8192), dtype=np.float32)
+    xd = knet.KnetArray(x)
+    for d in (1, 2):
+        got = knet.Array(knet.sum(xd, dims=d))
+        check_sum(got, oracle.reduce("sum", x, dims=d).astype(np.float64), x, d - 1)
+    x = rng.standard_normal((56, 56, 256, 64), dtype=np.float32)
+    xd = knet.KnetArray(x)
+    got = knet.Array(knet.sum(xd, dims=[1, 2, 4]))
+    assert got.shape == (1, 1, 256, 1)
+    check_sum(got, oracle.reduce("sum", x, dims=(1, 2, 4)).astype(np.float64), x, (0, 1, 3))
+    # exactness on integer-valued data at the full shape (every element is visited exactly once)
+    xi = rng.integers(-2, 3, size=(56, 56, 256, 64)).astype(np.float32)
+    got = knet.Array(knet.sum(knet.KnetArray(xi), dims=[1, 2, 4]))
+    assert np.array_equal(got.ravel(), xi.sum(axis=(0, 1, 3), dtype=np.float64).astype(np.float32))
+    knet.libknet8().check()
+
+
+def test_sum_gradient_through_the_tape(knet):
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    p = knet.Param(knet.KnetArray(x))
+    J = knet.diff(lambda: knet.sum(p))
+    assert float(knet.value(J)) == x.sum()
+    assert np.array_equal(knet.Array(knet.grad(J, p)), np.ones((3, 4), np.float32))

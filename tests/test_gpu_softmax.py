@@ -1,0 +1,148 @@
+"""GPU parity of the softmax / logsoftmax / nll family against the oracle.  Tolerance (north star): 1e-5 relative;
+written here as max|gpu - oracle| <= 1e-5 * max|oracle| per matrix plus the invariants the reference's own tests
+assert (test/loss.jl:47-56).  Index work (labels, skipped columns, gathers) is exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MS = [1, 2, 3, 63, 64, 65, 250, 256, 257, 1000, 1001, 1024, 4096, 4100, 9999, 16384, 16388, 32000, 32769, 65536, 70001]
+
+
+def close(got, want, rtol=1e-5):
+    scale = max(float(np.abs(want).max()), 1e-30)
+    return float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max()) <= rtol * scale
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_forward_and_backward_over_column_lengths(knet, oracle, dt):
+    rng = np.random.default_rng(31)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    for m in MS:
+        n = 5 if m > 4096 else 37
+        x = (rng.standard_normal((m, n)) * 2).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        xd, dyd = knet.KnetArray(x), knet.KnetArray(dy)
+        lsm = knet.Array(knet.logsoftmax(xd, dims=1))
+        want = oracle.logsoftmax(x, dims=1)
+        assert np.abs(lsm - want).max() <= rtol * np.abs(want).max(), m
+        sm = knet.Array(knet.softmax(xd, dims=1))
+        assert close(sm, oracle.softmax(x, dims=1), rtol), m
+        assert np.allclose(sm.sum(axis=0), 1, atol=100 * rtol)
+        assert np.allclose(sm, np.exp(lsm), rtol=100 * rtol, atol=rtol)
+        got = knet.Array(knet.logsoftmaxback(knet.KnetArray(want), dyd, dims=1))
+        assert close(got, oracle.logsoftmaxback(want, dy, dims=1), rtol), m
+        y = oracle.softmax(x, dims=1)
+        got = knet.Array(knet.softmaxback(knet.KnetArray(y), dyd, dims=1))
+        assert close(got, oracle.softmaxback(y, dy, dims=1), rtol), m
+    knet.libknet8().check()
+
+
+def test_other_dims_and_misaligned_columns(knet, oracle):
+    rng = np.random.default_rng(32)
+    x = (rng.standard_normal((10, 100)) * 2).astype(np.float32)
+    xd = knet.KnetArray(x)
+    for dims in (None, 1, 2, [1, 2]):
+        got = knet.Array(knet.logsoftmax(xd, dims=dims))
+        want = oracle.logsoftmax(x, dims=dims if dims is not None else (1, 2))
+        assert close(got, want), dims
+        got = knet.Array(knet.softmax(xd, dims=dims))
+        assert close(got, oracle.softmax(x, dims=dims if dims is not None else (1, 2))), dims
+    x3 = (rng.standard_normal((3, 4, 5)) * 2).astype(np.float32)
+    got = knet.Array(knet.logsoftmax(knet.KnetArray(x3), dims=[1, 2]))
+    assert close(got, oracle.logsoftmax(x3, dims=(1, 2)))
+    v = (rng.standard_normal(777) * 3).astype(np.float32)
+    assert close(knet.Array(knet.logsoftmax(knet.KnetArray(v), dims=1)), oracle.logsoftmax(v, dims=1))
+    # columns that are not 16-byte aligned (m odd) and a base pointer inside an allocation
+    from gpu_util import misaligned
+    for m, n in [(999, 40), (1000, 40), (33, 7)]:
+        x = (rng.standard_normal((m, n)) * 2).astype(np.float32)
+        xd = misaligned(knet, x, 1).reshape(m, n)
+        assert close(knet.Array(knet.logsoftmax(xd, dims=1)), oracle.logsoftmax(x, dims=1))
+    # large magnitudes stay finite, shift invariance (test/loss.jl)
+    big = np.float32([[1000.0, 0.0], [999.0, -1000.0]])
+    assert np.all(np.isfinite(knet.Array(knet.logsoftmax(knet.KnetArray(big), dims=1))))
+    a = knet.Array(knet.logsoftmax(knet.KnetArray(x + np.float32(5)), dims=1))
+    assert np.allclose(a, oracle.logsoftmax(x, dims=1), atol=2e-5)
+    # logsumexp
+    got = knet.Array(knet.logsumexp(knet.KnetArray(x), dims=1))
+    assert np.allclose(got, oracle.logsumexp(x, dims=1), rtol=1e-5, atol=1e-5)
+
+
+def test_gather_scatter_bit_exact(knet, oracle):
+    rng = np.random.default_rng(33)
+    for dt in (np.float32, np.float64):
+        x = rng.standard_normal((50, 70)).astype(dt)
+        ents = rng.permutation(3500)[:333] + 1
+        xd = knet.KnetArray(x)
+        got = knet.Array(knet.getindex(xd, ents))
+        assert np.array_equal(got, oracle.getents(x, ents))
+        y = rng.standard_normal(333).astype(dt)
+        got = knet.Array(knet.ungetindex(xd, knet.KnetArray(y), ents))
+        assert np.array_equal(got, oracle.addents(np.zeros_like(x), ents, y))
+    with pytest.raises(IndexError):
+        knet.getindex(xd, [0])
+    with pytest.raises(IndexError):
+        knet.getindex(xd, [3501])
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("C,N", [(10, 100), (3, 2), (1000, 257), (4100, 9), (32000, 6), (70001, 2)])
+def test_nll_value_and_gradient_both_paths(knet, oracle, dt, C, N):
+    rng = np.random.default_rng(34)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    scores = (rng.standard_normal((C, N)) * 2).astype(dt)
+    labels = rng.integers(1, C + 1, size=N)
+    if N > 3:
+        labels[1] = 0  # skipped instance (src/ops20/loss.jl:125)
+    want_loss = oracle.nll(scores, labels)
+    want_grad = oracle.nll_back(scores, labels)
+    for fused in (False, True):
+        p = knet.Param(knet.KnetArray(scores))
+        J = knet.diff(lambda: knet.nll(p, labels, fused=fused))
+        assert abs(float(knet.value(J)) - float(want_loss)) <= rtol * abs(float(want_loss)), fused
+        g = knet.Array(knet.grad(J, p))
+        assert close(g, want_grad, rtol), fused
+        if N > 3:
+            assert np.all(g[:, 1] == 0)  # skipped column: exactly zero
+        assert np.abs(g.sum(axis=0)).max() <= 1e-4 * rtol / 1e-5 / N
+    # value without recording
+    assert abs(float(knet.nll(knet.KnetArray(scores), labels)) - float(want_loss)) <= rtol * abs(float(want_loss))
+    knet.libknet8().check()
+
+
+def test_nll_known_answer_and_dims2(knet, oracle):
+    # docstring example of src/ops20/loss.jl:22-27 (see the oracle test for the 2.6 % discrepancy of the printed figure)
+    scores = np.array([[12.2, 0.3], [2.0, 21.5], [0.0, -21.0]])
+    v = float(knet.nll(knet.KnetArray(scores), [1, 2]))
+    assert abs(v - 2.1100252335646503e-05) < 1e-15 and abs(v - 2.1657e-5) < 0.03 * 2.1657e-5
+    v2 = float(knet.nll(knet.KnetArray(scores.T.copy()), [1, 2], dims=2))
+    assert abs(v2 - v) < 1e-15
+    p = knet.Param(knet.KnetArray(scores.T.copy()))
+    J = knet.diff(lambda: knet.nll(p, [1, 2], dims=2))
+    assert np.allclose(knet.Array(knet.grad(J, p)), oracle.nll_back(scores.T.copy(), [1, 2], dims=2), atol=1e-15)
+    tot, cnt = knet.nll(knet.KnetArray(scores), [1, 0], average=False)
+    assert cnt == 1
+    assert knet.accuracy(knet.KnetArray(scores), [1, 2]) == 1.0 and knet.accuracy(knet.KnetArray(scores), [2, 2]) == 0.5
+    with pytest.raises(ValueError):
+        knet.nll(knet.KnetArray(scores), [1, 2, 3])
+
+
+def test_config4_full_size(knet, oracle):
+    """BASELINE config 4: logits (32000,512) ~ N(0,2), labels uniform, upstream 1/512; and (1000,4096)."""
+    rng = np.random.default_rng(35)
+    for C, N in [(32000, 512), (1000, 4096)]:
+        scores = (rng.standard_normal((C, N), dtype=np.float32) * 2)
+        labels = rng.integers(1, C + 1, size=N)
+        want_loss = oracle.nll(scores, labels)
+        want_grad = oracle.nll_back(scores, labels)
+        for fused in (False, True):
+            p = knet.Param(knet.KnetArray(scores))
+            J = knet.diff(lambda: knet.nll(p, labels, fused=fused))
+            assert abs(float(knet.value(J)) - float(want_loss)) <= 1e-5 * abs(float(want_loss))
+            assert close(knet.Array(knet.grad(J, p)), want_grad)
+        lsm = oracle.logsoftmax(scores, dims=1)
+        dy = rng.standard_normal((C, N), dtype=np.float32)
+        got = knet.Array(knet.logsoftmaxback(knet.KnetArray(lsm), knet.KnetArray(dy), dims=1))
+        assert close(got, oracle.logsoftmaxback(lsm, dy, dims=1))
+    knet.libknet8().check()
