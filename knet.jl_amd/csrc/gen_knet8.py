@@ -55,6 +55,7 @@ UNARY_OPS = [
     ("sign", "return xi > T(0) ? T(1) : xi < T(0) ? T(-1) : T(0);", "src/libknet8/ops.jl:55"),
     ("invx", "return T(1) / xi;", "src/libknet8/ops.jl:71"),
     ("one", "return T(1);", "src/libknet8/ops.jl:52"),
+    ("copy", "return xi;", "the contiguous case of xcopy, src/libknet8/cuda1.jl:130-165 (also the known-size 1R+1W kernel used to calibrate HBM counters)"),
     ("zero", "return T(0);", "src/libknet8/ops.jl:67"),
 ]
 
@@ -345,6 +346,11 @@ KNET8_API int knet8_synchronize(hipStream_t stream);
 /* elapsed device time between two marks on a stream, in milliseconds (HIP events) */
 KNET8_API void knet8_timer_start(hipStream_t stream);
 KNET8_API float knet8_timer_stop(hipStream_t stream);
+/* HIP events for timing individual launches on the stream they are issued to; elapsed is in milliseconds and waits for `stop` */
+KNET8_API void* knet8_event_create(void);
+KNET8_API void knet8_event_destroy(void* event);
+KNET8_API void knet8_event_record(void* event, hipStream_t stream);
+KNET8_API float knet8_event_elapsed(void* start, void* stop);
 /* last recorded failure as text (NULL if none); reading clears it */
 KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);

@@ -64,20 +64,33 @@ __device__ __forceinline__ T block_reduce(T v, T* lds, Merge merge, T identity) 
 }
 
 // Device-scope "last workgroup of a group finishes the job" ticket.  Workgroups that contribute to the
-// same output group publish their partials, fence, and take a ticket; the one that draws the last
-// ticket (returns true) may read all partials (after the fence inside) and must reset the counter so
-// the next launch on the same stream finds it zero.
+// same output group store their partials with st_coherent() and call this; the one that draws the last
+// ticket (returns true) may then read all partials and must reset the counter so the next launch on the
+// same stream finds it zero.
+//
+// The L2s of the eight XCDs are not coherent with each other, so the textbook form of this pattern (plain
+// stores, then an agent-scope release fence per workgroup) makes every workgroup write its whole L2 back
+// (buffer_wbl2); measured, a few thousand such fences cost 100+ us, several times the reduction itself.
+// Instead the partials are written through to the device-coherent level as they are stored (agent-scope
+// relaxed atomic stores: global_store ... sc1), each lane waits for its own stores to be acknowledged
+// (s_waitcnt vmcnt(0)), the barrier collects the lanes, and only then does lane 0 take the ticket with an
+// agent-scope atomic.  Whoever sees the last ticket therefore finds every partial at the coherent level;
+// it drops stale lines with one acquire fence (buffer_inv sc1) before the workgroup reads them.
+template <typename T> __device__ __forceinline__ void st_coherent(T* p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ bool last_block_ticket(unsigned* counter, unsigned nparts, unsigned* lds_flag) {
-  __threadfence();  // publish this workgroup's partials at agent scope
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   if (threadIdx.x == 0) {
-    unsigned t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    *lds_flag = (t == nparts - 1) ? 1u : 0u;
+    const unsigned t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = (t == nparts - 1);
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    *lds_flag = last ? 1u : 0u;
   }
   __syncthreads();
-  bool last = (*lds_flag != 0);
-  if (last) __threadfence();  // acquire: see every other workgroup's partials
-  return last;
+  return *lds_flag != 0;
 }
 
 template <typename T> __device__ __forceinline__ T ld_coherent(const T* p) {

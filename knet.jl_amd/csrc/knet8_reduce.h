@@ -95,14 +95,14 @@ __global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restri
     if (threadIdx.x == 0) y[j] = r;
     return;
   }
-  if (threadIdx.x == 0) partial[j * P + p] = r;
+  if (threadIdx.x == 0) st_coherent(partial + j * P + p, r);
   if (!last_block_ticket(counters + j, P, &flag)) return;
   T s = Op::init();
   for (unsigned q = threadIdx.x; q < P; q += kRedBlock) s = Op::merge(s, ld_coherent(partial + j * P + q));
   s = block_reduce<T, kRedWaves>(s, lds, MergeFn<Op, T>(), Op::init());
   if (threadIdx.x == 0) {
     y[j] = s;
-    counters[j] = 0;
+    st_coherent(counters + j, 0u);
   }
 }
 
@@ -169,13 +169,13 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __re
       T r = Op::init();
 #pragma unroll
       for (int w = 0; w < kRedWaves; w++) r = Op::merge(r, lds[w][threadIdx.x]);
-      partial[(group * P + p) * TILE + threadIdx.x] = r;
+      st_coherent(partial + (group * P + p) * TILE + threadIdx.x, r);
     }
     if (!last_block_ticket(counters + group, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
     strided_walk<T, Op, NV, false>(partial + group * P * TILE + lane * NV, TILE, 0, P, wave, acc);
-    if (threadIdx.x == 0) counters[group] = 0;
+    if (threadIdx.x == 0) st_coherent(counters + group, 0u);
   }
 #pragma unroll
   for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
@@ -231,14 +231,14 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_small_kernel(const T
     if (owner) y[b * s1 + threadIdx.x] = r;
     return;
   }
-  if (owner) partial[(b * P + p) * s1 + threadIdx.x] = r;
+  if (owner) st_coherent(partial + (b * P + p) * s1 + threadIdx.x, r);
   if (!last_block_ticket(counters + b, P, &flag)) return;
   if (owner) {
     T s = Op::init();
     for (unsigned q = 0; q < P; q++) s = Op::merge(s, ld_coherent(partial + (b * P + q) * s1 + threadIdx.x));
     y[b * s1 + threadIdx.x] = s;
   }
-  if (threadIdx.x == 0) counters[b] = 0;
+  if (threadIdx.x == 0) st_coherent(counters + b, 0u);
 }
 
 // ---- host-side planning ----------------------------------------------------------------------------

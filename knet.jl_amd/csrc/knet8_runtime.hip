@@ -264,6 +264,25 @@ KNET8_API float knet8_timer_stop(hipStream_t stream) {
   return ms;
 }
 
+KNET8_API void* knet8_event_create(void) {
+  hipEvent_t e = nullptr;
+  ok(hipEventCreate(&e), "hipEventCreate");
+  return e;
+}
+
+KNET8_API void knet8_event_destroy(void* event) {
+  if (event) ok(hipEventDestroy(static_cast<hipEvent_t>(event)), "hipEventDestroy");
+}
+
+KNET8_API void knet8_event_record(void* event, hipStream_t stream) { ok(hipEventRecord(static_cast<hipEvent_t>(event), stream), "hipEventRecord"); }
+
+KNET8_API float knet8_event_elapsed(void* start, void* stop) {
+  float ms = -1.f;
+  if (ok(hipEventSynchronize(static_cast<hipEvent_t>(stop)), "hipEventSynchronize"))
+    ok(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)), "hipEventElapsedTime");
+  return ms;
+}
+
 KNET8_API const char* knet8_last_error(void) {
   std::lock_guard<std::mutex> lock(g_err_mutex);
   if (g_err.empty()) return nullptr;
