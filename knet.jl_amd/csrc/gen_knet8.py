@@ -354,7 +354,7 @@ KNET8_API float knet8_event_elapsed(void* start, void* stop);
 /* last recorded failure as text (NULL if none); reading clears it */
 KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
-/* launch-heuristic knobs (0: bytes per reduction workgroup, 1/2: min/max workgroups per reduction launch) */
+/* launch-heuristic knobs (0: number of compute units the reduction planner aims at; default: asked from the device); returns the old value */
 KNET8_API int knet8_tune(int key, int value);
 /* replaces cublasSgemm_v2 / cublasDgemm_v2 at src/knetarrays/linalg.jl:26-52 (column-major, transa/transb in 'N','T'): hipBLASLt */
 KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc, hipStream_t stream);

@@ -43,10 +43,11 @@ template <typename Op, typename T> struct MergeFn {
 // NV = elements per lane per load (Vec16<T>::N on the aligned path, 1 otherwise); on the vector path
 // sy % NV == 0 so a vector never straddles two runs.  Workgroup (j,p) covers units [p*chunk, (p+1)*chunk)
 // of the K/NV units of output j.
-template <typename T, typename Op, int NV, bool SINGLE>
-__global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restrict__ x, long sy, long ny, long units, long chunk,
+template <typename T, typename Op, int NV, bool SINGLE, int BT, int U>
+__global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x, long sy, long ny, long units, long chunk,
                                                                unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
-  __shared__ T lds[kRedWaves];
+  constexpr int NW = BT / kWave;
+  __shared__ T lds[NW];
   __shared__ unsigned flag;
   const long j = blockIdx.x / P;
   const unsigned p = blockIdx.x % P;
@@ -59,16 +60,15 @@ __global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restri
   T acc[NV];
 #pragma unroll
   for (int e = 0; e < NV; e++) acc[e] = Op::init();
-  constexpr int U = 4;
-  for (long u = u0 + threadIdx.x; u < u1; u += kRedBlock * U) {
+  for (long u = u0 + threadIdx.x; u < u1; u += BT * U) {
     T v[U][NV];
 #pragma unroll
     for (int q = 0; q < U; q++) {
-      const long uu = u + q * kRedBlock;
+      const long uu = u + q * BT;
       if (uu < u1) {
         long off;
         if (SINGLE) off = uu * NV;
-        else { const long o = uu / usy; off = o * slab + (uu - o * usy) * NV; }
+        else { const unsigned o = (unsigned)uu / (unsigned)usy; off = o * slab + ((unsigned)uu - o * (unsigned)usy) * NV; }
         if (NV > 1) {
           typedef typename Vec16<T>::type V;
           V t = ld_stream(reinterpret_cast<const V*>(xj + off));
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restri
   T r = acc[0];
 #pragma unroll
   for (int e = 1; e < NV; e++) r = Op::merge(r, acc[e]);
-  r = block_reduce<T, kRedWaves>(r, lds, MergeFn<Op, T>(), Op::init());
+  r = block_reduce<T, NW>(r, lds, MergeFn<Op, T>(), Op::init());
   if (P == 1) {
     if (threadIdx.x == 0) y[j] = r;
     return;
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restri
   if (threadIdx.x == 0) st_coherent(partial + j * P + p, r);
   if (!last_block_ticket(counters + j, P, &flag)) return;
   T s = Op::init();
-  for (unsigned q = threadIdx.x; q < P; q += kRedBlock) s = Op::merge(s, ld_coherent(partial + j * P + q));
-  s = block_reduce<T, kRedWaves>(s, lds, MergeFn<Op, T>(), Op::init());
+  for (unsigned q = threadIdx.x; q < P; q += BT) s = Op::merge(s, ld_coherent(partial + j * P + q));
+  s = block_reduce<T, NW>(s, lds, MergeFn<Op, T>(), Op::init());
   if (threadIdx.x == 0) {
     y[j] = s;
     st_coherent(counters + j, 0u);
@@ -111,14 +111,13 @@ __global__ __launch_bounds__(kRedBlock) void reduce_run_kernel(const T* __restri
 // lane; the four waves of a workgroup take k = k0+wave, k0+wave+4, ...; P workgroups split the k range.
 // The same walk (rows `stride` apart, this wave's share of [k0,k1)) combines the P partial tiles at the end
 // (ITEM=false: partials are merged as they are, the item map was applied when they were made).
-template <typename T, typename Op, int NV, bool ITEM>
+template <typename T, typename Op, int NV, bool ITEM, int NW, int U>
 __device__ __forceinline__ void strided_walk(const T* base, long stride, long k0, long k1, int wave, T (&acc)[NV]) {
-  constexpr int U = 8;
-  for (long k = k0 + wave; k < k1; k += kRedWaves * U) {
+  for (long k = k0 + wave; k < k1; k += NW * U) {
     T v[U][NV];
 #pragma unroll
     for (int q = 0; q < U; q++) {
-      const long kk = k + q * kRedWaves;
+      const long kk = k + q * NW;
       if (kk < k1) {
         if (NV > 1) {
           typedef typename Vec16<T>::type V;
@@ -141,11 +140,12 @@ __device__ __forceinline__ void strided_walk(const T* base, long stride, long k0
   }
 }
 
-template <typename T, typename Op, int NV>
-__global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
+template <typename T, typename Op, int NV, int BT, int U>
+__global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
                                                                    unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
   constexpr int TILE = kWave * NV;
-  __shared__ T lds[kRedWaves][TILE];
+  constexpr int NW = BT / kWave;
+  __shared__ T lds[NW][TILE];
   __shared__ unsigned flag;
   const long group = blockIdx.x / P;   // (b, atile)
   const unsigned p = blockIdx.x % P;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __re
   T acc[NV];
 #pragma unroll
   for (int e = 0; e < NV; e++) acc[e] = Op::init();
-  if (live) strided_walk<T, Op, NV, true>(x + b * s1 * d + a0, s1, k0, k1, wave, acc);
+  if (live) strided_walk<T, Op, NV, true, NW, U>(x + b * s1 * d + a0, s1, k0, k1, wave, acc);
   if (P > 1) {
     // partial tile p of this group = this workgroup's reduction over its k range
 #pragma unroll
@@ -168,13 +168,13 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __re
     if (threadIdx.x < TILE) {
       T r = Op::init();
 #pragma unroll
-      for (int w = 0; w < kRedWaves; w++) r = Op::merge(r, lds[w][threadIdx.x]);
+      for (int w = 0; w < NW; w++) r = Op::merge(r, lds[w][threadIdx.x]);
       st_coherent(partial + (group * P + p) * TILE + threadIdx.x, r);
     }
     if (!last_block_ticket(counters + group, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
-    strided_walk<T, Op, NV, false>(partial + group * P * TILE + lane * NV, TILE, 0, P, wave, acc);
+    strided_walk<T, Op, NV, false, NW, U>(partial + group * P * TILE + lane * NV, TILE, 0, P, wave, acc);
     if (threadIdx.x == 0) st_coherent(counters + group, 0u);
   }
 #pragma unroll
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_kernel(const T* __re
   if (threadIdx.x < TILE && a < s1) {
     T r = Op::init();
 #pragma unroll
-    for (int w = 0; w < kRedWaves; w++) r = Op::merge(r, lds[w][threadIdx.x]);
+    for (int w = 0; w < NW; w++) r = Op::merge(r, lds[w][threadIdx.x]);
     y[b * s1 + a] = r;
   }
 }
@@ -242,20 +242,17 @@ __global__ __launch_bounds__(kRedBlock) void reduce_strided_small_kernel(const T
 }
 
 // ---- host-side planning ----------------------------------------------------------------------------
-
+// Measured on MI355X (256 CUs): these HBM-bound reductions run fastest when a launch has about one
+// large workgroup per CU and no second stage; every extra split costs 2-4 us of ticket traffic and every
+// extra round of workgroups a partial tail.  So: no split while the outputs alone give at least half a
+// workgroup per CU; otherwise split until there is about one workgroup per CU, as long as each part keeps
+// enough loads per lane to cover the memory latency.
 inline long ceil_div(long a, long b) { return (a + b - 1) / b; }
 
-// Number of workgroups per output group: about `wg_bytes` of input each, but at least enough to give the
-// launch `min_wgs` workgroups and at most enough to reach `max_wgs`; never so many that a workgroup has
-// less than `min_units_per_wg` loads to issue.
-inline unsigned plan_parts(long groups, long units_per_group, long unit_bytes, long min_units_per_wg) {
-  const long wg_bytes = tuning(kTuneRedWgBytes), min_wgs = tuning(kTuneRedMinWgs), max_wgs = tuning(kTuneRedMaxWgs);
-  long P = ceil_div(units_per_group * unit_bytes, wg_bytes);
-  const long fill = ceil_div(min_wgs, groups);
-  long most = max_wgs / groups;
-  if (most < fill) most = fill;
-  if (P > most) P = most;
-  if (P < fill) P = fill;
+inline unsigned plan_parts(long groups, long units_per_group, long min_units_per_wg) {
+  const long ncu = tuning(kTuneNumCUs);
+  long P = 1;
+  if (groups * 2 <= ncu) P = ceil_div(ncu, groups);
   const long cap = units_per_group / min_units_per_wg;
   if (P > cap) P = cap;
   if (P > 65535) P = 65535;
@@ -270,18 +267,23 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;
   const long units = sy / nv * no;
-  unsigned P = plan_parts(ny, units, (long)nv * sizeof(T), kRedBlock);
+  unsigned P = plan_parts(ny, units, 2048);
   long chunk = ceil_div(units, P);
   P = (unsigned)ceil_div(units, chunk > 0 ? chunk : 1);
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)ny * P, (size_t)ny);
-  const dim3 grid((unsigned)(ny * P)), block(kRedBlock);
   T* partial = static_cast<T*>(ws.partial);
-#define KNET8_RUN(NV, SINGLE) \
-  hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE>), grid, block, 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters)
-  if (vec) { if (no == 1) KNET8_RUN(N, true); else KNET8_RUN(N, false); }
-  else     { if (no == 1) KNET8_RUN(1, true); else KNET8_RUN(1, false); }
+  // workgroup size by the work of one part: a wave for short runs, 512 lanes when there is plenty
+  const int bt = chunk <= 2 * kWave ? 64 : chunk <= 4096 ? 256 : 512;
+  const dim3 grid((unsigned)(ny * P));
+#define KNET8_RUN(NV, SINGLE, BT, U) \
+  hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE, BT, U>), grid, dim3(BT), 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters)
+#define KNET8_RUN_BT(NV, SINGLE) \
+  do { if (bt == 64) KNET8_RUN(NV, SINGLE, 64, 8); else if (bt == 256) KNET8_RUN(NV, SINGLE, 256, 4); else KNET8_RUN(NV, SINGLE, 512, 4); } while (0)
+  if (vec) { if (no == 1) KNET8_RUN_BT(N, true); else KNET8_RUN_BT(N, false); }
+  else     { if (no == 1) KNET8_RUN_BT(1, true); else KNET8_RUN_BT(1, false); }
+#undef KNET8_RUN_BT
 #undef KNET8_RUN
 }
 
@@ -292,7 +294,7 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   if (s1 < kWave) {
     const int reps = kRedBlock / (int)s1, L = reps * (int)s1;
     const long total = s1 * d;
-    unsigned P = plan_parts(nb, ceil_div(total, L), (long)L * sizeof(T), 1);
+    unsigned P = plan_parts(nb, ceil_div(total, L), 16);
     long chunk = ceil_div(ceil_div(total, L), P) * L;
     P = (unsigned)ceil_div(total, chunk > 0 ? chunk : 1);
     if (P < 1) P = 1;
@@ -307,18 +309,20 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   const long tile = (long)kWave * nv;
   const long atiles = ceil_div(s1, tile);
   const long groups = atiles * nb;
-  unsigned P = plan_parts(groups, d, tile * sizeof(T), kRedWaves * 8);
+  unsigned P = plan_parts(groups, d, 64);
   long kchunk = ceil_div(d, P);
   P = (unsigned)ceil_div(d, kchunk > 0 ? kchunk : 1);
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups);
-  const dim3 grid((unsigned)(groups * P)), block(kRedBlock);
+  const dim3 grid((unsigned)(groups * P));
   T* partial = static_cast<T*>(ws.partial);
-  if (vec)
-    hipLaunchKernelGGL((reduce_strided_kernel<T, Op, N>), grid, block, 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters);
-  else
-    hipLaunchKernelGGL((reduce_strided_kernel<T, Op, 1>), grid, block, 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters);
+  const bool big = kchunk >= 128;  // sixteen waves share a tile when each still gets >= 8 rows
+#define KNET8_STR(NV, BT, U) \
+  hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters)
+  if (vec) { if (big) KNET8_STR(N, 1024, 2); else KNET8_STR(N, 256, 8); }
+  else     { if (big) KNET8_STR(1, 1024, 2); else KNET8_STR(1, 256, 8); }
+#undef KNET8_STR
 }
 
 // `_21` contract: x[i] goes into y[(i/sy)%ny]  (src/libknet8/cuda21.jl:23).

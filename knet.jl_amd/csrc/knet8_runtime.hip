@@ -41,12 +41,20 @@ static bool ok(hipError_t e, const char* what) {
 }
 
 // ---- launch-heuristic knobs ------------------------------------------------------------------------------
-static int g_tune[kTuneCount] = {
-    64 * 1024,  // kTuneRedWgBytes: input bytes one reduction workgroup should move
-    2048,       // kTuneRedMinWgs:  split until a reduction launch has at least this many workgroups
-    16384,      // kTuneRedMaxWgs:  ... and never split beyond this many
-    0, 0, 0, 0, 0};
-int tuning(int key) { return (key >= 0 && key < kTuneCount) ? g_tune[key] : 0; }
+static int g_tune[kTuneCount] = {0, 0, 0, 0, 0, 0, 0, 0};
+int tuning(int key) {
+  if (key < 0 || key >= kTuneCount) return 0;
+  if (key == kTuneNumCUs && g_tune[key] == 0) {  // compute units of the current device, asked once
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_tune[key] = n;
+    else {
+      (void)hipGetLastError();
+      g_tune[key] = 256;
+    }
+  }
+  return g_tune[key];
+}
 
 // ---- per-stream scratch for split reductions ------------------------------------------------------------
 struct StreamScratch {

@@ -17,8 +17,14 @@
 
 namespace knet8 {
 
+// exp for the softmax family.  fp32 uses the hardware 2^x unit (v_exp_f32, 1 ulp) on a pre-scaled argument: the
+// only extra error is the rounding of x*log2(e), about |x| * 6e-8 relative -- two orders of magnitude inside the
+// 1e-5 contract of these kernels -- and it costs 2 instructions instead of the ~20 of the correctly rounded expf.
+// With a 32000-row column resident per workgroup the exp work is not hidden behind memory traffic (only two columns
+// fit in a CU's registers, so load, compute and store phases run in lock-step), so this is measurable wall time.
+// The elementwise activation kernels, whose contract is 2 ulp, keep the precise expf.
 template <typename T> __device__ __forceinline__ T dev_exp(T x);
-template <> __device__ __forceinline__ float dev_exp<float>(float x) { return expf(x); }
+template <> __device__ __forceinline__ float dev_exp<float>(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 template <> __device__ __forceinline__ double dev_exp<double>(double x) { return exp(x); }
 template <typename T> __device__ __forceinline__ T dev_log(T x);
 template <> __device__ __forceinline__ float dev_log<float>(float x) { return logf(x); }
@@ -182,6 +188,109 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel
   if (Algo::kNll && colok && lab == 0 && tl == 0) loss[col] = T(0);
 }
 
+// ---- fused nll + logsoftmax backward, register-resident, single reduction ---------------------------------
+// The generic kernel above needs two workgroup-wide reductions (max, then sum of exp) and two exp per element.
+// Here each lane first reduces its own elements (local max m_t, e_i = exp(a_i - m_t) kept in the registers that
+// held a_i, s_t = sum e_i); the (max, sum) pairs are merged in ONE reduction with
+// (m1,s1)+(m2,s2) = (M, s1*exp(m1-M) + s2*exp(m2-M)), M = max(m1,m2); then softmax_i = e_i * exp(m_t-M)/S is a
+// single multiply per element.  One exp per element, one barrier phase less: the long serial tail of the
+// 32000-row columns shrinks, which matters because only two such columns fit in the registers of a CU at a time.
+// Rounding differs from the step-by-step formula by a few 1e-7 relative, inside the 1e-5 contract.
+template <typename T> struct MaxSum { T m, s; };
+template <typename T> __device__ __forceinline__ MaxSum<T> ms_merge(MaxSum<T> a, MaxSum<T> b) {
+  const T M = a.m > b.m ? a.m : b.m;
+  const T sa = a.m == M ? a.s : a.s * dev_exp(a.m - M);
+  const T sb = b.m == M ? b.s : b.s * dev_exp(b.m - M);
+  MaxSum<T> r = {M, sa + sb};
+  return r;
+}
+template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum<T> v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    MaxSum<T> o = {__shfl_xor(v.m, off, kWave), __shfl_xor(v.s, off, kWave)};
+    v = ms_merge(v, o);
+  }
+  return v;
+}
+
+template <typename T, int TEAM, int E, bool VEC>
+__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
+                                                                            T scale, T* loss) {
+  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int TEAMS = BT / TEAM;
+  constexpr int NW = TEAM / kWave;
+  constexpr int NV = VEC ? Vec16<T>::N : 1;
+  constexpr int ITEMS = E / NV;
+  typedef typename Vec16<T>::type V;
+  __shared__ T lds_m[BT / kWave], lds_s[BT / kWave];
+  const int tl = threadIdx.x % TEAM;
+  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
+  const bool colok = col < n;
+  const long base = colok ? col * (long)m : 0;
+  const T* ac = a + base;
+  T* oc = out + base;
+  const int lab = colok ? labels[col] : 0;
+
+  T ra[E];
+  T alab = T(0);
+  bool own = false;
+  T mt = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    const int r = (tl + i * TEAM) * NV;
+    const bool ok = colok && r < m;
+    V va = {};
+    if (ok) {
+      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+      else va[0] = __builtin_nontemporal_load(ac + r);
+    }
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      const T v = ok ? va[e] : T(-INFINITY);
+      ra[i * NV + e] = v;
+      mt = mt > v ? mt : v;
+      if (ok && r + e + 1 == lab) { alab = v; own = true; }
+    }
+  }
+  T st = T(0);
+  const T mref = mt == T(-INFINITY) ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
+#pragma unroll
+  for (int i = 0; i < E; i++) {
+    const T e = dev_exp(ra[i] - mref);
+    ra[i] = e;
+    st = st + e;
+  }
+  MaxSum<T> ms = {mt, st};
+  ms = ms_wave_reduce(ms);
+  if (NW > 1) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) { lds_m[wave] = ms.m; lds_s[wave] = ms.s; }
+    __syncthreads();
+    MaxSum<T> t = {lane < NW ? lds_m[lane] : T(-INFINITY), lane < NW ? lds_s[lane] : T(0)};
+    ms = ms_wave_reduce(t);
+  }
+  const T logS = dev_log(ms.s);
+  // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
+  const T f = (mt == T(-INFINITY) ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
+  if (own) loss[col] = -((alab - ms.m) - logS);
+  if (colok && lab == 0 && tl == 0) loss[col] = T(0);
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    const int r = (tl + i * TEAM) * NV;
+    const bool ok = colok && r < m;
+    if (!ok) continue;
+    V vo;
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      const T p = ra[i * NV + e] * f;
+      const T dlp = (r + e + 1 == lab) ? -scale : T(0);
+      vo[e] = lab == 0 ? T(0) : dlp + p;
+    }
+    if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+    else __builtin_nontemporal_store(vo[0], oc + r);
+  }
+}
+
 // ---- streaming fallback for very long columns ----------------------------------------------------------
 // One 1024-thread workgroup per column; the inputs are read once per pass (max, sum, output).
 template <typename T, typename Algo>
@@ -224,10 +333,15 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
   constexpr int BT = TEAM == kWave ? 256 : TEAM;
   constexpr int TEAMS = BT / TEAM;
   const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS)), block(BT);
-  if (vec)
-    hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
-  else
-    hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+  if constexpr (Algo::kNll) {
+    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+    else
+      hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+  }
 }
 
 template <typename T, typename Algo>

@@ -309,14 +309,18 @@ def gemm(A, B, ta=False, tb=False):
     return _shape_like(C, (m, n))
 
 
-def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None):
+def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None, gemm=None):
     """Reference MLP step: ``x = relu.(w*x .+ b)`` per hidden layer (+ dropout with the given
     uniform buffers), ``nll`` on the last layer's scores; returns (loss, [dW1, db1, dW2, ...]).
 
     Follows the model of examples/mnist-mlp/mlp.jl:25-35 and the gradient expressions the
     reference registers for each primitive (matmul: src/knetarrays/linalg.jl:11-18; bias:
     ``sum(dy;dims=2)``; relu: ``reluback.(dy,y)``; dropout: ``dropback``; nll: ``ko_nll_back``).
+
+    ``gemm(A, B, ta=False, tb=False)`` may replace the wide-accumulation C loop for the matrix products (e.g. a BLAS
+    sgemm for shapes the loop cannot finish in reasonable time); everything else always runs through the C restatement.
     """
+    gemm = gemm or globals()["gemm"]
     nl = len(weights) // 2
     acts = [np.asarray(x)]
     saved = []

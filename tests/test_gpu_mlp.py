@@ -1,0 +1,121 @@
+"""End-to-end backward step through KnetArray, the tape and the C ABI (BASELINE configs 1 and 5) against the oracle.
+
+Tolerances: the loss and the gradients go through GEMMs (hipBLASLt on the device, wide-accumulation loops or BLAS in
+the oracle), so they are compared norm-wise: ||g - g_ref|| <= 1e-4 ||g_ref|| in fp32 (accumulation order over k up to
+4096 differs), and 1e-5 relative for the loss.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def build(knet, ws):
+    return [knet.Param(knet.KnetArray(w)) for w in ws]
+
+
+def predict(knet, params, x, pdrop=0.0, uniforms=None):
+    # examples/mnist-mlp/mlp.jl:25-33
+    h = x
+    for i in range(0, len(params), 2):
+        h = knet.add(knet.matmul(params[i], knet.mat(h)), params[i + 1])
+        if i < len(params) - 2:
+            h = knet.relu(h)
+            if pdrop > 0:
+                h = knet.dropout(h, pdrop, uniform=uniforms[i // 2])
+    return h
+
+
+def rel(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_config1_mlp_784_64_10(knet, oracle, fused):
+    rng = np.random.default_rng(41)
+    ws = [(rng.standard_normal((64, 784)) * 0.01).astype(np.float32), np.zeros((64, 1), np.float32),
+          (rng.standard_normal((10, 64)) * 0.01).astype(np.float32), np.zeros((10, 1), np.float32)]
+    x = rng.random((784, 100), dtype=np.float32)
+    labels = rng.integers(1, 11, size=100)
+    loss_ref, grads_ref = oracle.mlp_backward(ws, x, labels)
+    params = build(knet, ws)
+    xd = knet.KnetArray(x)
+    J = knet.diff(lambda: knet.nll(predict(knet, params, xd), labels, fused=fused))
+    assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
+    for p, g in zip(params, grads_ref):
+        got = knet.Array(knet.grad(J, p))
+        assert got.shape == g.shape
+        assert rel(got, g) <= 1e-4
+    # a 4-d input batch goes through mat() like the MNIST images of the example (28,28,1,100)
+    x4 = knet.KnetArray(x.reshape(28, 28, 1, 100, order="F"))
+    J4 = knet.diff(lambda: knet.nll(predict(knet, params, x4), labels, fused=fused))
+    assert float(knet.value(J4)) == float(knet.value(J))
+    knet.libknet8().check()
+
+
+def test_small_deep_mlp_with_dropout_fp64_matches_oracle_tightly(knet, oracle):
+    rng = np.random.default_rng(42)
+    sizes = [33, 40, 24, 17, 9]
+    ws = []
+    for i in range(4):
+        ws += [rng.standard_normal((sizes[i + 1], sizes[i])) * 0.3, rng.standard_normal((sizes[i + 1], 1)) * 0.1]
+    x = rng.random((33, 50))
+    labels = rng.integers(0, 10, size=50)  # includes skipped instances (label 0)
+    uni = [rng.random((sizes[i + 1], 50)) for i in range(3)]
+    loss_ref, grads_ref = oracle.mlp_backward(ws, x, labels, pdrop=0.5, uniforms=uni)
+    params = build(knet, ws)
+    xd = knet.KnetArray(x)
+    for fused in (False, True):
+        J = knet.diff(lambda: knet.nll(predict(knet, params, xd, 0.5, uni), labels, fused=fused))
+        assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-12 * abs(float(loss_ref))
+        for p, g in zip(params, grads_ref):
+            assert rel(knet.Array(knet.grad(J, p)), g) <= 1e-11
+    # outside diff() dropout is the identity and nothing is recorded
+    out = predict(knet, params, xd, 0.5, uni)
+    assert isinstance(out, knet.KnetArray)
+
+
+def test_config5_deep_mlp_full_size(knet, oracle):
+    """8 layers of width 4096 (7 hidden 4096x4096 + output 1000x4096), batch 2048, relu + dropout 0.5 with explicit masks."""
+    rng = np.random.default_rng(43)
+    sizes = [4096] * 8 + [1000]
+    ws = []
+    for i in range(8):
+        ws += [(rng.standard_normal((sizes[i + 1], sizes[i]), dtype=np.float32) * np.float32(0.02)), np.zeros((sizes[i + 1], 1), np.float32)]
+    x = rng.random((4096, 2048), dtype=np.float32)
+    labels = rng.integers(1, 1001, size=2048)
+    uni = [rng.random((4096, 2048), dtype=np.float32) for _ in range(7)]
+
+    def blas_gemm(A, B, ta=False, tb=False):
+        A = A.T if ta else A
+        B = B.T if tb else B
+        return np.asfortranarray(A @ B)
+    loss_ref, grads_ref = oracle.mlp_backward(ws, x, labels, pdrop=0.5, uniforms=uni, gemm=blas_gemm)
+    params = build(knet, ws)
+    xd = knet.KnetArray(x)
+    unid = [knet.KnetArray(u) for u in uni]
+    J = knet.diff(lambda: knet.nll(predict(knet, params, xd, 0.5, unid), labels, fused=True))
+    assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
+    errs = [rel(knet.Array(knet.grad(J, p)), g) for p, g in zip(params, grads_ref)]
+    print("config5 relative gradient errors (dW1, db1, ..., dW8, db8):", ["%.1e" % e for e in errs])
+    # Two fp32 GEMM implementations differ in accumulation order (k = 4096), so of the 8.4 M pre-activations of a
+    # hidden layer the handful that lie within rounding of zero land on different sides of relu's step.  Each such
+    # flip is a 100 % error on one element of the upstream gradient: sqrt(flips / 8.4e6) ~ 1e-3 norm-wise, which is
+    # what layers 1-7 show.  The output layer has no relu between it and the loss and must agree to 1e-4
+    # (measured: 2e-6), which is the check that the GEMM, bias-gradient and fused nll kernels themselves are right.
+    assert max(errs[-2:]) <= 1e-4, errs
+    assert max(errs) <= 5e-3, errs
+    knet.libknet8().check()
+
+
+def test_pool_reuses_device_memory(knet):
+    info = (4 * __import__("ctypes").c_size_t)()
+    fn = knet.libknet8().fn
+    a = knet.KnetArray(np.zeros(100000, np.float32))
+    pa = a.ptr
+    del a
+    fn["knet8_meminfo"](info)
+    hits = info[3]
+    b = knet.KnetArray(np.zeros(100000, np.float32))
+    fn["knet8_meminfo"](info)
+    assert b.ptr == pa and info[3] == hits + 1  # same block handed out again without a new hipMalloc
