@@ -280,6 +280,14 @@ def gen_softmax():
         o.entry("logsoftmaxback_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")],
                 "launch_softmax<%s, AlgoLogSoftmaxBack<%s>>(stream, m, n, y, dy, dx, nullptr, %s(0), nullptr)" % (T, T, T),
                 "unsafe_cudnnSoftmaxBackward(LOG) at src/ops20_gpu/softmax.jl:51-56")
+        o.decl.append("/* The same four operations along the middle axis of an (inner, d, outer) column-major view (inner > 1): softmax over a\n"
+                      "   non-leading dimension, which the reference builds from broadcast and reduction kernels (src/ops20_gpu/softmax.jl:22). */")
+        for nm, algo, two in (("softmax", "AlgoSoftmax", False), ("logsoftmax", "AlgoLogSoftmax", False),
+                              ("softmaxback", "AlgoSoftmaxBack", True), ("logsoftmaxback", "AlgoLogSoftmaxBack", True)):
+            params = [("int", "inner"), ("int", "d"), ("int", "outer")] + ([(T + "*", "y"), (T + "*", "dy"), (T + "*", "dx")] if two else [(T + "*", "x"), (T + "*", "y")])
+            call = ("launch_softmax_strided<%s, %s<%s>>(stream, inner, d, outer, y, dy, dx)" % (T, algo, T)) if two else \
+                   ("launch_softmax_strided<%s, %s<%s>>(stream, inner, d, outer, x, %s, y)" % (T, algo, T, z))
+            o.entry("%s_strided_%s" % (nm, S), "void", params, call, "the generic _softmax/_logsoftmax path of src/ops20/softmax.jl:42-63 for dims that are not leading")
         o.decl.append("/* Fused gradient of nll(scores, labels; dims=1) wrt scores: dx = scale*(softmax(x) - onehot(label)) per column and\n"
                       "   loss[col] = -logsoftmax(x)[label, col]; labels are 1-based int32, label 0 skips the column (dx = 0, loss = 0).\n"
                       "   One pass over the scores instead of logsoftmax + getents + fill + addents + logsoftmaxback. */")

@@ -122,9 +122,51 @@ __global__ __launch_bounds__(kEwBlock) void ew_bcast12_kernel(long n, const T* x
   }
 }
 
+// Fast path of the vector broadcast for the shapes the MLP path produces: one operand is the full array, the
+// other a vector along a single dimension, everything 16-byte aligned and the vector's stride or length a
+// multiple of the lanes of a 16-byte access.  XFULL says which operand is the full one (operand order matters
+// for sub/div).  s == 1: the vector runs along the contiguous dimension, so the four elements of an access
+// take four consecutive vector entries (one aligned 16-byte load of the vector, which stays in cache);
+// s > 1: all four elements of an access share one vector entry.
+template <typename T, typename F, bool XFULL>
+__global__ __launch_bounds__(kEwBlock) void ew_bias_vec_kernel(long nvec, const T* full, const T* vec, int s, int nv, T* z, F f) {
+  typedef typename Vec16<T>::type V;
+  constexpr int N = Vec16<T>::N;
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i >= nvec) return;
+  const long e = i * N;
+  const V a = ld_stream(reinterpret_cast<const V*>(full + e));
+  V b;
+  if (s == 1) {
+    b = *reinterpret_cast<const V*>(vec + ((unsigned)e % (unsigned)nv));  // n is a 32-bit int at the ABI: 32-bit division
+  } else {
+    const T bv = vec[((unsigned)e / (unsigned)s) % (unsigned)nv];
+#pragma unroll
+    for (int k = 0; k < N; k++) b[k] = bv;
+  }
+  V r;
+#pragma unroll
+  for (int k = 0; k < N; k++) r[k] = XFULL ? f(a[k], b[k]) : f(b[k], a[k]);
+  st_stream(reinterpret_cast<V*>(z + e), r);
+}
+
 template <typename T, typename F>
 inline void launch_bcast12(hipStream_t stream, long n, const T* x, int sx, int nx, const T* y, int sy, int ny, T* z, F f) {
   if (n <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  const bool xfull = (nx == n), yfull = (ny == n);
+  if (xfull != yfull && n % N == 0 && aligned16(x) && aligned16(y) && aligned16(z)) {
+    const int s = xfull ? sy : sx, nv = xfull ? ny : nx;
+    const bool fits = (s == 1) ? (nv % N == 0) : (s % N == 0);
+    if (fits && nv > 1) {
+      const long nvec = n / N, grid = (nvec + kEwBlock - 1) / kEwBlock;
+      if (xfull)
+        hipLaunchKernelGGL((ew_bias_vec_kernel<T, F, true>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, x, y, s, nv, z, f);
+      else
+        hipLaunchKernelGGL((ew_bias_vec_kernel<T, F, false>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, y, x, s, nv, z, f);
+      return;
+    }
+  }
   const long grid = (n + kEwBlock * 4 - 1) / (kEwBlock * 4);
   hipLaunchKernelGGL((ew_bcast12_kernel<T, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, x, sx, nx, y, sy, ny, z, f);
 }

@@ -89,6 +89,9 @@ __device__ __forceinline__ T team_reduce(T v, T* lds, Merge merge, T identity) {
 template <typename T, typename Algo, int TEAM, int E, bool VEC>
 __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out,
                                                                                 const int* labels, T scale, T* loss) {
+  // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
+  // output pass, so the dependent chain is one memory round trip instead of two.
+  constexpr bool kHold = Algo::kHoldA || (TEAM == kWave && E <= 16);
   constexpr int BT = TEAM == kWave ? 256 : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
@@ -103,22 +106,22 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel
   const T* bc = Algo::kInputs == 2 ? b + base : nullptr;
   T* oc = out + base;
 
-  T ra[Algo::kHoldA ? E : 1], rb[Algo::kInputs == 2 ? E : 1];
+  T ra[kHold ? E : 1], rb[Algo::kInputs == 2 ? E : 1];
 #pragma unroll
   for (int i = 0; i < ITEMS; i++) {
     const int r = (tl + i * TEAM) * NV;
     const bool ok = colok && r < m;
     if (VEC) {
       V va = {}, vb = {};
-      if (ok && Algo::kHoldA) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+      if (ok && kHold) va = ld_stream(reinterpret_cast<const V*>(ac + r));
       if (ok && Algo::kInputs == 2) vb = ld_stream(reinterpret_cast<const V*>(bc + r));
 #pragma unroll
       for (int e = 0; e < NV; e++) {
-        if (Algo::kHoldA) ra[i * NV + e] = ok ? va[e] : T(0);
+        if (kHold) ra[i * NV + e] = ok ? va[e] : T(0);
         if (Algo::kInputs == 2) rb[i * NV + e] = ok ? vb[e] : T(0);
       }
     } else {
-      if (Algo::kHoldA) ra[i] = ok ? __builtin_nontemporal_load(ac + r) : T(0);
+      if (kHold) ra[i] = ok ? __builtin_nontemporal_load(ac + r) : T(0);
       if (Algo::kInputs == 2) rb[i] = ok ? __builtin_nontemporal_load(bc + r) : T(0);
     }
   }
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel
 #pragma unroll
     for (int e = 0; e < NV; e++) {
       const bool ok = colok && (tl + i * TEAM) * NV + e < m;
-      if (ok) s = s + Algo::term(Algo::kHoldA ? ra[i * NV + e] : T(0), Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx);
+      if (ok) s = s + Algo::term(kHold ? ra[i * NV + e] : T(0), Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx);
     }
   s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
   const T fin = Algo::finish(s);
@@ -159,13 +162,13 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel
     if (!ok) continue;
     T o[NV];
     V va = {};
-    if (!Algo::kHoldA) {
+    if (!kHold) {
       if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
       else va[0] = __builtin_nontemporal_load(ac + r);
     }
 #pragma unroll
     for (int e = 0; e < NV; e++) {
-      const T av = Algo::kHoldA ? ra[i * NV + e] : va[e];
+      const T av = kHold ? ra[i * NV + e] : va[e];
       T v = Algo::out(av, Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx, fin);
       if (Algo::kNll) {
         const bool hit = (r + e + 1 == lab);
@@ -325,6 +328,35 @@ __global__ __launch_bounds__(1024) void softmax_col_stream_kernel(long m, long n
     oc[r] = v;
   }
   if (Algo::kNll && lab == 0 && threadIdx.x == 0) loss[col] = T(0);
+}
+
+// ---- softmax along a non-leading axis: x viewed as (inner, d, outer), softmax over d -----------------------
+// Lanes run along `inner` (contiguous), so every access is coalesced; each lane walks its own d elements three
+// times (max, sum, output).  The reference handles these `dims` with a chain of broadcast and reduction kernels
+// (src/ops20/softmax.jl:42-63 through src/ops20_gpu/softmax.jl:22); one kernel replaces the chain.
+template <typename T, typename Algo>
+__global__ __launch_bounds__(256) void softmax_strided_kernel(long inner, long d, long outer, const T* a, const T* b, T* out) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= inner * outer) return;
+  const long i = idx % inner, o = idx / inner;
+  const long base = o * d * inner + i;
+  T mx = T(0);
+  if (Algo::kNeedMax) {
+    mx = -INFINITY;
+    for (long k = 0; k < d; k++) { const T v = a[base + k * inner]; mx = mx > v ? mx : v; }
+  }
+  T s = T(0);
+  for (long k = 0; k < d; k++) s = s + Algo::term(a[base + k * inner], Algo::kInputs == 2 ? b[base + k * inner] : T(0), mx);
+  const T fin = Algo::finish(s);
+  for (long k = 0; k < d; k++)
+    out[base + k * inner] = Algo::out(a[base + k * inner], Algo::kInputs == 2 ? b[base + k * inner] : T(0), mx, fin);
+}
+
+template <typename T, typename Algo>
+inline void launch_softmax_strided(hipStream_t stream, long inner, long d, long outer, const T* a, const T* b, T* out) {
+  if (inner <= 0 || d <= 0 || outer <= 0) return;
+  const long total = inner * outer;
+  hipLaunchKernelGGL((softmax_strided_kernel<T, Algo>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, inner, d, outer, a, b, out);
 }
 
 template <typename T, typename Algo, int TEAM, int E>

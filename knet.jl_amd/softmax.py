@@ -25,6 +25,22 @@ def _columns(x, dims):
     return None
 
 
+def _view3(x, dims):
+    """(inner, d, outer) when ``dims`` is a run of adjacent dimensions, else None."""
+    d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
+    if not d or d != list(range(d[0], d[-1] + 1)) or d[-1] > x.ndims:
+        return None
+    inner = mid = outer = 1
+    for i in range(1, x.ndims + 1):
+        if i < d[0]:
+            inner *= x.size(i)
+        elif i <= d[-1]:
+            mid *= x.size(i)
+        else:
+            outer *= x.size(i)
+    return inner, mid, outer
+
+
 def _fwd(kernel, x, m, n):
     y = x.similar()
     knet8("%s_%s" % (kernel, x.suffix), m, n, x.ptr, y.ptr)
@@ -55,14 +71,18 @@ def _make(kernel, backkernel):
             m, n = mn
             y = _fwd(kernel, x, m, n)
             return y, (lambda dy: (_bwd(backkernel, y, dy, m, n),))  # @primitive1 _cudnnSoftmaxForward(x),dy,y _cudnnSoftmaxBackward(y,dy)
-        d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
-        if x.ndims == 2 and d == [2]:
-            xt = permutedims(x)
-            m, n = xt.size(1), xt.size(2)
-            yt = _fwd(kernel, xt, m, n)
-            y = permutedims(yt)
-            return y, (lambda dy: (permutedims(_bwd(backkernel, yt, permutedims(dy), m, n)),))
-        raise NotImplementedError("softmax over dims=%r of a %d-d array" % (dims, x.ndims))
+        v3 = _view3(x, dims)
+        if v3 is not None:  # a run of adjacent non-leading dims: one strided kernel instead of the reference's transposes/broadcast chain
+            inner, d, outer = v3
+            y = x.similar()
+            knet8("%s_strided_%s" % (kernel, x.suffix), inner, d, outer, x.ptr, y.ptr)
+
+            def back(dy):
+                dx = y.similar()
+                knet8("%s_strided_%s" % (backkernel, y.suffix), inner, d, outer, y.ptr, dy.ptr, dx.ptr)
+                return (dx,)
+            return y, back
+        raise NotImplementedError("softmax over non-adjacent dims=%r of a %d-d array" % (dims, x.ndims))
 
     f.__name__ = kernel
     return f

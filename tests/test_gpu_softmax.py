@@ -51,6 +51,16 @@ def test_other_dims_and_misaligned_columns(knet, oracle):
     x3 = (rng.standard_normal((3, 4, 5)) * 2).astype(np.float32)
     got = knet.Array(knet.logsoftmax(knet.KnetArray(x3), dims=[1, 2]))
     assert close(got, oracle.logsoftmax(x3, dims=(1, 2)))
+    # non-leading dims (test/loss.jl:10-45 sweeps dims 1,2,3,(1,2),(2,3)...) incl. gradients through the tape
+    for shape, dims in [((3, 4, 5), 2), ((3, 4, 5), 3), ((3, 4, 5), [2, 3]), ((70, 33, 9), 2), ((300, 1000), 2), ((5, 1, 7), 2)]:
+        xx = (rng.standard_normal(shape) * 2).astype(np.float32)
+        dyy = rng.standard_normal(shape).astype(np.float32)
+        od = tuple(dims) if isinstance(dims, list) else dims
+        for f, fo, bo in ((knet.logsoftmax, oracle.logsoftmax, oracle.logsoftmaxback), (knet.softmax, oracle.softmax, oracle.softmaxback)):
+            p = knet.Param(knet.KnetArray(xx))
+            assert close(knet.Array(f(knet.KnetArray(xx), dims=dims)), fo(xx, dims=od)), (shape, dims)
+            J = knet.diff(lambda: knet.sum(knet.mul(f(p, dims=dims), knet.KnetArray(dyy))))
+            assert close(knet.Array(knet.grad(J, p)), bo(fo(xx, dims=od), dyy, dims=od), 2e-5), (shape, dims)
     v = (rng.standard_normal(777) * 3).astype(np.float32)
     assert close(knet.Array(knet.logsoftmax(knet.KnetArray(v), dims=1)), oracle.logsoftmax(v, dims=1))
     # columns that are not 16-byte aligned (m odd) and a base pointer inside an allocation
