@@ -30,6 +30,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of reluback_32_11 on 2^28 elements from the two `rocprofv3 --pmc` runs summarised in
+# profiles/libknet8_kernels_profile_pass.txt: FETCH_SIZE 1048576 KiB x 2.0000 + WRITE_SIZE 1048600 KiB x 0.9990, each scaled by
+# what the same counter reads for the 1 GiB + 1 GiB copy kernel of that run.  (Algorithmic: 3 * 4 * 2^28 = 3221225472.)
+RELUBACK_32_TRAFFIC_BYTES = int((2048.0 + 1023.0) * (1 << 20))
 OPS = [("reluback", "relu"), ("sigmback", "sigm"), ("tanhback", "tanh"), ("eluback", "elu"), ("seluback", "selu")]
 
 
@@ -315,7 +319,7 @@ def main():
         "config": {"workload": "BASELINE config 2: {relu,sigm,tanh,elu,selu}back on 2^28 fp32 and 2^27 fp64 vectors, "
                                "x,dy~N(0,1) seeded, y=f(x); 10 launches per step", "frac_of_hbm_peak": value / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "reluback_32_11 (ew_vec_kernel<float,2>)", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": dom["bytes"],
+                     "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": RELUBACK_32_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": dom["bytes"],
                      "avg_launch_us": dom["us"]},
         "kernels_config2": {k: {"us": round(v["us"], 2), "GBps": round(v["GBps"], 1), "frac": round(v["GBps"] / HBM_PEAK_GBS, 4)} for k, v in per_kernel.items()},
     }
