@@ -1,0 +1,152 @@
+"""The C ABI itself on the GPU: both forms of an entry point, caller-owned streams, no-op sizes, operand order of the
+broadcast forms, error reporting, the allocator and the GEMM entry points."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import bits_equal
+
+pytestmark = pytest.mark.gpu
+
+
+def test_plain_twin_and_stream_form_agree(knet, oracle):
+    rng = np.random.default_rng(51)
+    fn = knet.libknet8().fn
+    n = 70001
+    dy, y = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    dyd, yd = knet.KnetArray(dy), knet.KnetArray(y)
+    a, b = dyd.similar(), dyd.similar()
+    fn["tanhback_32_11"](n, dyd.ptr, yd.ptr, a.ptr)                      # plain form: null stream
+    s = fn["knet8_stream_create"]()
+    assert s
+    fn["tanhback_32_11_stream"](n, dyd.ptr, yd.ptr, b.ptr, s)            # what @knet8 binds
+    assert fn["knet8_synchronize"](s) == 0
+    want = oracle.back11("tanhback", dy, y)
+    assert bits_equal(knet.Array(a), want) and bits_equal(knet.Array(b), want)
+    fn["knet8_stream_destroy"](s)
+    knet.libknet8().check()
+
+
+def test_split_reductions_on_two_streams_do_not_share_scratch(knet):
+    rng = np.random.default_rng(52)
+    fn = knet.libknet8().fn
+    x1 = rng.integers(-3, 4, size=(4096, 600)).astype(np.float32)
+    x2 = rng.integers(-3, 4, size=(2048, 900)).astype(np.float32)
+    d1, d2 = knet.KnetArray(x1), knet.KnetArray(x2)
+    y1, y2 = knet.KnetArray(np.zeros(4096, np.float32)), knet.KnetArray(np.zeros(2048, np.float32))
+    s1, s2 = fn["knet8_stream_create"](), fn["knet8_stream_create"]()
+    for _ in range(20):  # interleave launches that both need partials + tickets
+        fn["sum_32_21_stream"](x1.size, d1.ptr, 1, 4096, y1.ptr, s1)
+        fn["sum_32_21_stream"](x2.size, d2.ptr, 1, 2048, y2.ptr, s2)
+    fn["knet8_synchronize"](s1)
+    fn["knet8_synchronize"](s2)
+    assert np.array_equal(knet.Array(y1), x1.sum(axis=1)) and np.array_equal(knet.Array(y2), x2.sum(axis=1))
+    r = fn["sum_32_20_stream"](x1.size, d1.ptr, s1)
+    assert r == x1.sum()
+    fn["knet8_stream_destroy"](s1)
+    fn["knet8_stream_destroy"](s2)
+    knet.libknet8().check()
+
+
+def test_zero_and_negative_sizes_are_no_ops(knet):
+    fn = knet.libknet8().fn
+    a = knet.KnetArray(np.full(8, 3.0, np.float32))
+    for n in (0, -5):
+        fn["reluback_32_11"](n, a.ptr, a.ptr, a.ptr)
+        fn["relu_32"](n, a.ptr, a.ptr)
+        fn["fill_32"](n, ctypes.c_float(9), a.ptr)
+        fn["dropback_32"](n, ctypes.c_float(0.5), a.ptr, a.ptr, a.ptr, a.ptr)
+        fn["add_32_12"](n, a.ptr, 1, 8, a.ptr, 1, 8, a.ptr)
+        fn["logsoftmaxback_32"](n, 4, a.ptr, a.ptr, a.ptr)
+        fn["getents_32"](n, a.ptr, a.ptr, a.ptr)
+    assert fn["sum_32_20"](0, a.ptr) == 0.0 and fn["maximum_32_20"](0, a.ptr) == -np.inf and fn["prod_64_20"](0, a.ptr) == 1.0
+    assert np.all(knet.Array(a) == 3.0)
+    knet.libknet8().check()
+
+
+def test_broadcast_forms_keep_operand_order(knet):
+    rng = np.random.default_rng(53)
+    fn = knet.libknet8().fn
+    for shape, k in [((64, 100), 0), ((64, 100), 1), ((6, 10, 7), 1), ((513, 1025), 1), ((5, 7), 0)]:
+        x = rng.standard_normal(shape).astype(np.float64)
+        vshape = [1] * len(shape)
+        vshape[k] = shape[k]
+        v = (rng.standard_normal(vshape) + 3).astype(np.float64)
+        xd, vd = knet.KnetArray(x), knet.KnetArray(v)
+        n, stride = x.size, int(np.prod(shape[:k], dtype=np.int64))
+        z = xd.similar()
+        for op, f in (("sub", np.subtract), ("div", np.divide), ("add", np.add), ("max", np.maximum)):
+            fn["%s_64_12" % op](n, xd.ptr, 1, n, vd.ptr, stride, shape[k], z.ptr)      # full (op) vector
+            assert bits_equal(knet.Array(z), f(x, v)), (op, shape, k)
+            fn["%s_64_12" % op](n, vd.ptr, stride, shape[k], xd.ptr, 1, n, z.ptr)      # vector (op) full
+            assert bits_equal(knet.Array(z), f(v, x)), (op, shape, k)
+            fn["%s_64_13_x_y" % op](xd.ptr, vd.ptr, z.ptr, stride, 0, 1, n, shape[k])  # x[i] (op) vec
+            assert bits_equal(knet.Array(z), f(x, v)), (op, shape, k)
+            fn["%s_64_13_y_x" % op](xd.ptr, vd.ptr, z.ptr, stride, 0, 1, n, shape[k])  # vec (op) x[i]
+            assert bits_equal(knet.Array(z), f(v, x)), (op, shape, k)
+        fn["sub_64_01"](n, ctypes.c_double(2.5), xd.ptr, z.ptr)                        # scalar (op) array
+        assert bits_equal(knet.Array(z), 2.5 - x)
+        fn["div_64_01"](n, ctypes.c_double(2.5), xd.ptr, z.ptr)
+        assert bits_equal(knet.Array(z), 2.5 / x)
+    knet.libknet8().check()
+
+
+def test_errors_are_recorded_not_dropped(knet):
+    lib = knet.libknet8()
+    a = knet.KnetArray(np.zeros(12, np.float32))
+    lib.fn["sum_32_21"](12, a.ptr, 5, 2, a.ptr)       # 12 is not a multiple of 5*2
+    with pytest.raises(RuntimeError, match="multiple"):
+        lib.check()
+    lib.check()                                        # reading clears it
+    lib.fn["knet8_free"](ctypes.c_void_p(12345))
+    with pytest.raises(RuntimeError, match="knet8_malloc"):
+        lib.check()
+    assert lib.fn["knet8_memcpy"](a.ptr, a.ptr, 4, 7, None) == -1
+    with pytest.raises(RuntimeError, match="kind"):
+        lib.check()
+
+
+def test_allocator_pool(knet):
+    fn = knet.libknet8().fn
+    info = (4 * ctypes.c_size_t)()
+    fn["knet8_trim"]()
+    fn["knet8_meminfo"](info)
+    live0 = info[0]
+    ptrs = [fn["knet8_malloc"](1000) for _ in range(4)]
+    assert len(set(ptrs)) == 4 and all(p % 256 == 0 for p in ptrs)
+    fn["knet8_meminfo"](info)
+    assert info[0] == live0 + 4 * 1024            # 1000 rounds up to 1024
+    for p in ptrs:
+        fn["knet8_free"](p)
+    fn["knet8_meminfo"](info)
+    assert info[0] == live0 and info[1] >= 4 * 1024
+    again = fn["knet8_malloc"](1001)              # same size class: served from the free list
+    assert again in ptrs
+    fn["knet8_free"](again)
+    assert fn["knet8_trim"]() >= 4 * 1024
+    fn["knet8_meminfo"](info)
+    assert info[1] == 0
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt,S", [(np.float32, "32"), (np.float64, "64")])
+def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
+    rng = np.random.default_rng(54)
+    rtol = 1e-5 if dt == np.float32 else 1e-13
+    for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000)]:
+        A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
+        want = oracle.gemm(A, B)
+        Ad, Bd, Atd, Btd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.ascontiguousarray(A.T)), knet.KnetArray(np.ascontiguousarray(B.T))
+        for ta, tb, a, b in (("N", "N", Ad, Bd), ("T", "N", Atd, Bd), ("N", "T", Ad, Btd), ("T", "T", Atd, Btd)):
+            C = knet.gemm(ta, tb, 1, a, b, 0, knet.KnetArray(np.zeros((m, n), dt)))
+            got = knet.Array(C)
+            assert np.linalg.norm(got - want) <= rtol * np.linalg.norm(want), (m, n, k, ta, tb)
+        # alpha / beta
+        C0 = rng.standard_normal((m, n)).astype(dt)
+        C = knet.gemm("N", "N", 0.5, Ad, Bd, 2.0, knet.KnetArray(C0))
+        assert np.linalg.norm(knet.Array(C) - (0.5 * want + 2 * C0)) <= 10 * rtol * np.linalg.norm(want)
+        assert bits_equal(knet.Array(knet.transpose(Ad)), np.ascontiguousarray(A.T))
+    with pytest.raises(ValueError):
+        knet.gemm("N", "N", 1, knet.KnetArray(np.zeros((3, 4), dt)), knet.KnetArray(np.zeros((5, 2), dt)), 0, knet.KnetArray(np.zeros((3, 2), dt)))
+    knet.libknet8().check()
