@@ -266,6 +266,36 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused):
     return {"steps_per_sec": steps / dt, "ms_per_step": dt / steps * 1e3, "loss": float(K.value(J))}
 
 
+def cpu_side_table():
+    """The oracle's loops for the config 3-5 kernels, one thread, full shapes (each takes well under a second)."""
+    from oracle import knet_oracle as ko
+    rng = np.random.default_rng(1)
+    out = {}
+
+    def t(name, nbytes, f):
+        f()
+        t0 = time.perf_counter()
+        f()
+        dt = time.perf_counter() - t0
+        out[name] = {"ms": round(dt * 1e3, 2), "GBps": round(nbytes / dt * 1e-9, 2)}
+    x = rng.standard_normal((4096, 8192), dtype=np.float32)
+    xf = x.ravel(order="F")
+    t("sum (4096,8192) dims=1", x.nbytes, lambda: ko.sum_21(xf, 4096, 8192))
+    t("sum (4096,8192) dims=2", x.nbytes, lambda: ko.sum_21(xf, 1, 4096))
+    x = rng.standard_normal((56, 56, 256, 64), dtype=np.float32)
+    xf = x.ravel(order="F")
+    t("sum NCHW (56,56,256,64)->(1,1,256,1)", x.nbytes, lambda: ko.sum_21(xf, 3136, 256))
+    for C, N in ((32000, 512), (1000, 4096)):
+        y = rng.standard_normal((C, N), dtype=np.float32)
+        dy = rng.standard_normal((C, N), dtype=np.float32)
+        labels = rng.integers(1, C + 1, size=N)
+        t("logsoftmaxback (%d,%d)" % (C, N), 12 * C * N, lambda: ko.logsoftmaxback(y, dy, dims=1))
+        t("nll backward chain (%d,%d)" % (C, N), 8 * C * N, lambda: ko.nll_back(y, labels))
+    y = rng.standard_normal(4096 * 2048).astype(np.float32)
+    t("dropback (4096,2048)", 12 * y.size, lambda: ko.dropback(0.5, y, y, y))
+    return out
+
+
 def cpu_baseline():
     """The oracle's *back loops (plain C, one thread) on a bounded sample of the config-2 workload."""
     from oracle import knet_oracle as ko
@@ -336,6 +366,8 @@ def main():
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
         }
     line["cpu_baseline"] = cpu_baseline()
+    if not args.no_extras:
+        line["cpu_oracle_config3_4_5 (1 thread, algorithmic GB/s)"] = cpu_side_table()
     print(json.dumps(line))
 
 

@@ -191,6 +191,23 @@ void F(ko_reduce)(int op, int nd, const long *dims, const int *mask, const T *x,
   free(acc);
 }
 
+/* The `_21` contract stated directly: x[i] goes into y[(i/sy)%ny] (src/libknet8/cuda21.jl:23), walked in memory
+ * order with a wide accumulator per output.  Same result as ko_reduce on the (sy,ny,nx/(sy*ny)) view with dims 1
+ * and 3 reduced; kept separate because it is the form the C ABI takes and the loop the CPU baseline times. */
+void F(ko_sum_21)(long nx, const T *x, long sy, long ny, T *y) {
+  W *acc = (W *)calloc((size_t)(ny > 0 ? ny : 1), sizeof(W));
+  const long slab = sy * ny;
+  for (long o = 0; o + slab <= nx; o += slab)
+    for (long j = 0; j < ny; j++) {
+      const T *run = x + o + j * sy;
+      W a = acc[j];
+      for (long s = 0; s < sy; s++) a += (W)run[s];
+      acc[j] = a;
+    }
+  for (long j = 0; j < ny; j++) y[j] = (T)acc[j];
+  free(acc);
+}
+
 /* ---- softmax family over the middle axis of an (inner, d, outer) view ------
  * dims=1 of an (m,n) matrix is inner=1,d=m,outer=n; dims=2 is inner=m,d=n,outer=1.
  * _logsoftmax: x = x .- maximum(x); x .- log.(sum(exp.(x)))  -- src/ops20/softmax.jl:42-47 */

@@ -137,6 +137,16 @@ def reduce(op, x, dims=None):
     return _shape_like(y, yshape)
 
 
+def sum_21(x, sy, ny):
+    """The raw ``sum_S_21`` contract on a flat array: ``x[i]`` goes into ``y[(i // sy) % ny]``."""
+    x = np.asarray(x)
+    s, _ = _sfx(x.dtype)
+    xf = _flat(x)
+    y = np.empty(ny, dtype=x.dtype)
+    getattr(lib(), "ko_sum_21_%s" % s)(ctypes.c_long(xf.size), _ptr(xf), ctypes.c_long(sy), ctypes.c_long(ny), _ptr(y))
+    return y
+
+
 def _view3(shape, dims):
     """(inner, d, outer) for a softmax along the contiguous group of 1-based ``dims``."""
     nd = len(shape)

@@ -71,6 +71,20 @@ def test_sum_invariants_and_regression_shapes(oracle):
     assert np.array_equal(oracle.reduce("sum", x, dims=(1, 2, 4)).ravel(), x.sum(axis=(0, 1, 3)))
 
 
+def test_sum_21_contract_matches_the_generic_reduction(oracle):
+    # x[i] goes into y[(i/sy)%ny] (src/libknet8/cuda21.jl:23) == reduce dims 1 and 3 of the (sy,ny,no) view
+    rng = np.random.default_rng(11)
+    for sy, ny, no in [(1, 7, 13), (5, 3, 9), (4, 1, 6), (3136 // 8, 16, 4), (1, 1, 50)]:
+        x = rng.integers(-5, 6, size=(sy, ny, no)).astype(np.float32)
+        got = oracle.sum_21(x, sy, ny)
+        assert np.array_equal(got, x.sum(axis=(0, 2)))
+        assert np.array_equal(got, oracle.reduce("sum", x, dims=(1, 3)).ravel())
+        brute = np.zeros(ny)
+        for i, v in enumerate(x.ravel(order="F")):
+            brute[(i // sy) % ny] += v
+        assert np.array_equal(got, brute)
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_softmax_family_invariants(oracle, dt):
     # invariants asserted by test/loss.jl:47-56
