@@ -17,6 +17,7 @@ from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
 from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback
 from .loss import nll, findindices, accuracy, getindex, ungetindex
 from .dropout import dropout, dropback, dropout_, dropback_
+from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
 from .linalg import matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose
 
 libknet8()  # fail loudly at import time if the HIP library is missing

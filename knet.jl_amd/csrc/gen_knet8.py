@@ -98,6 +98,36 @@ BACK111_OPS = [
      "src/ops21/activation.jl:171, src/libknet8/ops.jl:135"),
 ]
 
+# Fused optimizer updates: name, scalar parameters (all of type T, derived on the host exactly as the Julia code derives
+# them: T(-lr), T(1-rho), T(1-beta1^t) ...), arrays (in order), write mask, body on v[...], citation.  Each body is the
+# per-element sequence of the reference's lmul!/axpy!/broadcast chain, one rounding per operation.
+OPTIMIZER_OPS = [
+    ("momentum", ["nlr", "gamma"], ["g", "vel", "w"], 0b110,
+     "const T v1 = gamma * v[1]; const T p = nlr * v[0]; const T v2 = v1 + p; v[1] = v2; v[2] = v[2] + v2;",
+     "src/train20/update.jl:517-522"),
+    ("nesterov", ["nlr", "gamma", "opg"], ["g", "vel", "w"], 0b110,
+     "const T v1 = gamma * v[1]; const T m1 = T(-1) * v1; const T w1 = v[2] + m1; const T p = nlr * v[0]; const T v2 = v1 + p; "
+     "const T q = opg * v2; v[1] = v2; v[2] = w1 + q;",
+     "src/train20/update.jl:525-531"),
+    ("adagrad", ["nlr", "eps"], ["g", "G", "w"], 0b110,
+     "const T gg = v[0] * v[0]; const T G1 = v[1] + gg; const T t = G1 + eps; const T q = v[0] / ksqrt(t); const T p = nlr * q; v[1] = G1; v[2] = v[2] + p;",
+     "src/train20/update.jl:533-538"),
+    ("rmsprop", ["nlr", "rho", "omr", "eps"], ["g", "G", "w"], 0b110,
+     "const T G1 = rho * v[1]; const T gg = v[0] * v[0]; const T a = omr * gg; const T G2 = G1 + a; const T t = G2 + eps; const T q = v[0] / ksqrt(t); "
+     "const T p = nlr * q; v[1] = G2; v[2] = v[2] + p;",
+     "src/train20/update.jl:540-546"),
+    ("adadelta", ["nlr", "rho", "omr", "eps"], ["g", "G", "delta", "w"], 0b1110,
+     "const T G1 = rho * v[1]; const T gg = v[0] * v[0]; const T a = omr * gg; const T G2 = G1 + a; const T sd = ksqrt(v[2] + eps); const T num = v[0] * sd; "
+     "const T dw = num / ksqrt(G2 + eps); const T d1 = rho * v[2]; const T dd = dw * dw; const T b = omr * dd; const T p = nlr * dw; "
+     "v[1] = G2; v[2] = d1 + b; v[3] = v[3] + p;",
+     "src/train20/update.jl:548-557"),
+    ("adam", ["nlr", "beta1", "omb1", "beta2", "omb2", "c1", "c2", "eps"], ["g", "fstm", "scndm", "w"], 0b1110,
+     "const T m1 = beta1 * v[1]; const T a = omb1 * v[0]; const T m2 = m1 + a; const T s1 = beta2 * v[2]; const T gg = v[0] * v[0]; const T b = omb2 * gg; "
+     "const T s2 = s1 + b; const T mc = m2 / c1; const T sc = s2 / c2; const T den = ksqrt(sc) + eps; const T q = mc / den; const T p = nlr * q; "
+     "v[1] = m2; v[2] = s2; v[3] = v[3] + p;",
+     "src/train20/update.jl:559-570"),
+]
+
 # Reduction operators: order and meaning of src/libknet8/ops.jl:144-156.
 REDUCTION_OPS = [("sum", "RedSum"), ("prod", "RedProd"), ("maximum", "RedMaximum"), ("minimum", "RedMinimum"),
                  ("sumabs", "RedSumabs"), ("sumabs2", "RedSumabs2"), ("maxabs", "RedMaxabs"), ("minabs", "RedMinabs"),
@@ -231,6 +261,18 @@ def gen_elementwise():
         o.entry("scal_%s" % S, "void", [("int", "n"), (T, "alpha"), (T + "*", "x")],
                 "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, x, OpScal<%s>{alpha})" % (T, T, T, T),
                 "cublas%sscal_v2 with unit increment at src/knetarrays/linalg.jl:75-90" % ("S" if S == "32" else "D"))
+    o.decl.append("\n/* ---- fused optimizer updates (in place).  No libknet8 counterpart: each replaces the lmul!/axpy!/broadcast chain of one\n"
+                  "   _update! method of src/train20/update.jl:513-570 (SGD itself is axpy_S).  Scalars are the T-rounded constants the\n"
+                  "   Julia code forms: nlr = T(-lr), opg = T(1+gamma), omr = T(1-rho), omb1 = T(1-beta1), c1 = T(1-beta1^t) ... ---- */")
+    for name, scalars, arrays, mask, body, cite in OPTIMIZER_OPS:
+        fields = " ".join("T %s;" % x for x in scalars)
+        s.append("template <typename T> struct Opt_%s { %s __device__ __forceinline__ void operator()(T (&v)[%d]) const { %s } };\n"
+                 % (name, fields, len(arrays), body))
+        for T, S in TYPES:
+            params = [("int", "n")] + [(T, x) for x in scalars] + [(T + "*", a) for a in arrays]
+            ptrs = arrays + ["(%s*)nullptr" % T] * (4 - len(arrays))
+            o.entry("%s_%s" % (name, S), "void", params,
+                    "launch_update<%s, %d, %du>(stream, n, %s, Opt_%s<%s>{%s})" % (T, len(arrays), mask, ", ".join(ptrs), name, T, ", ".join(scalars)), cite)
     return o
 
 

@@ -171,4 +171,78 @@ inline void launch_bcast12(hipStream_t stream, long n, const T* x, int sx, int n
   hipLaunchKernelGGL((ew_bcast12_kernel<T, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, x, sx, nx, y, sy, ny, z, f);
 }
 
+// In-place update of NARR same-length arrays: v[k] = element of array k; f(v) rewrites some of them; the arrays
+// whose bit is set in WMASK are stored back.  One pass over every array instead of the axpy!/lmul!/broadcast
+// chains of the optimizers (src/train20/update.jl:513-570).  HBM roofline: (NARR + popcount(WMASK))*sizeof(T)
+// bytes per element.  Vector path when every array is 16-byte aligned, scalar otherwise; the last n % N
+// elements are done as scalars by workgroup 0.
+template <typename T, int NARR, unsigned WMASK, typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_update_vec_kernel(long nvec, long n, T* a0, T* a1, T* a2, T* a3, F f) {
+  typedef typename Vec16<T>::type V;
+  constexpr int N = Vec16<T>::N;
+  T* arr[4] = {a0, a1, a2, a3};
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i < nvec) {
+    V in[NARR];
+#pragma unroll
+    for (int k = 0; k < NARR; k++) in[k] = ld_stream(reinterpret_cast<const V*>(arr[k] + i * N));
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      T v[NARR];
+#pragma unroll
+      for (int k = 0; k < NARR; k++) v[k] = in[k][e];
+      f(v);
+#pragma unroll
+      for (int k = 0; k < NARR; k++) in[k][e] = v[k];
+    }
+#pragma unroll
+    for (int k = 0; k < NARR; k++)
+      if (WMASK & (1u << k)) st_stream(reinterpret_cast<V*>(arr[k] + i * N), in[k]);
+  }
+  if (blockIdx.x == 0) {
+    const long e = nvec * N + threadIdx.x;
+    if (e < n) {
+      T v[NARR];
+#pragma unroll
+      for (int k = 0; k < NARR; k++) v[k] = arr[k][e];
+      f(v);
+#pragma unroll
+      for (int k = 0; k < NARR; k++)
+        if (WMASK & (1u << k)) arr[k][e] = v[k];
+    }
+  }
+}
+
+template <typename T, int NARR, unsigned WMASK, typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_update_scalar_kernel(long n, T* a0, T* a1, T* a2, T* a3, F f) {
+  T* arr[4] = {a0, a1, a2, a3};
+  const long e = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (e >= n) return;
+  T v[NARR];
+#pragma unroll
+  for (int k = 0; k < NARR; k++) v[k] = arr[k][e];
+  f(v);
+#pragma unroll
+  for (int k = 0; k < NARR; k++)
+    if (WMASK & (1u << k)) arr[k][e] = v[k];
+}
+
+template <typename T, int NARR, unsigned WMASK, typename F>
+inline void launch_update(hipStream_t stream, long n, T* a0, T* a1, T* a2, T* a3, F f) {
+  if (n <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  T* arr[4] = {a0, a1, a2, a3};
+  bool al = true;
+  for (int k = 0; k < NARR; k++) al = al && aligned16(arr[k]);
+  if (al) {
+    const long nvec = n / N;
+    long grid = (nvec + kEwBlock - 1) / kEwBlock;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL((ew_update_vec_kernel<T, NARR, WMASK, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, n, a0, a1, a2, a3, f);
+  } else {
+    const long grid = (n + kEwBlock - 1) / kEwBlock;
+    hipLaunchKernelGGL((ew_update_scalar_kernel<T, NARR, WMASK, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, a0, a1, a2, a3, f);
+  }
+}
+
 }  // namespace knet8

@@ -90,6 +90,7 @@ long ko_findindices(long y1, long y2, const int *labels, long ninstances, int di
 #define LOG logf
 #define TANH tanhf
 #define ERF erff
+#define SQRT sqrtf
 #include "knet_cpu_body.h"
 #undef T
 #undef W
@@ -98,6 +99,7 @@ long ko_findindices(long y1, long y2, const int *labels, long ninstances, int di
 #undef LOG
 #undef TANH
 #undef ERF
+#undef SQRT
 
 #define T double
 #define W long double
@@ -106,6 +108,7 @@ long ko_findindices(long y1, long y2, const int *labels, long ninstances, int di
 #define LOG log
 #define TANH tanh
 #define ERF erf
+#define SQRT sqrt
 #include "knet_cpu_body.h"
 #undef T
 #undef W
@@ -114,3 +117,4 @@ long ko_findindices(long y1, long y2, const int *labels, long ninstances, int di
 #undef LOG
 #undef TANH
 #undef ERF
+#undef SQRT

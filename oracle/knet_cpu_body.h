@@ -347,6 +347,42 @@ void F(ko_gemm)(int ta, int tb, long m, long n, long k, const T *A, long lda, co
   }
 }
 
+/* ---- optimizer updates, per element, in the order of the lmul!/axpy!/broadcast chains of
+ * src/train20/update.jl:513-570 (lmul!(a,x): x = a*x; axpy!(a,x,y): y = y + a*x, product rounded first).
+ * Scalars arrive already rounded to T, as the Julia code rounds them (alpha = T[alpha], T(p.eps), T(1 - beta^t)). */
+void F(ko_momentum)(long n, T nlr, T gamma, const T *g, T *vel, T *w) {                       /* update.jl:517-522 */
+  for (long i = 0; i < n; i++) { T v1 = gamma * vel[i]; T p = nlr * g[i]; T v2 = v1 + p; vel[i] = v2; w[i] = w[i] + v2; }
+}
+void F(ko_nesterov)(long n, T nlr, T gamma, T opg, const T *g, T *vel, T *w) {                /* update.jl:525-531 */
+  for (long i = 0; i < n; i++) {
+    T v1 = gamma * vel[i]; T m1 = (T)-1 * v1; T w1 = w[i] + m1; T p = nlr * g[i]; T v2 = v1 + p; T q = opg * v2;
+    vel[i] = v2; w[i] = w1 + q;
+  }
+}
+void F(ko_adagrad)(long n, T nlr, T eps, const T *g, T *G, T *w) {                            /* update.jl:533-538 */
+  for (long i = 0; i < n; i++) { T gg = g[i] * g[i]; T G1 = G[i] + gg; T t = G1 + eps; T q = g[i] / SQRT(t); T p = nlr * q; G[i] = G1; w[i] = w[i] + p; }
+}
+void F(ko_rmsprop)(long n, T nlr, T rho, T omr, T eps, const T *g, T *G, T *w) {              /* update.jl:540-546 */
+  for (long i = 0; i < n; i++) {
+    T G1 = rho * G[i]; T gg = g[i] * g[i]; T a = omr * gg; T G2 = G1 + a; T t = G2 + eps; T q = g[i] / SQRT(t); T p = nlr * q;
+    G[i] = G2; w[i] = w[i] + p;
+  }
+}
+void F(ko_adadelta)(long n, T nlr, T rho, T omr, T eps, const T *g, T *G, T *delta, T *w) {   /* update.jl:548-557 */
+  for (long i = 0; i < n; i++) {
+    T G1 = rho * G[i]; T gg = g[i] * g[i]; T a = omr * gg; T G2 = G1 + a; T sd = SQRT(delta[i] + eps); T num = g[i] * sd;
+    T dw = num / SQRT(G2 + eps); T d1 = rho * delta[i]; T dd = dw * dw; T b = omr * dd; T p = nlr * dw;
+    G[i] = G2; delta[i] = d1 + b; w[i] = w[i] + p;
+  }
+}
+void F(ko_adam)(long n, T nlr, T beta1, T omb1, T beta2, T omb2, T c1, T c2, T eps, const T *g, T *m, T *v, T *w) { /* update.jl:559-570 */
+  for (long i = 0; i < n; i++) {
+    T m1 = beta1 * m[i]; T a = omb1 * g[i]; T m2 = m1 + a; T s1 = beta2 * v[i]; T gg = g[i] * g[i]; T b = omb2 * gg; T s2 = s1 + b;
+    T mc = m2 / c1; T sc = s2 / c2; T den = SQRT(sc) + eps; T q = mc / den; T p = nlr * q;
+    m[i] = m2; v[i] = s2; w[i] = w[i] + p;
+  }
+}
+
 #undef F
 #undef CAT
 #undef CAT_

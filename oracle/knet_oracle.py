@@ -319,6 +319,38 @@ def gemm(A, B, ta=False, tb=False):
     return _shape_like(C, (m, n))
 
 
+def optimizer_scalars(kind, dtype, t=1, **hp):
+    """The T-rounded constants one update of ``kind`` needs, formed as the Julia code forms them
+    (src/train20/update.jl:513-570: ``alpha = T[alpha]``, ``T(p.eps)``, ``T(1 - p.beta1 ^ p.t)``; hyper-parameters are Float64 there)."""
+    T = np.dtype(dtype).type
+    lr = hp["lr"]
+    if kind == "momentum":
+        return [T(-lr), T(hp["gamma"])]
+    if kind == "nesterov":
+        return [T(-lr), T(hp["gamma"]), T(1 + hp["gamma"])]
+    if kind == "adagrad":
+        return [T(-lr), T(hp["eps"])]
+    if kind in ("rmsprop", "adadelta"):
+        return [T(-lr), T(hp["rho"]), T(1 - hp["rho"]), T(hp["eps"])]
+    if kind == "adam":
+        return [T(-lr), T(hp["beta1"]), T(1 - hp["beta1"]), T(hp["beta2"]), T(1 - hp["beta2"]),
+                T(1 - hp["beta1"] ** t), T(1 - hp["beta2"] ** t), T(hp["eps"])]
+    raise KeyError(kind)
+
+
+def optimizer_update(kind, g, state, w, t=1, **hp):
+    """One in-place-style update; returns (new_state_list, new_w) as fresh arrays.  ``state`` is the list of state arrays
+    in the order of the reference's struct fields (velocity | G | G, delta | fstm, scndm)."""
+    w = np.asarray(w)
+    s, ct = _sfx(w.dtype)
+    gf = _flat(g, w.dtype)
+    st = [_flat(a, w.dtype).copy() for a in state]
+    wf = _flat(w).copy()
+    sc = [ct(v) for v in optimizer_scalars(kind, w.dtype, t=t, **hp)]
+    getattr(lib(), "ko_%s_%s" % (kind, s))(ctypes.c_long(wf.size), *sc, _ptr(gf), *[_ptr(a) for a in st], _ptr(wf))
+    return [_shape_like(a, w.shape) for a in st], _shape_like(wf, w.shape)
+
+
 def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None, gemm=None):
     """Reference MLP step: ``x = relu.(w*x .+ b)`` per hidden layer (+ dropout with the given
     uniform buffers), ``nll`` on the last layer's scores; returns (loss, [dW1, db1, dW2, ...]).
