@@ -14,6 +14,7 @@
 // HBM roofline: forward 2*sizeof(T)*m*n; backward 3*sizeof(T)*m*n; fused nll backward 2*sizeof(T)*m*n.
 #pragma once
 #include "knet8_device.h"
+#include "knet8_runtime.h"
 
 namespace knet8 {
 
@@ -216,7 +217,14 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
   return v;
 }
 
-template <typename T, int TEAM, int E, bool VEC>
+// COLS: columns handled by one team, one after the other, with the loads of ALL of them issued up front.  With one
+// column per team every workgroup on the chip loads, then reduces, then stores at the same moments, and HBM idles
+// during the reduce/exp phases; with two, the second column's loads are still arriving while the first is reduced
+// and stored (a wave's loads return in order, so the first column's registers are ready while the second's loads
+// are in flight), which keeps the memory system busy end to end.
+// The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
+// fished out of the register that happens to hold it.
+template <typename T, int TEAM, int E, bool VEC, int COLS>
 __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
                                                                             T scale, T* loss) {
   constexpr int BT = TEAM == kWave ? 256 : TEAM;
@@ -225,72 +233,82 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void nll_col_kernel(int
   constexpr int NV = VEC ? Vec16<T>::N : 1;
   constexpr int ITEMS = E / NV;
   typedef typename Vec16<T>::type V;
-  __shared__ T lds_m[BT / kWave], lds_s[BT / kWave];
+  __shared__ T lds_m[COLS][BT / kWave], lds_s[COLS][BT / kWave];
   const int tl = threadIdx.x % TEAM;
-  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
-  const bool colok = col < n;
-  const long base = colok ? col * (long)m : 0;
-  const T* ac = a + base;
-  T* oc = out + base;
-  const int lab = colok ? labels[col] : 0;
+  const long col0 = ((long)blockIdx.x * TEAMS + threadIdx.x / TEAM) * COLS;
+  // lane tl owns accesses tl, tl+TEAM, ... of the m/NV accesses of a column: the first `cnt` of its ITEMS slots
+  const int macc = m / NV;  // VEC implies m % NV == 0
+  int cnt = (macc - tl + TEAM - 1) / TEAM;
+  cnt = cnt < 0 ? 0 : cnt;
 
-  T ra[E];
-  T alab = T(0);
-  bool own = false;
-  T mt = -INFINITY;
+  V rv[COLS][ITEMS];
+  int lab[COLS];
+  T alab[COLS];
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    const int r = (tl + i * TEAM) * NV;
-    const bool ok = colok && r < m;
-    V va = {};
-    if (ok) {
-      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
-      else va[0] = __builtin_nontemporal_load(ac + r);
-    }
+  for (int c = 0; c < COLS; c++) {
+    const long col = col0 + c;
+    const bool colok = col < n;
+    const T* ac = a + (colok ? col * (long)m : 0);
+    lab[c] = colok ? labels[col] : 0;
+    alab[c] = (tl == 0 && lab[c] > 0) ? ac[lab[c] - 1] : T(0);
 #pragma unroll
-    for (int e = 0; e < NV; e++) {
-      const T v = ok ? va[e] : T(-INFINITY);
-      ra[i * NV + e] = v;
-      mt = mt > v ? mt : v;
-      if (ok && r + e + 1 == lab) { alab = v; own = true; }
+    for (int i = 0; i < ITEMS; i++) {
+      if (colok && i < cnt) {
+        if (VEC) rv[c][i] = ld_stream(reinterpret_cast<const V*>(ac + (long)(tl + i * TEAM) * NV));
+        else rv[c][i][0] = __builtin_nontemporal_load(ac + (tl + i * TEAM));
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; e++) rv[c][i][e] = T(-INFINITY);
+      }
     }
   }
-  T st = T(0);
-  const T mref = mt == T(-INFINITY) ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
 #pragma unroll
-  for (int i = 0; i < E; i++) {
-    const T e = dev_exp(ra[i] - mref);
-    ra[i] = e;
-    st = st + e;
-  }
-  MaxSum<T> ms = {mt, st};
-  ms = ms_wave_reduce(ms);
-  if (NW > 1) {
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    if (lane == 0) { lds_m[wave] = ms.m; lds_s[wave] = ms.s; }
-    __syncthreads();
-    MaxSum<T> t = {lane < NW ? lds_m[lane] : T(-INFINITY), lane < NW ? lds_s[lane] : T(0)};
-    ms = ms_wave_reduce(t);
-  }
-  const T logS = dev_log(ms.s);
-  // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
-  const T f = (mt == T(-INFINITY) ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
-  if (own) loss[col] = -((alab - ms.m) - logS);
-  if (colok && lab == 0 && tl == 0) loss[col] = T(0);
+  for (int c = 0; c < COLS; c++) {
+    const long col = col0 + c;
+    const bool colok = col < n;
+    T* oc = out + (colok ? col * (long)m : 0);
+    T mt = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    const int r = (tl + i * TEAM) * NV;
-    const bool ok = colok && r < m;
-    if (!ok) continue;
-    V vo;
+    for (int i = 0; i < ITEMS; i++)
 #pragma unroll
-    for (int e = 0; e < NV; e++) {
-      const T p = ra[i * NV + e] * f;
-      const T dlp = (r + e + 1 == lab) ? -scale : T(0);
-      vo[e] = lab == 0 ? T(0) : dlp + p;
+      for (int e = 0; e < NV; e++) mt = mt > rv[c][i][e] ? mt : rv[c][i][e];
+    T st = T(0);
+    const T mref = mt == T(-INFINITY) ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++)
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        const T ex = dev_exp(rv[c][i][e] - mref);
+        rv[c][i][e] = ex;
+        st = st + ex;
+      }
+    MaxSum<T> ms = {mt, st};
+    ms = ms_wave_reduce(ms);
+    if (NW > 1) {
+      const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+      if (lane == 0) { lds_m[c][wave] = ms.m; lds_s[c][wave] = ms.s; }
+      __syncthreads();
+      MaxSum<T> t = {lane < NW ? lds_m[c][lane] : T(-INFINITY), lane < NW ? lds_s[c][lane] : T(0)};
+      ms = ms_wave_reduce(t);
     }
-    if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
-    else __builtin_nontemporal_store(vo[0], oc + r);
+    const T logS = dev_log(ms.s);
+    // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
+    const T f = (mt == T(-INFINITY) ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
+    if (colok && tl == 0) loss[col] = lab[c] > 0 ? -((alab[c] - ms.m) - logS) : T(0);
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      if (!(colok && i < cnt)) continue;
+      const int r = (tl + i * TEAM) * NV;
+      V vo;
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        const T p = rv[c][i][e] * f;
+        const T dlp = (r + e + 1 == lab[c]) ? -scale : T(0);
+        vo[e] = lab[c] == 0 ? T(0) : dlp + p;
+      }
+      if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+      else __builtin_nontemporal_store(vo[0], oc + r);
+    }
   }
 }
 
@@ -366,8 +384,19 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
   constexpr int TEAMS = BT / TEAM;
   const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS)), block(BT);
   if constexpr (Algo::kNll) {
-    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
-    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    // two columns per team (see nll_col_kernel) for long columns when there are enough of them to still give every CU a
+    // workgroup; for short columns (one wave each) more columns per wave only removes parallelism (measured: slower)
+    const bool two = vec && TEAM > kWave && E <= 32 && n >= 2 * (long)tuning(kTuneNumCUs);
+#define KNET8_NLL(COLS) do { \
+      const dim3 g((unsigned)((n + (long)TEAMS * COLS - 1) / ((long)TEAMS * COLS))); \
+      if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, COLS>), g, block, 0, stream, m, n, a, out, labels, scale, loss); \
+      else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, COLS>), g, block, 0, stream, m, n, a, out, labels, scale, loss); } while (0)
+    if constexpr (TEAM > kWave && E <= 32) {
+      if (two) KNET8_NLL(2); else KNET8_NLL(1);
+    } else {
+      KNET8_NLL(1);
+    }
+#undef KNET8_NLL
   } else {
     if (vec)
       hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
