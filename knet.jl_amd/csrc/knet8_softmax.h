@@ -86,13 +86,15 @@ __device__ __forceinline__ T team_reduce(T v, T* lds, Merge merge, T identity) {
 
 // ---- register-resident column kernel -----------------------------------------------------------------
 // TEAM lanes per column (64: four columns per 256-thread workgroup; 256 or 1024: the whole workgroup),
-// E elements of each held input per lane, VEC: 16-byte accesses (m % N == 0 and 16-byte aligned operands).
-template <typename T, typename Algo, int TEAM, int E, bool VEC>
-__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out,
-                                                                                const int* labels, T scale, T* loss) {
+// E elements of each held input per lane, VEC: 16-byte accesses (m % N == 0 and 16-byte aligned operands),
+// COLS: columns a team handles one after the other with the loads of all of them issued up front (an experiment in
+// hiding the reduce phase behind the next column's loads; the launcher explains why it always passes 1).
+template <typename T, typename Algo, int TEAM, int E, bool VEC, int COLS>
+__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
   // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
   // output pass, so the dependent chain is one memory round trip instead of two.
   constexpr bool kHold = Algo::kHoldA || (TEAM == kWave && E <= 16);
+  constexpr bool kTwo = Algo::kInputs == 2;
   constexpr int BT = TEAM == kWave ? 256 : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
@@ -100,96 +102,72 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel
   typedef typename Vec16<T>::type V;
   __shared__ T lds[BT / kWave];
   const int tl = threadIdx.x % TEAM;
-  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
-  const bool colok = col < n;       // only wave teams can be out of range, and those use no barriers
-  const long base = colok ? col * (long)m : 0;
-  const T* ac = a + base;
-  const T* bc = Algo::kInputs == 2 ? b + base : nullptr;
-  T* oc = out + base;
+  const long col0 = ((long)blockIdx.x * TEAMS + threadIdx.x / TEAM) * COLS;
+  // lane tl owns accesses tl, tl+TEAM, ... of the m/NV accesses of a column: the first `cnt` of its ITEMS slots
+  int cnt = (m / NV - tl + TEAM - 1) / TEAM;
+  cnt = cnt < 0 ? 0 : cnt;
 
-  T ra[kHold ? E : 1], rb[Algo::kInputs == 2 ? E : 1];
+  V ra[kHold ? COLS : 1][kHold ? ITEMS : 1], rb[kTwo ? COLS : 1][kTwo ? ITEMS : 1];
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    const int r = (tl + i * TEAM) * NV;
-    const bool ok = colok && r < m;
-    if (VEC) {
-      V va = {}, vb = {};
-      if (ok && kHold) va = ld_stream(reinterpret_cast<const V*>(ac + r));
-      if (ok && Algo::kInputs == 2) vb = ld_stream(reinterpret_cast<const V*>(bc + r));
+  for (int c = 0; c < COLS; c++) {
+    const long col = col0 + c;
+    const bool colok = col < n;  // only wave teams and the last of COLS can be out of range
+    const long base = colok ? col * (long)m : 0;
 #pragma unroll
-      for (int e = 0; e < NV; e++) {
-        if (kHold) ra[i * NV + e] = ok ? va[e] : T(0);
-        if (Algo::kInputs == 2) rb[i * NV + e] = ok ? vb[e] : T(0);
+    for (int i = 0; i < ITEMS; i++) {
+      const long r = (long)(tl + i * TEAM) * NV;
+      if (colok && i < cnt) {
+        if (VEC) {
+          if (kHold) ra[c][i] = ld_stream(reinterpret_cast<const V*>(a + base + r));
+          if (kTwo) rb[c][i] = ld_stream(reinterpret_cast<const V*>(b + base + r));
+        } else {
+          if (kHold) ra[c][i][0] = __builtin_nontemporal_load(a + base + r);
+          if (kTwo) rb[c][i][0] = __builtin_nontemporal_load(b + base + r);
+        }
       }
-    } else {
-      if (kHold) ra[i] = ok ? __builtin_nontemporal_load(ac + r) : T(0);
-      if (Algo::kInputs == 2) rb[i] = ok ? __builtin_nontemporal_load(bc + r) : T(0);
     }
   }
-
-  T mx = T(0);
-  if (Algo::kNeedMax) {
-    mx = -INFINITY;
+#pragma unroll
+  for (int c = 0; c < COLS; c++) {
+    const long col = col0 + c;
+    const bool colok = col < n;
+    const long base = colok ? col * (long)m : 0;
+    T mx = T(0);
+    if (Algo::kNeedMax) {
+      mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < ITEMS; i++)
+        if (colok && i < cnt) {
+#pragma unroll
+          for (int e = 0; e < NV; e++) mx = mx > ra[c][i][e] ? mx : ra[c][i][e];
+        }
+      mx = team_reduce<T, TEAM>(mx, lds, MaxFn(), T(-INFINITY));
+    }
+    T s = T(0);
 #pragma unroll
     for (int i = 0; i < ITEMS; i++)
+      if (colok && i < cnt) {
 #pragma unroll
-      for (int e = 0; e < NV; e++) {
-        const bool ok = colok && (tl + i * TEAM) * NV + e < m;
-        if (ok) mx = mx > ra[i * NV + e] ? mx : ra[i * NV + e];
+        for (int e = 0; e < NV; e++) s = s + Algo::term(kHold ? ra[c][i][e] : T(0), kTwo ? rb[c][i][e] : T(0), mx);
       }
-    mx = team_reduce<T, TEAM>(mx, lds, MaxFn(), T(-INFINITY));
-  }
-  T s = T(0);
+    s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
+    const T fin = Algo::finish(s);
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++)
-#pragma unroll
-    for (int e = 0; e < NV; e++) {
-      const bool ok = colok && (tl + i * TEAM) * NV + e < m;
-      if (ok) s = s + Algo::term(kHold ? ra[i * NV + e] : T(0), Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx);
-    }
-  s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
-  const T fin = Algo::finish(s);
-
-  int lab = 0;
-  T st = T(0);
-  if (Algo::kNll) {
-    lab = colok ? labels[col] : 0;
-    st = -scale;  // sum of dlp over the column: its single non-zero entry
-  }
-#pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    const int r = (tl + i * TEAM) * NV;
-    const bool ok = colok && r < m;
-    if (!ok) continue;
-    T o[NV];
-    V va = {};
-    if (!kHold) {
-      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
-      else va[0] = __builtin_nontemporal_load(ac + r);
-    }
-#pragma unroll
-    for (int e = 0; e < NV; e++) {
-      const T av = kHold ? ra[i * NV + e] : va[e];
-      T v = Algo::out(av, Algo::kInputs == 2 ? rb[i * NV + e] : T(0), mx, fin);
-      if (Algo::kNll) {
-        const bool hit = (r + e + 1 == lab);
-        if (hit) loss[col] = -v;
-        const T dlp = hit ? st : T(0);
-        const T p = dev_exp(v) * st;
-        v = lab == 0 ? T(0) : dlp - p;
+    for (int i = 0; i < ITEMS; i++) {
+      if (!(colok && i < cnt)) continue;
+      const long r = (long)(tl + i * TEAM) * NV;
+      V va = {};
+      if (!kHold) {
+        if (VEC) va = ld_stream(reinterpret_cast<const V*>(a + base + r));
+        else va[0] = __builtin_nontemporal_load(a + base + r);
       }
-      o[e] = v;
-    }
-    if (VEC) {
       V vo;
 #pragma unroll
-      for (int e = 0; e < NV; e++) vo[e] = o[e];
-      st_stream(reinterpret_cast<V*>(oc + r), vo);
-    } else {
-      __builtin_nontemporal_store(o[0], oc + r);
+      for (int e = 0; e < NV; e++) vo[e] = Algo::out(kHold ? ra[c][i][e] : va[e], kTwo ? rb[c][i][e] : T(0), mx, fin);
+      if (VEC) st_stream(reinterpret_cast<V*>(out + base + r), vo);
+      else __builtin_nontemporal_store(vo[0], out + base + r);
     }
   }
-  if (Algo::kNll && colok && lab == 0 && tl == 0) loss[col] = T(0);
 }
 
 // ---- fused nll + logsoftmax backward, register-resident, single reduction ---------------------------------
@@ -217,11 +195,7 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
   return v;
 }
 
-// COLS: columns handled by one team, one after the other, with the loads of ALL of them issued up front.  With one
-// column per team every workgroup on the chip loads, then reduces, then stores at the same moments, and HBM idles
-// during the reduce/exp phases; with two, the second column's loads are still arriving while the first is reduced
-// and stored (a wave's loads return in order, so the first column's registers are ready while the second's loads
-// are in flight), which keeps the memory system busy end to end.
+// COLS: as in softmax_col_kernel.
 // The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
 // fished out of the register that happens to hold it.
 template <typename T, int TEAM, int E, bool VEC, int COLS>
@@ -382,27 +356,27 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
                                T scale, T* loss) {
   constexpr int BT = TEAM == kWave ? 256 : TEAM;
   constexpr int TEAMS = BT / TEAM;
-  const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS)), block(BT);
+  const dim3 block(BT);
+  // COLS (columns per team, all loads issued up front) is always 1: measured on (32000,512), two columns per
+  // workgroup brought nothing for the fused nll kernel (23.0 us either way) and cost 8 % on the forward kernels --
+  // both phases are limited by HBM itself, not by the bubbles between them.
+  constexpr bool kCanTwo = false;
+  const bool two = false;
+#define KNET8_GRID(COLS) dim3((unsigned)((n + (long)TEAMS * COLS - 1) / ((long)TEAMS * COLS)))
   if constexpr (Algo::kNll) {
-    // two columns per team (see nll_col_kernel) for long columns when there are enough of them to still give every CU a
-    // workgroup; for short columns (one wave each) more columns per wave only removes parallelism (measured: slower)
-    const bool two = vec && TEAM > kWave && E <= 32 && n >= 2 * (long)tuning(kTuneNumCUs);
 #define KNET8_NLL(COLS) do { \
-      const dim3 g((unsigned)((n + (long)TEAMS * COLS - 1) / ((long)TEAMS * COLS))); \
-      if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, COLS>), g, block, 0, stream, m, n, a, out, labels, scale, loss); \
-      else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, COLS>), g, block, 0, stream, m, n, a, out, labels, scale, loss); } while (0)
-    if constexpr (TEAM > kWave && E <= 32) {
-      if (two) KNET8_NLL(2); else KNET8_NLL(1);
-    } else {
-      KNET8_NLL(1);
-    }
+      if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, out, labels, scale, loss); \
+      else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, out, labels, scale, loss); } while (0)
+    if constexpr (kCanTwo) { if (two) KNET8_NLL(2); else KNET8_NLL(1); } else { KNET8_NLL(1); }
 #undef KNET8_NLL
   } else {
-    if (vec)
-      hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
-    else
-      hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out, labels, scale, loss);
+#define KNET8_COL(COLS) do { \
+      if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, b, out); \
+      else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, b, out); } while (0)
+    if constexpr (kCanTwo) { if (two) KNET8_COL(2); else KNET8_COL(1); } else { KNET8_COL(1); }
+#undef KNET8_COL
   }
+#undef KNET8_GRID
 }
 
 template <typename T, typename Algo>
