@@ -234,14 +234,19 @@ def profile_pass(torch, K):
     K.libknet8().check()
 
 
-def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused):
+def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False):
+    """Forward + backward of an MLP through KnetArray and the tape.  graph=True: the step is captured once into a hipGraph
+    (labels resident on the device, loss kept on the device) and `steps` replays are timed."""
     rng = np.random.default_rng(0)
+    lib = K.libknet8()
+    old_stream = lib.stream
     params = []
     for i in range(len(sizes) - 1):
         params.append(K.Param(K.KnetArray((rng.standard_normal((sizes[i + 1], sizes[i])) * 0.01).astype(np.float32))))
         params.append(K.Param(K.KnetArray(np.zeros((sizes[i + 1], 1), np.float32))))
     x = K.KnetArray(rng.random((sizes[0], batch), dtype=np.float32))
     labels = rng.integers(1, sizes[-1] + 1, size=batch)
+    dlabels = K.KnetArray(labels.astype(np.int32))
     uni = [K.KnetArray(rng.random((sizes[i + 1], batch), dtype=np.float32)) for i in range(len(sizes) - 2)] if pdrop > 0 else None
 
     def loss():
@@ -252,18 +257,42 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused):
                 h = K.relu(h)
                 if pdrop > 0:
                     h = K.dropout(h, pdrop, uniform=uni[i // 2])
+        if graph:
+            return K.nll(h, dlabels, fused=True, count=batch)
         return K.nll(h, labels, fused=fused)
 
-    for _ in range(3):
-        K.diff(loss)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        J = K.diff(loss)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    K.libknet8().check()
-    return {"steps_per_sec": steps / dt, "ms_per_step": dt / steps * 1e3, "loss": float(K.value(J))}
+    try:
+        if graph:
+            def step():
+                J = K.diff(loss)
+                return [J.value] + [K.grad(J, p) for p in params]
+            g = K.capture(step)
+            for _ in range(3):
+                g.replay()
+            K.synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                g.replay()
+            K.synchronize()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            lossv = float(K.Array(g.outputs[0])[0])
+            del g
+        else:
+            for _ in range(3):
+                K.diff(loss)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                J = K.diff(loss)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            lossv = float(K.value(J))
+        lib.check()
+    finally:
+        lib.stream = old_stream
+    return {"steps_per_sec": steps / dt, "ms_per_step": dt / steps * 1e3, "loss": lossv}
 
 
 def cpu_side_table():
@@ -361,9 +390,14 @@ def main():
         torch.cuda.empty_cache()
         K.libknet8().fn["knet8_trim"]()
         line["mlp"] = {
-            "config1 MLP 784-64-10 batch 100 (fwd+bwd, tape, unfused nll)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, False),
-            "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, fused nll)":
+            "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager through the tape, step-by-step nll as in the reference)":
+                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, False),
+            "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager, fused nll)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, True),
+            "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
+                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
+            "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
+            "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),
         }
     line["cpu_baseline"] = cpu_baseline()
     if not args.no_extras:

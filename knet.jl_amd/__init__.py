@@ -6,7 +6,7 @@ Names, argument order, 1-based ``dims``/labels and error behaviour follow the re
 ``value`` as ``diff``/``grad``/``value``).  Importing the package loads the library; there is no CPU fallback.
 """
 from .libknet8 import libknet8, knet8, LIB_PATH
-from .karray import KnetArray, KnetPtr, Array, synchronize
+from .karray import KnetArray, KnetPtr, Array, synchronize, Graph, capture
 from .autograd import Param, diff, grad, value, recording
 from .activation import (relu, sigm, tanh, elu, selu, reluback, sigmback, tanhback, eluback, seluback,
                          gelu, hardsigmoid, hardswish, swish, tanh_, geluback, hardsigmoidback, hardswishback,

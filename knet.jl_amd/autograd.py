@@ -119,8 +119,11 @@ def diff(f):
         return Result(value(out), {})
     v = out.value
     if isinstance(v, KnetArray):
-        raise ValueError("diff() needs a scalar result")
-    out.outgrad = type(v)(1) if isinstance(v, (np.floating, float)) else 1.0
+        if v.length != 1:
+            raise ValueError("diff() needs a scalar result")
+        out.outgrad = 1.0  # a scalar kept on the device (1-element array): see nll(..., fused=True) with device labels
+    else:
+        out.outgrad = type(v)(1) if isinstance(v, (np.floating, float)) else 1.0
     for node in reversed(tape.nodes):
         if node.outgrad is None or node.back is None:
             continue

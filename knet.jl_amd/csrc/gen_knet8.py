@@ -401,6 +401,13 @@ KNET8_API void* knet8_event_create(void);
 KNET8_API void knet8_event_destroy(void* event);
 KNET8_API void knet8_event_record(void* event, hipStream_t stream);
 KNET8_API float knet8_event_elapsed(void* start, void* stop);
+/* hipGraph capture of a sequence of launches on a caller-created stream (no counterpart in the reference; for launch-bound
+   steps such as the MNIST MLP).  The sequence must have run once eagerly on that stream first; begin/end bracket the calls to
+   record, end returns an executable graph (NULL on failure), launch replays it. */
+KNET8_API int knet8_graph_begin(hipStream_t stream);
+KNET8_API void* knet8_graph_end(hipStream_t stream);
+KNET8_API int knet8_graph_launch(void* graph, hipStream_t stream);
+KNET8_API void knet8_graph_destroy(void* graph);
 /* last recorded failure as text (NULL if none); reading clears it */
 KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);

@@ -291,6 +291,36 @@ KNET8_API float knet8_event_elapsed(void* start, void* stop) {
   return ms;
 }
 
+// ---- hipGraph capture of a launch sequence ------------------------------------------------------------------
+// A backward step over small arrays is bound by launch latency, not bandwidth: capture the whole sequence once and
+// replay it with one call.  Capture needs a caller-created stream; everything the sequence needs
+// from the driver (pool blocks, reduction scratch, GEMM plans) should exist already, i.e. the sequence has run once
+// eagerly on the same stream (relaxed mode tolerates a late hipMalloc, but not the synchronisation a new GEMM plan needs).  No memset nodes are recorded: the library clears memory with fill kernels only.
+KNET8_API int knet8_graph_begin(hipStream_t stream) {
+  if (!stream) {
+    record_error("knet8_graph_begin: capture needs a stream created with knet8_stream_create");
+    return -1;
+  }
+  return ok(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture") ? 0 : -1;
+}
+
+KNET8_API void* knet8_graph_end(hipStream_t stream) {
+  hipGraph_t graph = nullptr;
+  if (!ok(hipStreamEndCapture(stream, &graph), "hipStreamEndCapture") || !graph) return nullptr;
+  hipGraphExec_t exec = nullptr;
+  const bool inst = ok(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+  (void)hipGraphDestroy(graph);
+  return inst ? exec : nullptr;
+}
+
+KNET8_API int knet8_graph_launch(void* graph, hipStream_t stream) {
+  return ok(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), stream), "hipGraphLaunch") ? 0 : -1;
+}
+
+KNET8_API void knet8_graph_destroy(void* graph) {
+  if (graph) ok(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)), "hipGraphExecDestroy");
+}
+
 KNET8_API const char* knet8_last_error(void) {
   std::lock_guard<std::mutex> lock(g_err_mutex);
   if (g_err.empty()) return nullptr;

@@ -13,6 +13,10 @@ from .libknet8 import libknet8
 
 _SUFFIX = {np.dtype(np.float32): "32", np.dtype(np.float64): "64"}
 
+# While a launch sequence is being captured into a graph, device blocks released by the garbage collector must not go
+# back to the pool: the graph keeps using their addresses.  capture() parks them here and the Graph object owns them.
+_PARKED = None
+
 
 class KnetPtr:
     """Owner of one device allocation (src/knetarrays/kptr.jl:10-15)."""
@@ -32,6 +36,10 @@ class KnetPtr:
 
     def __del__(self):
         if self._keep is None and self.ptr:
+            if _PARKED is not None:
+                _PARKED.append(self.ptr)
+                self.ptr = 0
+                return
             try:
                 libknet8().fn["knet8_free"](self.ptr)
             except Exception:
@@ -95,7 +103,7 @@ class KnetArray:
 
     @property
     def suffix(self):
-        return _SUFFIX[self.dtype]
+        return _SUFFIX.get(self.dtype)
 
     @property
     def ctype(self):
@@ -170,3 +178,62 @@ def synchronize():
     lib = libknet8()
     lib.fn["knet8_synchronize"](lib.stream)
     lib.check()
+
+
+class Graph:
+    """A captured launch sequence (hipGraph).  ``replay()`` launches it on the stream it was captured on; ``outputs`` is what the
+    captured function returned (device arrays whose contents every replay overwrites)."""
+
+    def __init__(self, handle, stream, outputs, parked):
+        self.handle, self.stream, self.outputs, self._parked = handle, stream, outputs, parked
+
+    def replay(self):
+        lib = libknet8()
+        if lib.fn["knet8_graph_launch"](self.handle, self.stream) != 0:
+            lib.check()
+            raise RuntimeError("graph launch failed")
+
+    def __del__(self):
+        try:
+            lib = libknet8()
+            lib.fn["knet8_synchronize"](self.stream)
+            lib.fn["knet8_graph_destroy"](self.handle)
+            for p in self._parked:
+                lib.fn["knet8_free"](p)
+        except Exception:
+            pass
+
+
+def capture(fn):
+    """Run ``fn()`` once eagerly (so that pool blocks, reduction scratch and GEMM plans exist), then once more under
+    stream capture, and return a ``Graph``.  ``fn`` must not synchronise with the host (no ``Array(x)``, no ``dims=:``
+    reductions, no host labels): it may only enqueue work."""
+    global _PARKED
+    lib = libknet8()
+    if lib.stream is None:
+        lib.stream = lib.fn["knet8_stream_create"]()
+    # Warm-up under the same parking rule as the capture itself, so that the pool ends up holding one block for every
+    # allocation of the sequence (blocks freed while parked are not recycled within the run).
+    warm = _PARKED = []
+    try:
+        fn()
+    finally:
+        _PARKED = None
+    lib.fn["knet8_synchronize"](lib.stream)
+    for p in warm:
+        lib.fn["knet8_free"](p)
+    lib.check()
+    parked = _PARKED = []
+    try:
+        if lib.fn["knet8_graph_begin"](lib.stream) != 0:
+            lib.check()
+        try:
+            out = fn()
+        finally:
+            handle = lib.fn["knet8_graph_end"](lib.stream)
+    finally:
+        _PARKED = None
+    if not handle:
+        lib.check()
+        raise RuntimeError("graph capture failed")
+    return Graph(handle, lib.stream, out, parked)

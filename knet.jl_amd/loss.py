@@ -65,25 +65,41 @@ def getindex(x, indices):
 
 
 @primitive
-def _nll_fused(scores, labels, dims=1):
-    """nll and its gradient wrt ``scores`` in one pass over the scores (``nll_logsoftmax_back_S``)."""
+def _nll_fused(scores, labels, dims=1, count=None):
+    """nll and its gradient wrt ``scores`` in one pass over the scores (``nll_logsoftmax_back_S``).
+
+    ``labels`` may be a host integer array (checked and uploaded, loss returned as a host scalar, as the reference's nll does) or
+    an Int32 ``KnetArray`` already on the device together with ``count`` = number of non-zero labels; in that case nothing
+    synchronises with the host and the loss comes back as a 1-element ``KnetArray`` (what a captured graph needs)."""
     if dims != 1 or scores.ndims != 2:
         raise NotImplementedError("fused nll needs a (classes, instances) matrix and dims=1")
     m, n = scores.dims
-    lab = np.asarray(labels).ravel(order="F")
-    if lab.size != n:
-        raise ValueError("DimensionMismatch")
-    if lab.size and (lab.min() < 0 or lab.max() > m):
-        raise IndexError("BoundsError")
-    count = int(np.count_nonzero(lab))
     T = scores.dtype.type
-    dlab = KnetArray(lab.astype(np.int32))
+    on_device = isinstance(labels, KnetArray)
+    if on_device:
+        if labels.dtype != np.int32 or labels.length != n:
+            raise ValueError("DimensionMismatch: device labels must be Int32 of length %d" % n)
+        dlab = labels
+        count = n if count is None else int(count)
+    else:
+        lab = np.asarray(labels).ravel(order="F")
+        if lab.size != n:
+            raise ValueError("DimensionMismatch")
+        if lab.size and (lab.min() < 0 or lab.max() > m):
+            raise IndexError("BoundsError")
+        count = int(np.count_nonzero(lab))
+        dlab = KnetArray(lab.astype(np.int32))
     dx = scores.similar()
     lossv = scores.similar((n,))
     scale = T(1) / T(count) if count else T(np.inf)
     knet8("nll_logsoftmax_back_%s" % scores.suffix, m, n, scores.ptr, dlab.ptr, scores.ctype(scale), dx.ptr, lossv.ptr)
-    total = R.reduce_op("sum", lossv)
-    loss = T(total) / T(count)
+    if on_device:
+        loss = scores.similar((1,))
+        knet8("sum_%s_21" % scores.suffix, n, lossv.ptr, n, 1, loss.ptr)
+        knet8("scal_%s" % scores.suffix, 1, scores.ctype(scale), loss.ptr)
+    else:
+        total = R.reduce_op("sum", lossv)
+        loss = T(total) / T(count)
 
     def back(dy):
         from .linalg import scal
@@ -93,14 +109,16 @@ def _nll_fused(scores, labels, dims=1):
     return loss, back
 
 
-def nll(scores, labels, dims=1, average=True, fused=False):
+def nll(scores, labels, dims=1, average=True, fused=False, count=None):
     """``nll(scores, labels; dims=1, average=true)`` (src/ops20/loss.jl:37-41).
 
     ``fused=False`` follows the reference step by step (logsoftmax, gather, sum); ``fused=True`` computes the loss
     and, when recording, the gradient with the single-pass kernel (same result within rounding).
     """
+    if isinstance(labels, KnetArray) and not fused:
+        raise TypeError("MethodError: nll takes host labels (an integer array), as in the reference; device labels need fused=True")
     if fused and average:
-        return _nll_fused(scores, labels, dims=dims)
+        return _nll_fused(scores, labels, dims=dims, count=count)
     indices = findindices(value(scores), labels, dims=dims)
     lp = getindex(logsoftmax(scores, dims=dims), indices)
     n = len(indices)
