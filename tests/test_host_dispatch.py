@@ -1,0 +1,97 @@
+"""Host-side logic on the CPU: which entry point the mirror of Knet's dispatchers picks, and with which arguments.
+
+Device arrays are faked (a KnetArray over a made-up pointer) and `knet8` is replaced by a recorder, so nothing is launched.
+The expectations restate src/knetarrays/reduction.jl:30-74 and src/knetarrays/binary.jl:13-149.
+"""
+import numpy as np
+import pytest
+
+
+@pytest.fixture
+def rec(knet, monkeypatch):
+    calls = []
+
+    def fake(fun, *args):
+        calls.append((fun,) + tuple(a if isinstance(a, (int, bytes)) else getattr(a, "value", a) for a in args))
+        return 0
+
+    import sys
+    for name, mod in list(sys.modules.items()):
+        if name.startswith("knet_jl_amd") and hasattr(mod, "knet8"):
+            monkeypatch.setattr(mod, "knet8", fake)
+
+    def arr(dims, dtype=np.float32):
+        return knet.KnetArray(dtype=dtype, dims=dims, _ptr=knet.KnetPtr(nbytes=4, ptr=0x1000, keep=object()))
+
+    def similar(self, dims=None, dtype=None):
+        return arr(self.dims if dims is None else dims, dtype or self.dtype)
+    monkeypatch.setattr(knet.KnetArray, "similar", similar)
+    return calls, arr
+
+
+def test_reduction_dispatch_follows_the_reference(knet, rec):
+    calls, arr = rec
+    x = arr((4096, 8192))
+    y = knet.reduce_op("sum", x, 1)          # vdims == 1 -> _21 with sy = stride(x,2), ny = size(x,2)   (reduction.jl:42-57)
+    assert y.dims == (1, 8192) and calls[-1][:1] + calls[-1][3:5] == ("sum_32_21", 4096, 8192) and calls[-1][1] == 4096 * 8192
+    y = knet.reduce_op("sum", x, 2)
+    assert y.dims == (4096, 1) and calls[-1][0] == "sum_32_21" and calls[-1][3:5] == (1, 4096)
+    x4 = arr((56, 56, 256, 64))
+    y = knet.reduce_op("sum", x4, [1, 2, 4])  # conv-bias gradient: one surviving dim -> _21 with sy = 3136, ny = 256
+    assert y.dims == (1, 1, 256, 1) and calls[-1][0] == "sum_32_21" and calls[-1][3:5] == (3136, 256)
+    x3 = arr((8, 16, 32), np.float64)
+    y = knet.reduce_op("maximum", x3, 2)      # vdims == ndims-1 -> _22 (nx, xd1, x, s1, s2, ny, y)       (reduction.jl:58-65)
+    assert y.dims == (8, 1, 32) and calls[-1][0] == "maximum_64_22" and calls[-1][1:3] == (4096, 15) and calls[-1][4:7] == (8, 128, 256)
+    n0 = len(calls)
+    y = knet.reduce_op("sum", arr((2, 3, 4, 5)), [1, 3])   # neither: one dim at a time                   (reduction.jl:66-73)
+    assert y.dims == (1, 3, 1, 5) and [c[0] for c in calls[n0:]] == ["sum_32_22", "sum_32_22"]
+    with pytest.raises(TypeError):
+        knet.reduce_op("sum", np.zeros((2, 2)))
+    with pytest.raises(ValueError):
+        knet.reduce_op("sum", x, 0)
+
+
+def test_broadcast_dispatch(knet, rec):
+    calls, arr = rec
+    x, b, r = arr((64, 100)), arr((64, 1)), arr((1, 100))
+    knet.broadcast_op("add", x, b)            # vector along dim 1 of the result: stride 1, length 64 -> _12
+    assert calls[-1][0] == "add_32_12" and calls[-1][1] == 6400 and calls[-1][3:5] == (1, 6400) and calls[-1][6:8] == (1, 64)
+    knet.broadcast_op("add", x, r)            # vector along dim 2: stride 64, length 100
+    assert calls[-1][0] == "add_32_12" and calls[-1][6:8] == (64, 100)
+    knet.broadcast_op("sub", b, x)            # vector first: operand order is kept
+    assert calls[-1][0] == "sub_32_12" and calls[-1][3:5] == (1, 64) and calls[-1][6:8] == (1, 6400)
+    knet.broadcast_op("mul", x, x)
+    assert calls[-1][0] == "mul_32_11"
+    knet.broadcast_op("mul", 2.0, x)
+    assert calls[-1][0] == "mul_32_01" and calls[-1][2] == 2.0
+    with pytest.raises(ValueError):
+        knet.broadcast_op("add", x, arr((100, 64)))
+    with pytest.raises(TypeError):
+        knet.broadcast_op("add", x, arr((64, 100), np.float64))
+    # unbroadcast: which dims get summed (AutoGrad's rule)
+    g = knet.unbroadcast(b, x)
+    assert g.dims == (64, 1) and calls[-1][0] == "sum_32_21" and calls[-1][3:5] == (1, 64)
+    g = knet.unbroadcast(arr((1, 1, 256, 1)), arr((56, 56, 256, 64)))
+    assert g.dims == (1, 1, 256, 1) and calls[-1][3:5] == (3136, 256)
+    assert knet.unbroadcast(x, x) is x
+
+
+def test_softmax_and_activation_dispatch(knet, rec):
+    calls, arr = rec
+    x = arr((32000, 512))
+    knet.logsoftmax(x, dims=1)
+    assert calls[-1][:3] == ("logsoftmax_32", 32000, 512)
+    knet.softmax(arr((10, 20, 30)), dims=[1, 2])          # leading dims collapse into the column length (TD4, softmax.jl:95-103)
+    assert calls[-1][:3] == ("softmax_32", 200, 30)
+    knet.logsoftmax(arr((7,)), dims=1)
+    assert calls[-1][:3] == ("logsoftmax_32", 7, 1)
+    knet.logsoftmax(x, dims=2)                             # non-leading: strided kernel (inner, d, outer)
+    assert calls[-1][:4] == ("logsoftmax_strided_32", 32000, 512, 1)
+    knet.logsoftmaxback(x, x, dims=1)
+    assert calls[-1][:3] == ("logsoftmaxback_32", 32000, 512)
+    knet.reluback(x, x)
+    assert calls[-1][:2] == ("reluback_32_11", 32000 * 512)
+    knet.geluback(x, x, x)
+    assert calls[-1][:2] == ("geluback_32_111", 32000 * 512)
+    with pytest.raises(ValueError):
+        knet.reluback(x, arr((5,)))
