@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
 
-A "step" is one pass of the isolated unary gradients of BASELINE config 2: reluback, sigmback, tanhback,
+A "step" is one pass of the isolated unary gradients of benchmark config 2: reluback, sigmback, tanhback,
 eluback, seluback on 2^28-element fp32 vectors and on 2^27-element fp64 vectors (ten launches, 3.22 GB of
 algorithmic traffic each: 2 reads + 1 write).  Inputs are synthetic (x, dy ~ N(0,1) drawn on the device with
 a fixed seed, y = f(x) from the library's forward kernels) and resident in HBM before the timed region.
@@ -375,7 +375,7 @@ def main():
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32+f64", "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: {relu,sigm,tanh,elu,selu}back on 2^28 fp32 and 2^27 fp64 vectors, "
+        "config": {"workload": "benchmark config 2: {relu,sigm,tanh,elu,selu}back on 2^28 fp32 and 2^27 fp64 vectors, "
                                "x,dy~N(0,1) seeded, y=f(x); 10 launches per step", "frac_of_hbm_peak": value / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "reluback_32_11 (ew_vec_kernel<float,2>)", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": RELUBACK_32_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": dom["bytes"],

@@ -1,4 +1,4 @@
-"""End-to-end backward step through KnetArray, the tape and the C ABI (BASELINE configs 1 and 5) against the oracle.
+"""End-to-end backward step through KnetArray, the tape and the C ABI (benchmark configs 1 and 5) against the oracle.
 
 Tolerances: the loss and the gradients go through GEMMs (hipBLASLt on the device, wide-accumulation loops or BLAS in
 the oracle), so they are compared norm-wise: ||g - g_ref|| <= 1e-4 ||g_ref|| in fp32 (accumulation order over k up to

@@ -106,7 +106,7 @@ def test_repeated_launches_reuse_the_scratch_correctly(knet):
 
 
 def test_config3_full_size(knet, oracle):
-    """BASELINE config 3: dy (4096,8192) over dims=1 and dims=2; NCHW bias gradient (56,56,256,64) -> (1,1,256,1)."""
+    """Benchmark config 3: dy (4096,8192) over dims=1 and dims=2; NCHW bias gradient (56,56,256,64) -> (1,1,256,1)."""
     rng = np.random.default_rng(25)
     x = rng.standard_normal((4096, 8192), dtype=np.float32)
     xd = knet.KnetArray(x)

@@ -139,7 +139,7 @@ def test_nll_known_answer_and_dims2(knet, oracle):
 
 
 def test_config4_full_size(knet, oracle):
-    """BASELINE config 4: logits (32000,512) ~ N(0,2), labels uniform, upstream 1/512; and (1000,4096)."""
+    """Benchmark config 4: logits (32000,512) ~ N(0,2), labels uniform, upstream 1/512; and (1000,4096)."""
     rng = np.random.default_rng(35)
     for C, N in [(32000, 512), (1000, 4096)]:
         scores = (rng.standard_normal((C, N), dtype=np.float32) * 2)
