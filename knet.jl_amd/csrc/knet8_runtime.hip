@@ -1,6 +1,7 @@
 // Host runtime of libknet8: error slot, per-stream reduction scratch, device-memory pool for KnetArray
 // storage, copies, stream/timer helpers and the hipBLASLt GEMM entry points.
 #include "knet8_runtime.h"
+#include "knet8_gemm_small.h"
 
 #include <hipblaslt/hipblaslt.h>
 
@@ -376,6 +377,11 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   if (m <= 0 || n <= 0) return 0;
   const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
   const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
+  if (gemm_is_small(m, n, k)) {
+    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    check_launch("gemm (small)");
+    return 0;
+  }
   const hipDataType dt = sizeof(T) == 4 ? HIP_R_32F : HIP_R_64F;
   const hipblasComputeType_t ct = sizeof(T) == 4 ? HIPBLAS_COMPUTE_32F : HIPBLAS_COMPUTE_64F;
   int dev = 0;
