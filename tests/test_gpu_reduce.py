@@ -131,3 +131,32 @@ def test_sum_gradient_through_the_tape(knet):
     J = knet.diff(lambda: knet.sum(p))
     assert float(knet.value(J)) == x.sum()
     assert np.array_equal(knet.Array(knet.grad(J, p)), np.ones((3, 4), np.float32))
+
+
+def test_random_shapes_cover_every_launch_plan(knet):
+    """Seeded sweep over the (sy,ny,no) and (s1,d,nb) views with exact integer data: every combination of workgroup size, split
+    factor, vector/scalar path and short-axis variant of the planner is hit many times."""
+    rng = np.random.default_rng(26)
+    fn = knet.libknet8().fn
+    sizes = [1, 2, 3, 4, 5, 7, 8, 15, 16, 31, 33, 63, 64, 65, 100, 127, 128, 255, 256, 257, 511, 1000, 1024, 4096, 5000, 30000, 200000]
+    done = 0
+    while done < 160:
+        a, b, c = (int(rng.choice(sizes)) for _ in range(3))
+        if a * b * c > 6_000_000 or a * b * c == 0:
+            continue
+        done += 1
+        dt, S = ((np.float32, "32"), (np.float64, "64"))[done % 2]
+        x = rng.integers(-3, 4, size=(a, b, c)).astype(dt)
+        xd = knet.KnetArray(x)
+        # run view: reduce axes 1 and 3
+        y = knet.KnetArray(np.full(b, 99, dt))
+        fn["sum_%s_21" % S](x.size, xd.ptr, a, b, y.ptr)
+        assert np.array_equal(knet.Array(y), x.sum(axis=(0, 2))), ("run", a, b, c)
+        # strided view: reduce axis 2
+        y2 = knet.KnetArray(np.full((a, c), 99, dt))
+        fn["sum_%s_22" % S](x.size, b - 1, xd.ptr, a, a * b, a * c, y2.ptr)
+        assert np.array_equal(knet.Array(y2), x.sum(axis=1)), ("strided", a, b, c)
+        fn["maximum_%s_22" % S](x.size, b - 1, xd.ptr, a, a * b, a * c, y2.ptr)
+        assert np.array_equal(knet.Array(y2), x.max(axis=1)), ("strided max", a, b, c)
+        assert fn["sum_%s_20" % S](x.size, xd.ptr) == x.sum()
+    knet.libknet8().check()

@@ -156,3 +156,30 @@ def test_config4_full_size(knet, oracle):
         got = knet.Array(knet.logsoftmaxback(knet.KnetArray(lsm), knet.KnetArray(dy), dims=1))
         assert close(got, oracle.logsoftmaxback(lsm, dy, dims=1))
     knet.libknet8().check()
+
+
+def test_random_column_shapes(knet, oracle):
+    """Seeded sweep over (m, n): every team size / capacity / vector-scalar combination of the column kernels, plus labels that are
+    first, last and skipped."""
+    rng = np.random.default_rng(36)
+    ms = [1, 2, 5, 17, 64, 100, 255, 256, 260, 1023, 1024, 1028, 3000, 4096, 4097, 8200, 16384, 16390, 20000, 32768, 32772, 40000, 65536, 65540]
+    for it in range(40):
+        m = int(rng.choice(ms))
+        n = int(rng.integers(1, 9)) if m > 4096 else int(rng.integers(1, 300))
+        dt = (np.float32, np.float64)[it % 2]
+        rtol = 1e-5 if dt == np.float32 else 1e-12
+        x = (rng.standard_normal((m, n)) * 3).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        labels = rng.integers(1, m + 1, size=n)
+        labels[0] = (1, m, 0)[it % 3]
+        xd = knet.KnetArray(x)
+        lsm = oracle.logsoftmax(x, dims=1)
+        assert close(knet.Array(knet.logsoftmax(xd, dims=1)), lsm, rtol), (m, n)
+        assert close(knet.Array(knet.softmax(xd, dims=1)), oracle.softmax(x, dims=1), rtol), (m, n)
+        assert close(knet.Array(knet.logsoftmaxback(knet.KnetArray(lsm), knet.KnetArray(dy), dims=1)), oracle.logsoftmaxback(lsm, dy, dims=1), rtol), (m, n)
+        if np.count_nonzero(labels):
+            p = knet.Param(xd)
+            J = knet.diff(lambda: knet.nll(p, labels, fused=True))
+            assert abs(float(knet.value(J)) - float(oracle.nll(x, labels))) <= rtol * abs(float(oracle.nll(x, labels))), (m, n)
+            assert close(knet.Array(knet.grad(J, p)), oracle.nll_back(x, labels), rtol), (m, n)
+    knet.libknet8().check()
