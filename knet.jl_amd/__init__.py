@@ -15,7 +15,7 @@ from .activation import (relu, sigm, tanh, elu, selu, reluback, sigmback, tanhba
 from .reduction import sum, prod, maximum, minimum, sumabs, sumabs2, maxabs, minabs, countnz, reduce_op
 from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
 from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback
-from .loss import nll, findindices, accuracy, getindex, ungetindex
+from .loss import nll, findindices, accuracy, getindex, ungetindex, bce, logistic
 from .dropout import dropout, dropback, dropout_, dropback_
 from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
 from .linalg import matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose

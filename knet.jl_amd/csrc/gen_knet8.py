@@ -261,6 +261,22 @@ def gen_elementwise():
         o.entry("scal_%s" % S, "void", [("int", "n"), (T, "alpha"), (T + "*", "x")],
                 "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, x, OpScal<%s>{alpha})" % (T, T, T, T),
                 "cublas%sscal_v2 with unit increment at src/knetarrays/linalg.jl:75-90" % ("S" if S == "32" else "D"))
+    o.decl.append("\n/* ---- binary cross entropy on raw scores with {0,1} labels already converted to T (oftype(scores,labels)).  No libknet8\n"
+                  "   counterpart: bce_S replaces the broadcast chain max.(0,s) .- y.*s .+ log.(1 .+ exp.(-abs.(s))) of src/ops20/loss.jl:107-111\n"
+                  "   (per-element losses, to be summed); bceback_S is its gradient wrt the scores times `scale`. ---- */")
+    s.append("template <typename T> struct OpBce { __device__ __forceinline__ T operator()(T sc, T y) const {\n"
+             "  const T a = sc > T(0) ? sc : T(0); const T b = y * sc; const T c = a - b; const T ab = sc < T(0) ? -sc : sc;\n"
+             "  const T e = kexp(-ab); const T f = T(1) + e; return c + klog(f); } };\n")
+    s.append("template <typename T> struct OpBceBack { T scale; __device__ __forceinline__ T operator()(T sc, T y) const {\n"
+             "  const T ab = sc < T(0) ? -sc : sc; const T e = kexp(-ab); const T q = e / (T(1) + e);\n"
+             "  const T step = sc > T(0) ? T(1) : T(0); const T sg = sc > T(0) ? T(1) : sc < T(0) ? T(-1) : T(0);\n"
+             "  const T g = (step - y) - sg * q; return scale * g; } };\n")
+    for T, S in TYPES:
+        o.entry("bce_%s" % S, "void", [("int", "n"), (T + "*", "scores"), (T + "*", "labels"), (T + "*", "loss")],
+                "launch_ew<%s, 2>(stream, n, scores, labels, (const %s*)nullptr, loss, OpBce<%s>())" % (T, T, T), "src/ops20/loss.jl:107-111")
+        o.entry("bceback_%s" % S, "void", [("int", "n"), (T, "scale"), (T + "*", "scores"), (T + "*", "labels"), (T + "*", "dscores")],
+                "launch_ew<%s, 2>(stream, n, scores, labels, (const %s*)nullptr, dscores, OpBceBack<%s>{scale})" % (T, T, T),
+                "the AutoGrad gradient of the same chain (max, abs, exp, log rules), src/ops20/loss.jl:107-111")
     o.decl.append("\n/* ---- fused optimizer updates (in place).  No libknet8 counterpart: each replaces the lmul!/axpy!/broadcast chain of one\n"
                   "   _update! method of src/train20/update.jl:513-570 (SGD itself is axpy_S).  Scalars are the T-rounded constants the\n"
                   "   Julia code forms: nlr = T(-lr), opg = T(1+gamma), omr = T(1-rho), omb1 = T(1-beta1), c1 = T(1-beta1^t) ... ---- */")

@@ -133,6 +133,41 @@ def _neg_div(total, n):
     return -total / T(n), (lambda dy: (-(T(dy) / T(n)), None))
 
 
+@primitive
+def _bce(scores, labels):
+    n = scores.length
+    y = KnetArray(np.asarray(labels).ravel(order="F").astype(scores.dtype))  # labels = oftype(scores, labels)
+    if y.length != n:
+        raise ValueError("DimensionMismatch")
+    l = scores.similar()
+    knet8("bce_%s" % scores.suffix, n, scores.ptr, y.ptr, l.ptr)
+    T = scores.dtype.type
+    total = T(R.reduce_op("sum", l))
+
+    def back(dy):
+        ds = scores.similar()
+        knet8("bceback_%s" % scores.suffix, n, scores.ctype(T(dy) / T(n)), scores.ptr, y.ptr, ds.ptr)
+        return (ds, None)
+    return total / T(n), back
+
+
+def bce(scores, labels, average=True):
+    """``bce(scores, labels; average=true)``: binary cross entropy on raw scores, labels in {0,1} (src/ops20/loss.jl:107-111)."""
+    labels = np.asarray(labels)
+    if not np.issubdtype(labels.dtype, np.integer) or labels.ndim != 1:
+        raise TypeError("MethodError: labels must be a vector of integers")
+    v = _bce(scores, labels)
+    if average:
+        return v
+    n = labels.size
+    return (value(v) * type(value(v))(n), n)
+
+
+def logistic(scores, labels, average=True):
+    """``logistic(scores, labels)``, labels in {-1,1}: ``bce(scores, (labels .+ 1) .÷ 2)`` (src/ops20/loss.jl:80-83)."""
+    return bce(scores, (np.asarray(labels) + 1) // 2, average=average)
+
+
 def accuracy(scores, labels, dims=1, average=True):
     """Ratio of instances whose labelled class has the largest score (src/ops20/loss.jl:52-62); as in the
     reference the scores are brought to the host for ``findmax``."""

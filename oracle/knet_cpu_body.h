@@ -347,6 +347,23 @@ void F(ko_gemm)(int ta, int tb, long m, long n, long k, const T *A, long lda, co
   }
 }
 
+/* bce(scores,labels): l = max.(0,s) .- y.*s .+ log.(1 .+ exp.(-abs.(s)))  -- src/ops20/loss.jl:107-111, labels already
+ * converted to T (oftype(scores,labels)); per-element losses.  Its gradient wrt s (sub-gradient 0 at s == 0 for max and abs,
+ * as AutoGrad's rules give): step(s) - y - sign(s)*e/(1+e), e = exp(-|s|), times the upstream scale. */
+void F(ko_bce)(long n, const T *s, const T *y, T *l) {
+  for (long i = 0; i < n; i++) {
+    T a = s[i] > 0 ? s[i] : (T)0; T b = y[i] * s[i]; T c = a - b; T ab = s[i] < 0 ? -s[i] : s[i];
+    T e = EXP(-ab); T f = (T)1 + e; l[i] = c + LOG(f);
+  }
+}
+void F(ko_bceback)(long n, T scale, const T *s, const T *y, T *ds) {
+  for (long i = 0; i < n; i++) {
+    T ab = s[i] < 0 ? -s[i] : s[i]; T e = EXP(-ab); T q = e / ((T)1 + e);
+    T step = s[i] > 0 ? (T)1 : (T)0; T sg = s[i] > 0 ? (T)1 : s[i] < 0 ? (T)-1 : (T)0;
+    T g = (step - y[i]) - sg * q; ds[i] = scale * g;
+  }
+}
+
 /* ---- optimizer updates, per element, in the order of the lmul!/axpy!/broadcast chains of
  * src/train20/update.jl:513-570 (lmul!(a,x): x = a*x; axpy!(a,x,y): y = y + a*x, product rounded first).
  * Scalars arrive already rounded to T, as the Julia code rounds them (alpha = T[alpha], T(p.eps), T(1 - beta^t)). */

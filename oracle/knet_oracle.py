@@ -255,6 +255,32 @@ def nll_back(scores, labels, dims=1):
     return _shape_like(dx, scores.shape)
 
 
+def bce(scores, labels, average=True):
+    """``bce(scores, labels)`` with {0,1} integer labels (src/ops20/loss.jl:107-111)."""
+    scores = np.asarray(scores)
+    s, _ = _sfx(scores.dtype)
+    sf, yf = _flat(scores), _flat(np.asarray(labels), scores.dtype)
+    l = np.empty_like(sf)
+    getattr(lib(), "ko_bce_%s" % s)(ctypes.c_long(sf.size), _ptr(sf), _ptr(yf), _ptr(l))
+    tot = reduce("sum", l)
+    return scores.dtype.type(tot / scores.dtype.type(sf.size)) if average else (tot, sf.size)
+
+
+def bce_back(scores, labels):
+    """Gradient of the averaged bce wrt the scores."""
+    scores = np.asarray(scores)
+    s, ct = _sfx(scores.dtype)
+    sf, yf = _flat(scores), _flat(np.asarray(labels), scores.dtype)
+    ds = np.empty_like(sf)
+    getattr(lib(), "ko_bceback_%s" % s)(ctypes.c_long(sf.size), ct(scores.dtype.type(1) / scores.dtype.type(sf.size)), _ptr(sf), _ptr(yf), _ptr(ds))
+    return _shape_like(ds, scores.shape)
+
+
+def logistic(scores, labels, average=True):
+    """``logistic(scores, labels)`` with {-1,1} labels: ``bce(scores, (labels .+ 1) .÷ 2)`` (src/ops20/loss.jl:80-83)."""
+    return bce(scores, (np.asarray(labels) + 1) // 2, average=average)
+
+
 def getents(x, ents):
     x = np.asarray(x)
     s, _ = _sfx(x.dtype)

@@ -183,3 +183,23 @@ def test_random_column_shapes(knet, oracle):
             assert abs(float(knet.value(J)) - float(oracle.nll(x, labels))) <= rtol * abs(float(oracle.nll(x, labels))), (m, n)
             assert close(knet.Array(knet.grad(J, p)), oracle.nll_back(x, labels), rtol), (m, n)
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_bce_and_logistic_value_and_gradient(knet, oracle, dt):
+    rng = np.random.default_rng(37)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    for n in (1, 10, 1000, 70001):
+        s = (rng.standard_normal(n) * 3).astype(dt)
+        y = rng.integers(0, 2, size=n)
+        p = knet.Param(knet.KnetArray(s))
+        J = knet.diff(lambda: knet.bce(p, y))
+        want = oracle.bce(s, y)
+        assert abs(float(knet.value(J)) - float(want)) <= rtol * abs(float(want)), n
+        assert close(knet.Array(knet.grad(J, p)), oracle.bce_back(s, y), rtol), n
+        assert float(knet.bce(knet.KnetArray(s), y)) == float(knet.logistic(knet.KnetArray(s), 2 * y - 1))  # test/ops20.jl:130
+    tot, cnt = knet.bce(knet.KnetArray(s), y, average=False)
+    assert cnt == n and abs(float(tot) / n - float(want)) <= 10 * rtol * abs(float(want))
+    with pytest.raises(TypeError):
+        knet.bce(knet.KnetArray(s), y.astype(np.float32))
+    knet.libknet8().check()

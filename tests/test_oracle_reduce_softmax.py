@@ -239,3 +239,26 @@ def test_mlp_backward_matches_finite_differences(oracle):
                 wm[k][i] -= h
                 g[i] = (oracle.mlp_backward(wp, x, labels, pdrop, uni)[0] - oracle.mlp_backward(wm, x, labels, pdrop, uni)[0]) / (2 * h)
             assert np.allclose(grads[k], g, atol=1e-7), (pdrop, k)
+
+
+def test_bce_and_logistic(oracle):
+    rng = np.random.default_rng(12)
+    s = rng.standard_normal(200) * 4
+    y01 = rng.integers(0, 2, size=200)
+    # the definition in the docstring: -(y log p + (1-y) log(1-p)), p = 1/(1+exp(-s))   (src/ops20/loss.jl:88-96)
+    p = 1 / (1 + np.exp(-s))
+    want = -(y01 * np.log(p) + (1 - y01) * np.log(1 - p)).mean()
+    assert abs(oracle.bce(s, y01) - want) < 1e-13
+    # bce(scores, labels) == logistic(scores, 2labels-1)   (test/ops20.jl:130)
+    assert oracle.bce(s, y01) == oracle.logistic(s, 2 * y01 - 1)
+    # log(1 + exp(-y s)) for +-1 labels (docstring of logistic)
+    ypm = 2 * y01 - 1
+    assert abs(oracle.logistic(s, ypm) - np.log1p(np.exp(-ypm * s)).mean()) < 1e-13
+    # stays finite for large scores
+    assert np.isfinite(oracle.bce(np.array([800.0, -800.0]), np.array([0, 1])))
+    # gradient: closed form (sigm(s) - y)/n and finite differences
+    g = oracle.bce_back(s, y01)
+    assert np.allclose(g, (p - y01) / 200, atol=1e-15)
+    assert np.allclose(g, _fd_grad(lambda v: np.array(oracle.bce(v, y01)), s, 1.0), atol=1e-8)
+    tot, cnt = oracle.bce(s, y01, average=False)
+    assert cnt == 200 and abs(tot / 200 - want) < 1e-13
