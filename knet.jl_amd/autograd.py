@@ -132,7 +132,13 @@ def diff(f):
             if parent is not None and g is not None:
                 parent.outgrad = addto(parent.outgrad, g)
         if node.param is None:
-            node.outgrad = None  # dead from here on: let the pool have it back (the reference's gcnode does this)
+            # Dead from here on: drop the gradient, the value and the closure that holds the saved activations, so their
+            # device blocks go back to the pool while the sweep is still running -- what the reference's tape-aware
+            # gcnode does after every node (src/autograd_gpu/gcnode.jl:63-93).
+            node.outgrad = None
+            node.back = None
+            if node is not out:
+                node.value = None
     return Result(v, {pid: n.outgrad for pid, n in tape.leaves.items()})
 
 

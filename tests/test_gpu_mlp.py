@@ -119,3 +119,32 @@ def test_pool_reuses_device_memory(knet):
     b = knet.KnetArray(np.zeros(100000, np.float32))
     fn["knet8_meminfo"](info)
     assert b.ptr == pa and info[3] == hits + 1  # same block handed out again without a new hipMalloc
+
+
+def test_backward_sweep_releases_intermediates(knet):
+    """After diff() only the parameters, the inputs and the parameter gradients are live: activations and upstream gradients went
+    back to the pool during the sweep (the role of gcnode in the reference)."""
+    import ctypes
+    import gc
+    fn = knet.libknet8().fn
+    info = (4 * ctypes.c_size_t)()
+    rng = np.random.default_rng(44)
+    gc.collect()
+    fn["knet8_meminfo"](info)
+    base = info[0]
+    ws = [knet.Param(knet.KnetArray((rng.standard_normal((256, 256)) * 0.1).astype(np.float32))) for _ in range(6)]
+    x = knet.KnetArray(rng.random((256, 512), dtype=np.float32))
+    labels = rng.integers(1, 257, size=512)
+
+    def loss():
+        h = x
+        for w in ws:
+            h = knet.relu(knet.matmul(w, h))
+        return knet.nll(h, labels, fused=True)
+    J = knet.diff(loss)
+    gc.collect()
+    fn["knet8_meminfo"](info)
+    live = info[0] - base
+    expect = 6 * 256 * 256 * 4 * 2 + 256 * 512 * 4   # weights + their gradients + the input batch
+    assert live <= expect + 64 * 1024, (live, expect)
+    assert all(knet.grad(J, w) is not None for w in ws)
