@@ -64,6 +64,7 @@ struct StreamScratch {
   unsigned* counters = nullptr;
   size_t ncounters = 0;
   void* scalar = nullptr;
+  std::vector<void*> retired;
   hipEvent_t t0 = nullptr, t1 = nullptr;
 };
 static std::mutex g_scratch_mutex;
@@ -78,16 +79,18 @@ static StreamScratch& scratch_of(hipStream_t stream) {
 Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   StreamScratch& s = scratch_of(stream);
+  // Buffers that have become too small are retired, not freed: launches already queued on the stream, and graphs
+  // captured on it, keep using their addresses.  Sizes grow geometrically, so the retired ones add up to less than
+  // the current one.
   if (s.partial_bytes < partial_bytes) {
-    // Work already queued on this stream may still use the old buffer: hipFree waits for the device.
-    if (s.partial) (void)hipFree(s.partial);
-    size_t want = partial_bytes < (size_t(1) << 20) ? (size_t(1) << 20) : partial_bytes + partial_bytes / 2;
+    if (s.partial) s.retired.push_back(s.partial);
+    size_t want = partial_bytes < (size_t(1) << 20) ? (size_t(1) << 20) : 2 * partial_bytes;
     s.partial = nullptr;
     s.partial_bytes = ok(hipMalloc(&s.partial, want), "hipMalloc(reduction partials)") ? want : 0;
   }
   if (s.ncounters < ncounters) {
-    if (s.counters) (void)hipFree(s.counters);
-    size_t want = ncounters < 4096 ? 4096 : ncounters + ncounters / 2;
+    if (s.counters) s.retired.push_back(s.counters);
+    size_t want = ncounters < 4096 ? 4096 : 2 * ncounters;
     s.counters = nullptr;
     s.ncounters = 0;
     if (ok(hipMalloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned)), "hipMalloc(reduction counters)") &&
