@@ -18,6 +18,12 @@
 
 namespace knet8 {
 
+// Workgroup size used when one wave owns a column (several columns per workgroup).
+#ifndef KNET8_WAVE_TEAM_BLOCK
+#define KNET8_WAVE_TEAM_BLOCK 256
+#endif
+constexpr int kWaveTeamBlock = KNET8_WAVE_TEAM_BLOCK;
+
 // exp for the softmax family.  fp32 uses the hardware 2^x unit (v_exp_f32, 1 ulp) on a pre-scaled argument: the
 // only extra error is the rounding of x*log2(e), about |x| * 6e-8 relative -- two orders of magnitude inside the
 // 1e-5 contract of these kernels -- and it costs 2 instructions instead of the ~20 of the correctly rounded expf.
@@ -90,12 +96,12 @@ __device__ __forceinline__ T team_reduce(T v, T* lds, Merge merge, T identity) {
 // COLS: columns a team handles one after the other with the loads of all of them issued up front (an experiment in
 // hiding the reduce phase behind the next column's loads; the launcher explains why it always passes 1).
 template <typename T, typename Algo, int TEAM, int E, bool VEC, int COLS>
-__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
+__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
   // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
   // output pass, so the dependent chain is one memory round trip instead of two.
   constexpr bool kHold = Algo::kHoldA || (TEAM == kWave && E <= 16);
   constexpr bool kTwo = Algo::kInputs == 2;
-  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
   constexpr int ITEMS = E / NV;
@@ -199,9 +205,9 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
 // The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
 // fished out of the register that happens to hold it.
 template <typename T, int TEAM, int E, bool VEC, int COLS>
-__global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
+__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
                                                                             T scale, T* loss) {
-  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NW = TEAM / kWave;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
@@ -224,6 +230,7 @@ __global__ __launch_bounds__(TEAM == kWave ? 256 : TEAM) void nll_col_kernel(int
     const bool colok = col < n;
     const T* ac = a + (colok ? col * (long)m : 0);
     lab[c] = colok ? labels[col] : 0;
+    if (lab[c] < 0 || lab[c] > m) lab[c] = 0;  // callers check labels on the host; an out-of-range one is skipped, never dereferenced
     alab[c] = (tl == 0 && lab[c] > 0) ? ac[lab[c] - 1] : T(0);
 #pragma unroll
     for (int i = 0; i < ITEMS; i++) {
@@ -306,7 +313,8 @@ __global__ __launch_bounds__(1024) void softmax_col_stream_kernel(long m, long n
   for (long r = threadIdx.x; r < m; r += 1024) s = s + Algo::term(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx);
   s = block_reduce<T, 1024 / kWave>(s, lds, AddFn(), T(0));
   const T fin = Algo::finish(s);
-  const int lab = Algo::kNll ? labels[col] : 0;
+  int lab = Algo::kNll ? labels[col] : 0;
+  if (lab < 0 || lab > m) lab = 0;
   const T st = -scale;
   for (long r = threadIdx.x; r < m; r += 1024) {
     T v = Algo::out(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx, fin);
@@ -354,7 +362,7 @@ inline void launch_softmax_strided(hipStream_t stream, long inner, long d, long 
 template <typename T, typename Algo, int TEAM, int E>
 inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, const T* a, const T* b, T* out, const int* labels,
                                T scale, T* loss) {
-  constexpr int BT = TEAM == kWave ? 256 : TEAM;
+  constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   const dim3 block(BT);
   // COLS (columns per team, all loads issued up front) is always 1: measured on (32000,512), two columns per
