@@ -15,7 +15,7 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def oracle():
     from oracle import knet_oracle
-    knet_oracle.lib()
+    knet_oracle.lib()  # builds oracle/libknet_oracle.so with gcc if it is missing
     return knet_oracle
 
 
@@ -23,4 +23,6 @@ def oracle():
 def knet():
     """The host-side mirror of the reference interface, backed by libknet8.so (HIP)."""
     import __graft_entry__ as ge
+    if not os.path.exists(os.path.join(ROOT, "knet.jl_amd", "lib", "libknet8.so")):
+        ge.build()  # nothing built yet (fresh checkout): cross-compile once; otherwise load what is there
     return ge.load_package()
