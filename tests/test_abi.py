@@ -76,3 +76,19 @@ def test_package_fails_loudly_without_the_library(tmp_path):
     lk = _load("lk_for_test2", "knet.jl_amd/libknet8.py")
     with pytest.raises(OSError):
         lk.LibKnet8(str(tmp_path / "libknet8.so"))
+
+
+def test_header_is_plain_c_and_links(built_lib, tmp_path):
+    """include/knet8.h must be usable from C (the boundary is a C ABI): compile and link a C translation unit against the library."""
+    src = tmp_path / "use_knet8.c"
+    src.write_text('#include "knet8.h"\n'
+                   'int main(void) {\n'
+                   '  void (*f)(int, float*, float*, float*, hipStream_t) = reluback_32_11_stream;\n'
+                   '  float (*g)(int, float*, hipStream_t) = sum_32_20_stream;\n'
+                   '  return (f != 0 && g != 0 && knet8_version() > 0) ? 0 : 1;\n'
+                   '}\n')
+    exe = tmp_path / "use_knet8"
+    libdir = os.path.dirname(built_lib)
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                           "-L", libdir, "-lknet8", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
+    assert subprocess.call([str(exe)]) == 0
