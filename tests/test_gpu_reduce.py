@@ -160,3 +160,33 @@ def test_random_shapes_cover_every_launch_plan(knet):
         assert np.array_equal(knet.Array(y2), x.max(axis=1)), ("strided max", a, b, c)
         assert fn["sum_%s_20" % S](x.size, xd.ptr) == x.sum()
     knet.libknet8().check()
+
+
+def test_ticket_protocol_under_repetition(knet):
+    """Split reductions publish partial results with write-through stores and a ticket (no release fence per workgroup).  Hammer it:
+    many back-to-back launches of shapes with different split factors, fresh data every few launches, every result exact."""
+    rng = np.random.default_rng(27)
+    fn = knet.libknet8().fn
+    shapes = [("strided", 4096, 2048), ("strided", 1024, 4099), ("run", 3136, 16, 64), ("run", 1000003, 1, 1), ("small", 10, 50000)]
+    data = {}
+    for rep in range(6):
+        for sh in shapes:
+            if sh[0] == "strided":
+                x = rng.integers(-3, 4, size=(sh[1], sh[2])).astype(np.float32)
+                data[sh] = (knet.KnetArray(x), x.sum(axis=1), (x.size, 1, sh[1]), sh[1])
+            elif sh[0] == "run":
+                x = rng.integers(-3, 4, size=(sh[1], sh[2], sh[3])).astype(np.float32)
+                data[sh] = (knet.KnetArray(x), x.sum(axis=(0, 2)), (x.size, sh[1], sh[2]), sh[2])
+            else:
+                x = rng.integers(-3, 4, size=(sh[1], sh[2])).astype(np.float32)
+                data[sh] = (knet.KnetArray(x), x.sum(axis=1), (x.size, 1, sh[1]), sh[1])
+        outs = []
+        for it in range(40):
+            for sh in shapes:
+                xd, want, (nx, sy, ny), nout = data[sh]
+                y = knet.KnetArray(dtype=np.float32, dims=(nout,))
+                fn["sum_32_21"](nx, xd.ptr, sy, ny, y.ptr)
+                outs.append((sh, y, want))
+        for sh, y, want in outs:
+            assert np.array_equal(knet.Array(y), want), (rep, sh)
+    knet.libknet8().check()
