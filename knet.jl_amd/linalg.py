@@ -18,22 +18,16 @@ def _size2(x, i):
 
 def gemm(transA, transB, alpha, A, B, beta, C):
     """``gemm!(transA, transB, alpha, A, B, beta, C)``."""
-    if transA == "N":
-        m, k = _size2(A, 1), _size2(A, 2)
-    else:
-        m, k = _size2(A, 2), _size2(A, 1)
-    if transB == "N":
-        n, kb = _size2(B, 2), _size2(B, 1)
-    else:
-        n, kb = _size2(B, 1), _size2(B, 2)
-    if k != kb or m != _size2(C, 1) or n != C.size(2):
+    a1, a2, b1, b2, c1, c2 = _size2(A, 1), _size2(A, 2), _size2(B, 1), _size2(B, 2), _size2(C, 1), C.size(2)
+    m, k = (a1, a2) if transA == "N" else (a2, a1)
+    kb, n = (b1, b2) if transB == "N" else (b2, b1)
+    if k != kb or m != c1 or n != c2:
         raise ValueError("DimensionMismatch: %r" % ((A.dims, B.dims, C.dims),))
     if A.dtype != B.dtype or A.dtype != C.dtype:
         raise TypeError("MethodError: element types differ")
     c = A.ctype
     lib = libknet8()
-    rc = lib.call("gemm_%s" % A.suffix, transA.encode(), transB.encode(), m, n, k, c(alpha), A.ptr, _size2(A, 1), B.ptr, _size2(B, 1),
-                  c(beta), C.ptr, _size2(C, 1))
+    rc = lib.call("gemm_%s" % A.suffix, transA.encode(), transB.encode(), m, n, k, c(alpha), A.ptr, a1, B.ptr, b1, c(beta), C.ptr, c1)
     if rc != 0:
         lib.check()
         raise RuntimeError("gemm failed")
