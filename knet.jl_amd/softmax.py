@@ -105,9 +105,12 @@ def softmaxback(y, dy, dims=None):
     return _bwd("softmaxback", y, dy, m, n)
 
 
+@primitive
 def logsumexp(x, dims=None):
-    """``xmax + log.(sum(exp.(x .- xmax)))`` (src/ops20/softmax.jl:65-70), from the logsoftmax kernel:
-    logsumexp = x - logsoftmax(x) at any one position of the reduced slice."""
+    """``xmax + log.(sum(exp.(x .- xmax)))`` (src/ops20/softmax.jl:65-70) with gradient ``dy .* exp.(x .- y)`` (``:72-74``).
+
+    Built on the column kernels: logsumexp = x - logsoftmax(x) at any position of the reduced slice, and
+    exp.(x .- y) is softmax(x)."""
     mn = _columns(x, dims)
     if mn is None:
         raise NotImplementedError("logsumexp over dims=%r" % (dims,))
@@ -117,6 +120,15 @@ def logsumexp(x, dims=None):
     diff = broadcast_op("sub", x, y)  # every row of a column holds the same value: take the maximum to pick one
     out = R.reduce_op("maximum", diff.reshape(m, n), 1)
     if dims is None:
-        return out.to_numpy().ravel()[0]
-    d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
-    return out.reshape(tuple(1 if (i + 1) in d else x.dims[i] for i in range(x.ndims)))
+        res = out.to_numpy().ravel()[0]
+    else:
+        d = sorted(set([dims] if isinstance(dims, int) else list(dims)))
+        res = out.reshape(tuple(1 if (i + 1) in d else x.dims[i] for i in range(x.ndims)))
+
+    def back(dy):
+        sm = _fwd("softmax", x, m, n)
+        if isinstance(dy, KnetArray):
+            g = broadcast_op("mul", sm.reshape(m, n), dy.reshape(1, n)) if n > 1 else broadcast_op("mul", float(dy.to_numpy().ravel()[0]), sm)
+            return (g.reshape(x.dims),)
+        return (broadcast_op("mul", dy, sm),)
+    return res, back

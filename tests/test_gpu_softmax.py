@@ -203,3 +203,24 @@ def test_bce_and_logistic_value_and_gradient(knet, oracle, dt):
     with pytest.raises(TypeError):
         knet.bce(knet.KnetArray(s), y.astype(np.float32))
     knet.libknet8().check()
+
+
+def test_logsumexp_value_and_gradient(knet, oracle):
+    rng = np.random.default_rng(38)
+    for shape, dims in [((10, 100), 1), ((257, 33), 1), ((3, 4, 5), [1, 2]), ((50,), None)]:
+        x = (rng.standard_normal(shape) * 2).astype(np.float32)
+        od = dims if dims is not None else tuple(range(1, len(shape) + 1))
+        od = tuple(od) if isinstance(od, list) else od
+        want = oracle.logsumexp(x, dims=od)
+        got = knet.logsumexp(knet.KnetArray(x), dims=dims)
+        got = knet.Array(got) if isinstance(got, knet.KnetArray) else np.float32(got)
+        assert np.allclose(got, want.reshape(np.shape(got)), rtol=1e-5, atol=1e-5), (shape, dims)
+        dy = rng.standard_normal(want.shape).astype(np.float32)
+        p = knet.Param(knet.KnetArray(x))
+        if dims is None:
+            J = knet.diff(lambda: knet.logsumexp(p))
+            wantg = oracle.logsumexpback(x, want, np.ones_like(want), dims=od)
+        else:
+            J = knet.diff(lambda: knet.sum(knet.mul(knet.logsumexp(p, dims=dims), knet.KnetArray(dy))))
+            wantg = oracle.logsumexpback(x, want, dy, dims=od)
+        assert close(knet.Array(knet.grad(J, p)), wantg, 2e-5), (shape, dims)
