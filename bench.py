@@ -178,6 +178,17 @@ def extras(torch, K):
     dxs = [y.similar() for y in ys[:4]]
     res["dropback_32 (4096,2048)"] = time_kernel(
         K, torch, lambda i: (lambda: K.knet8("dropback_32", n5, ctypes.c_float(0.5), ys[i].ptr, ys[i].ptr, dys[i].ptr, dxs[i % 4].ptr)), 12 * n5, list(range(40)))
+    # config 5 fused layer passes: bias + relu + dropout forward (z, u -> y) and dropback + reluback + bias gradient (dy, y -> dz, db)
+    zs = dys
+    us = [device_randn(torch, K, n5, f32, 230 + i) for i in range(4)]
+    bias = device_randn(torch, K, 4096, f32, 229)
+    db = bias.similar()
+    res["biasreludrop_32 (4096,2048)"] = time_kernel(
+        K, torch, lambda i: (lambda: K.knet8("biasreludrop_32", 4096, 2048, ctypes.c_float(0.5), zs[i].ptr, bias.ptr, us[i % 4].ptr)),
+        12 * n5 + 4 * 4096, list(range(40)))
+    res["dropreluback_biasgrad_32 (4096,2048)"] = time_kernel(
+        K, torch, lambda i: (lambda: K.knet8("dropreluback_biasgrad_32", 4096, 2048, ctypes.c_float(0.5), dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr, db.ptr)),
+        12 * n5 + 4 * 4096, list(range(40)))
     K.libknet8().check()
     return res
 
@@ -234,9 +245,10 @@ def profile_pass(torch, K):
     K.libknet8().check()
 
 
-def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False):
+def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=False):
     """Forward + backward of an MLP through KnetArray and the tape.  graph=True: the step is captured once into a hipGraph
-    (labels resident on the device, loss kept on the device) and `steps` replays are timed."""
+    (labels resident on the device, loss kept on the device) and `steps` replays are timed.  layers=True: each hidden layer's
+    bias add, relu and dropout (and their gradients plus the bias gradient) run as one fused launch each way."""
     rng = np.random.default_rng(0)
     lib = K.libknet8()
     old_stream = lib.stream
@@ -252,6 +264,9 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False):
     def loss():
         h = x
         for i in range(0, len(params), 2):
+            if layers and i < len(params) - 2:
+                h = K.bias_act(K.matmul(params[i], h), params[i + 1], act="relu", pdrop=pdrop, uniform=uni[i // 2] if pdrop > 0 else None)
+                continue
             h = K.add(K.matmul(params[i], h), params[i + 1])
             if i < len(params) - 2:
                 h = K.relu(h)
@@ -340,7 +355,26 @@ def cpu_baseline():
             ko.back11(back, dy, y)
             total_s += time.perf_counter() - t0
             total_bytes += 3 * n * x.itemsize
+    # The same loops over 16 equal slices in 16 threads (ctypes drops the interpreter lock during the call): what the port reaches
+    # on the host share of a one-GPU box when every core streams; a restatement's figure, not Knet's, whose Array path is one thread.
+    from concurrent.futures import ThreadPoolExecutor
+    threads = 16
+    x = rng.standard_normal(1 << 25).astype(np.float32)
+    dy = rng.standard_normal(1 << 25).astype(np.float32)
+    cut = np.linspace(0, x.size, threads + 1).astype(np.int64)
+    par_bytes, par_s = 0, 0.0
+    with ThreadPoolExecutor(threads) as pool:
+        for back, fwd in OPS:
+            y = ko.unary(fwd, x)
+            parts = [(dy[a:b], y[a:b]) for a, b in zip(cut[:-1], cut[1:])]
+            list(pool.map(lambda p: ko.back11(back, p[0][:1024], p[1][:1024]), parts))
+            t0 = time.perf_counter()
+            list(pool.map(lambda p: ko.back11(back, p[0], p[1]), parts))
+            par_s += time.perf_counter() - t0
+            par_bytes += 3 * x.size * x.itemsize
     return {"value": total_bytes / total_s * 1e-9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "all_cores": {"value": par_bytes / par_s * 1e-9, "unit": "GB/s", "cores": threads,
+                          "sample": "the five fp32 *back loops on 2^25 elements cut into 16 slices, one thread each"},
             "sample": "the five *back loops of oracle/knet_cpu.c (gcc -O2, no contraction) on 2^25 fp32 and 2^24 fp64 elements, one pass each, "
                       "timed through ctypes including the output allocation; Knet's CPU Array path for these ops is single-threaded broadcast"}
 
@@ -395,9 +429,12 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager, fused nll)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, True),
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
+            "config1 same graph with fused bias+relu layers": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),
+            "config5 same graph with fused bias+relu+dropout layers":
+                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True, layers=True),
         }
     line["cpu_baseline"] = cpu_baseline()
     if not args.no_extras:

@@ -8,7 +8,7 @@ Names, argument order, 1-based ``dims``/labels and error behaviour follow the re
 from .libknet8 import libknet8, knet8, LIB_PATH
 from .karray import KnetArray, KnetPtr, Array, synchronize, Graph, capture
 from .autograd import Param, diff, grad, value, recording
-from .activation import (relu, sigm, tanh, elu, selu, reluback, sigmback, tanhback, eluback, seluback,
+from .activation import (bias_act, relu, sigm, tanh, elu, selu, reluback, sigmback, tanhback, eluback, seluback,
                          gelu, hardsigmoid, hardswish, swish, tanh_, geluback, hardsigmoidback, hardswishback,
                          swishback, tanh_back, eluback21, seluback21, sigmback21, relu_kw, relu_kw_back,
                          unary_op, back11_op, back111_op)

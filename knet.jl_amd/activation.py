@@ -8,6 +8,8 @@ keyword arguments -> ``relu_S_1`` / ``reluback_S_1``).  In Julia these are reach
 """
 import math
 
+import numpy as np
+
 from .autograd import primitive
 from .karray import KnetArray
 from .libknet8 import knet8
@@ -130,3 +132,50 @@ def relu_kw(x, max_value=math.inf, negative_slope=0, threshold=0):
     c = x.ctype
     knet8("relu_%s_1" % x.suffix, y.length, c(max_value), c(negative_slope), c(threshold), x.ptr, y.ptr)
     return y, (lambda dy: (relu_kw_back(x, y, dy, max_value, negative_slope, threshold),))
+
+
+# ---- fused dense-layer passes ---------------------------------------------------------------------------
+
+_FUSED_ACTS = ("relu", "sigm", "tanh", "elu", "selu")
+
+
+@primitive
+def bias_act(z, b, act="relu", pdrop=0.0, uniform=None):
+    """``dropout(f.(z .+ b), pdrop)`` for a matrix ``z`` (m,n) and a bias ``b`` (m,1) in one pass each way.
+
+    The reference runs the forward as ``add_S_12``, ``F_S`` and ``dropout_S`` (src/knetarrays/binary.jl:61-95,
+    src/ops20_gpu/activation.jl:17-29, src/ops20_gpu/dropout.jl:12-21) and the backward as ``dropback_S``,
+    ``Fback_S_11`` and ``sum(dz;dims=2)``; ``biasF_S`` / ``biasreludrop_S`` and ``Fback_biasgrad_S`` /
+    ``dropreluback_biasgrad_S`` do the same arithmetic per element in one kernel.  Dropout (relu only) needs the
+    uniform buffer; like ``dropout`` it is applied only while recording."""
+    _check(z)
+    if act not in _FUSED_ACTS:
+        raise ValueError("bias_act: no fused kernel for %r" % (act,))
+    if z.ndims != 2 or not isinstance(b, KnetArray) or b.dtype != z.dtype or b.length != z.dims[0]:
+        raise ValueError("DimensionMismatch: bias_act needs z (m,n) and b (m,1), got %r and %r" % (z.dims, getattr(b, "dims", None)))
+    from .autograd import recording
+    m, n = z.dims
+    drop = pdrop > 0 and recording()
+    if drop and (act != "relu" or not 0 < pdrop < 1):
+        raise ValueError("bias_act: dropout is fused for relu and 0 < pdrop < 1 only")
+    c = z.ctype
+    if drop:
+        if uniform is None:
+            raise ValueError("bias_act: dropout needs the uniform buffer")
+        y = uniform.copy() if isinstance(uniform, KnetArray) else KnetArray(np.asarray(uniform, dtype=z.dtype))
+        if y.length != z.length:
+            raise ValueError("DimensionMismatch: uniform buffer %r vs %r" % (y.dims, z.dims))
+        y = y.reshape(z.dims)
+        knet8("biasreludrop_%s" % z.suffix, m, n, c(pdrop), z.ptr, b.ptr, y.ptr)
+    else:
+        y = z.similar()
+        knet8("bias%s_%s" % (act, z.suffix), m, n, z.ptr, b.ptr, y.ptr)
+
+    def back(dy):
+        dz, db = y.similar(), b.similar()
+        if drop:
+            knet8("dropreluback_biasgrad_%s" % z.suffix, m, n, c(pdrop), dy.ptr, y.ptr, dz.ptr, db.ptr)
+        else:
+            knet8("%sback_biasgrad_%s" % (act, z.suffix), m, n, dy.ptr, y.ptr, dz.ptr, db.ptr)
+        return dz, db
+    return y, back

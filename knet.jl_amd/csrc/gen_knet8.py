@@ -69,6 +69,8 @@ BINARY_OPS = [
     ("min", "return xi < yi ? xi : yi;", "src/libknet8/ops.jl:94"),
 ]
 
+FUSED_ACTS = ["relu", "sigm", "tanh", "elu", "selu"]
+
 # Two-input gradients NAME_S_11(n, dy, y, dx): xi = dy, yi = y.
 BACK11_OPS = [
     ("reluback", "return yi > T(0) ? xi : T(0);", "src/ops20/activation.jl:27, src/libknet8/ops.jl:118"),
@@ -161,6 +163,7 @@ class Out:
 PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_elementwise.h"
 #include "../knet8_reduce.h"
+#include "../knet8_fused.h"
 #include "../knet8_softmax.h"
 #include "../knet8_index.h"
 #include "../knet8_transpose.h"
@@ -289,6 +292,34 @@ def gen_elementwise():
             ptrs = arrays + ["(%s*)nullptr" % T] * (4 - len(arrays))
             o.entry("%s_%s" % (name, S), "void", params,
                     "launch_update<%s, %d, %du>(stream, n, %s, Opt_%s<%s>{%s})" % (T, len(arrays), mask, ", ".join(ptrs), name, T, ", ".join(scalars)), cite)
+    o.decl.append("\n/* ---- fused dense-layer passes on an m x n column-major matrix with bias b of shape (m,1).  No libknet8 counterpart:\n"
+                  "   biasF_S replaces add_S_12 followed by F_S (src/knetarrays/binary.jl:61-95, src/ops20_gpu/activation.jl:17-29);\n"
+                  "   biasreludrop_S also applies dropout! with y holding U[0,1) on entry (src/ops20/dropout.jl:45-58);\n"
+                  "   Fback_biasgrad_S replaces Fback_S_11 followed by sum(dz;dims=2) (src/ops20_gpu/activation.jl:30-37,\n"
+                  "   src/knetarrays/reduction.jl:21-77); dropreluback_biasgrad_S starts from the dropout output (dropback!,\n"
+                  "   src/ops20/dropout.jl:60-71).  y and dz carry the same bits as the separate launches. ---- */")
+    s.append("template <typename T, typename Op> struct BiasAct { __device__ __forceinline__ T operator()(T zb, T) const { return Op()(zb); } };\n")
+    s.append("template <typename T> struct BiasReluDrop { T p, q; __device__ __forceinline__ T operator()(T zb, T u) const {\n"
+             "  const T r = Op_relu<T>()(zb); return u > p ? r / q : T(0); } };\n")
+    s.append("// dropback! then reluback from the dropout output alone: the output is positive exactly where the element was kept and the relu active\n"
+             "template <typename T> struct OpDropReluBack { T q; __device__ __forceinline__ T operator()(T dy, T y) const { return y > T(0) ? dy / q : T(0); } };\n")
+    for act in FUSED_ACTS:
+        for T, S in TYPES:
+            o.entry("bias%s_%s" % (act, S), "void", [("int", "m"), ("int", "n"), (T + "*", "z"), (T + "*", "b"), (T + "*", "y")],
+                    "launch_bias_act<%s, false>(stream, m, n, z, b, y, BiasAct<%s, Op_%s<%s> >())" % (T, T, act, T),
+                    "add_S_12 + %s_S, src/knetarrays/binary.jl:61-95, src/ops20_gpu/activation.jl:17-29" % act)
+            o.entry("%sback_biasgrad_%s" % (act, S), "void",
+                    [("int", "m"), ("int", "n"), (T + "*", "dy"), (T + "*", "y"), (T + "*", "dz"), (T + "*", "db")],
+                    "launch_actback_biasgrad<%s>(stream, m, n, dy, y, dz, db, Op11_%sback<%s>())" % (T, act, T),
+                    "%sback_S_11 + sum_S_21, src/ops20_gpu/activation.jl:30-37, src/knetarrays/reduction.jl:21-77" % act)
+    for T, S in TYPES:
+        o.entry("biasreludrop_%s" % S, "void", [("int", "m"), ("int", "n"), (T, "p"), (T + "*", "z"), (T + "*", "b"), (T + "*", "y")],
+                "launch_bias_act<%s, true>(stream, m, n, z, b, y, BiasReluDrop<%s>{p, %s(1) - p})" % (T, T, T),
+                "add_S_12 + relu_S + dropout_S, src/ops20/dropout.jl:45-58")
+        o.entry("dropreluback_biasgrad_%s" % S, "void",
+                [("int", "m"), ("int", "n"), (T, "p"), (T + "*", "dy"), (T + "*", "y"), (T + "*", "dz"), (T + "*", "db")],
+                "launch_actback_biasgrad<%s>(stream, m, n, dy, y, dz, db, OpDropReluBack<%s>{%s(1) - p})" % (T, T, T),
+                "dropback_S + reluback_S_11 + sum_S_21, src/ops20/dropout.jl:60-71")
     return o
 
 

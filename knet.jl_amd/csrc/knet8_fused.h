@@ -1,0 +1,162 @@
+// Fused layer kernels for y = f(w*x .+ b) with b of shape (m,1) on an m x n column-major matrix.
+//
+// The reference runs this as separate launches: bias add (src/knetarrays/binary.jl:61-95 -> add_S_12),
+// activation (src/ops20_gpu/activation.jl:17-29), dropout (src/ops20_gpu/dropout.jl:12-21) on the way forward;
+// dropback, activation gradient (src/ops20_gpu/activation.jl:30-37) and the bias gradient sum(dz;dims=2)
+// (src/knetarrays/reduction.jl:21-77) on the way back.  Each fused kernel here makes one pass instead:
+//   forward   y = f(z + b[i])            [then dropout]   2 streams (3 with the uniform buffer) instead of 6 (9)
+//   backward  dz = f'(dy, y), db = sum_j dz               3 streams instead of 7 (10 with dropback)
+// Every element goes through the same rounded operations as the separate launches, so dz and y are bit-identical
+// to the chain; db differs from the chain's sum only by summation order.
+#pragma once
+#include "knet8_reduce.h"
+
+namespace knet8 {
+
+// ---- forward -----------------------------------------------------------------------------------------
+// F(T zb [, T u]) maps the biased pre-activation (and, with DROP, the uniform draw found in y) to the output.
+template <typename T, typename F, bool DROP, int NV>
+__global__ __launch_bounds__(kEwBlock) void bias_act_kernel(long nitems, const T* z, const T* b, unsigned m, T* y, F f) {
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i >= nitems) return;
+  const long e = i * NV;
+  const unsigned r = (unsigned)e % m;  // sizes are 32-bit ints at the ABI; m % NV == 0 on the vector path, so the NV elements share a column
+  if (NV > 1) {
+    typedef typename Vec16<T>::type V;
+    const V a = ld_stream(reinterpret_cast<const V*>(z + e));
+    const V bv = *reinterpret_cast<const V*>(b + r);
+    V u, o;
+    if (DROP) u = ld_stream(reinterpret_cast<const V*>(y + e));
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      const T zb = a[k] + bv[k];
+      o[k] = f(zb, DROP ? u[k] : T(0));
+    }
+    st_stream(reinterpret_cast<V*>(y + e), o);
+  } else {
+    const T zb = z[e] + b[r];
+    y[e] = f(zb, DROP ? y[e] : T(0));
+  }
+}
+
+template <typename T, bool DROP, typename F>
+inline void launch_bias_act(hipStream_t stream, long m, long n, const T* z, const T* b, T* y, F f) {
+  if (m <= 0 || n <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  const bool vec = (m % N == 0) && aligned16(z) && aligned16(b) && aligned16(y);
+  const long nitems = vec ? m * n / N : m * n;
+  const long grid = (nitems + kEwBlock - 1) / kEwBlock;
+  if (vec)
+    hipLaunchKernelGGL((bias_act_kernel<T, F, DROP, N>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nitems, z, b, (unsigned)m, y, f);
+  else
+    hipLaunchKernelGGL((bias_act_kernel<T, F, DROP, 1>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nitems, z, b, (unsigned)m, y, f);
+}
+
+// ---- backward ----------------------------------------------------------------------------------------
+// Row tile of 64*NV consecutive i's per workgroup, the BT/64 waves take columns j = j0+wave, j0+wave+NW, ...;
+// P workgroups split the columns of a tile and the last one to finish adds their partial sums (same ticket
+// scheme as the strided reduction).  F(dy, y) is the element gradient.  dz may be dy or y itself (each element is read
+// before the same lane writes it).
+template <typename T, typename F, int NV, int BT, int U>
+__global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const T* yv, long m, long n, long jchunk, unsigned P, T* dz, T* __restrict__ db,
+                                                              T* partial, unsigned* counters, F f) {
+  constexpr int TILE = kWave * NV;
+  constexpr int NW = BT / kWave;
+  __shared__ T lds[NW][TILE];
+  __shared__ unsigned flag;
+  const long at = blockIdx.x / P;
+  const unsigned p = blockIdx.x % P;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const long a0 = at * TILE + (long)lane * NV;
+  const bool live = a0 < m;
+  const long j0 = (long)p * jchunk;
+  long j1 = j0 + jchunk;
+  if (j1 > n) j1 = n;
+  T acc[NV];
+#pragma unroll
+  for (int e = 0; e < NV; e++) acc[e] = T(0);
+  if (live) {
+    for (long j = j0 + wave; j < j1; j += NW * U) {
+      T g[U][NV];
+#pragma unroll
+      for (int q = 0; q < U; q++) {
+        const long jj = j + q * NW;
+        if (jj < j1) {
+          const long off = jj * m + a0;
+          if (NV > 1) {
+            typedef typename Vec16<T>::type V;
+            const V d = ld_stream(reinterpret_cast<const V*>(dy + off));
+            const V o = ld_stream(reinterpret_cast<const V*>(yv + off));
+            V r;
+#pragma unroll
+            for (int e = 0; e < NV; e++) { r[e] = f(d[e], o[e]); g[q][e] = r[e]; }
+            st_stream(reinterpret_cast<V*>(dz + off), r);
+          } else {
+            const T r = f(__builtin_nontemporal_load(dy + off), __builtin_nontemporal_load(yv + off));
+            g[q][0] = r;
+            __builtin_nontemporal_store(r, dz + off);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < NV; e++) g[q][e] = T(0);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < U; q++)
+#pragma unroll
+        for (int e = 0; e < NV; e++) acc[e] = acc[e] + g[q][e];
+    }
+  }
+  if (P > 1) {
+#pragma unroll
+    for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+    __syncthreads();
+    if (threadIdx.x < TILE) {
+      T r = T(0);
+#pragma unroll
+      for (int w = 0; w < NW; w++) r = r + lds[w][threadIdx.x];
+      st_coherent(partial + (at * P + p) * TILE + threadIdx.x, r);
+    }
+    if (!last_block_ticket(counters + at, P, &flag)) return;
+#pragma unroll
+    for (int e = 0; e < NV; e++) acc[e] = T(0);
+    strided_walk<T, RedSum<T>, NV, false, NW, U>(partial + at * P * TILE + lane * NV, TILE, 0, P, wave, acc);
+    if (threadIdx.x == 0) st_coherent(counters + at, 0u);
+  }
+#pragma unroll
+  for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+  __syncthreads();
+  const long a = at * TILE + threadIdx.x;
+  if (threadIdx.x < TILE && a < m) {
+    T r = T(0);
+#pragma unroll
+    for (int w = 0; w < NW; w++) r = r + lds[w][threadIdx.x];
+    db[a] = r;
+  }
+}
+
+template <typename T, typename F>
+inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T* dy, const T* y, T* dz, T* db, F f) {
+  if (m <= 0) return;
+  constexpr int N = Vec16<T>::N;
+  const bool vec = (m % N == 0) && aligned16(dy) && aligned16(y) && aligned16(dz);
+  const int nv = vec ? N : 1;
+  const long tile = (long)kWave * nv;
+  const long atiles = ceil_div(m, tile);
+  unsigned P = n > 0 ? plan_parts(atiles, n, 32) : 1;
+  long jchunk = ceil_div(n, P);
+  P = (unsigned)ceil_div(n, jchunk > 0 ? jchunk : 1);
+  if (P < 1) P = 1;
+  Workspace ws = {nullptr, nullptr};
+  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)atiles * P * tile, (size_t)atiles);
+  const dim3 grid((unsigned)(atiles * P));
+  T* partial = static_cast<T*>(ws.partial);
+  const bool big = jchunk >= 64;
+#define KNET8_ABG(NV, BT, U) \
+  hipLaunchKernelGGL((actback_biasgrad_kernel<T, F, NV, BT, U>), grid, dim3(BT), 0, stream, dy, y, m, n, jchunk, P, dz, db, partial, ws.counters, f)
+  if (vec) { if (big) KNET8_ABG(N, 1024, 2); else KNET8_ABG(N, 256, 4); }
+  else     { if (big) KNET8_ABG(1, 1024, 2); else KNET8_ABG(1, 256, 4); }
+#undef KNET8_ABG
+}
+
+}  // namespace knet8

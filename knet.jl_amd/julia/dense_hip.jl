@@ -1,0 +1,50 @@
+# Optional fused dense-layer primitive on top of the library's biasF_S / Fback_biasgrad_S entry points.  NOT EXECUTED here.
+# The reference has no such op: a layer `relu.(w*x .+ b)` runs add_S_12, relu_S (and dropout_S) as separate launches
+# (src/knetarrays/binary.jl:61-95, src/ops20_gpu/activation.jl:17-29, src/ops20_gpu/dropout.jl:12-21) and its gradient as
+# dropback_S, reluback_S_11 and sum(dz;dims=2).  A model opts in by calling `biasact(relu, w*x, b)` instead of
+# `relu.(w*x .+ b)`; everything else (KnetArray, @diff, the op tables) is untouched.
+
+using .LibKnet8: @knet8
+import AutoGrad: @primitive
+
+for (T, S) in ((Float32, 32), (Float64, 64)), f in (:relu, :sigm, :tanh, :elu, :selu)
+    fwd, bwd = "bias$(f)_$S", "$(f)back_biasgrad_$S"
+    @eval begin
+        function biasact(::typeof($f), z::KnetArray{$T,2}, b::KnetArray{$T})
+            m, n = size(z); @assert length(b) == m
+            y = similar(z)
+            @knet8($fwd, (Cint, Cint, Ptr{$T}, Ptr{$T}, Ptr{$T}), m, n, z, b, y)
+            return y
+        end
+        # returns (dz, db); the tape asks for the two gradients one after the other, so the pair is cached on dy
+        function biasactback(::typeof($f), dy::KnetArray{$T,2}, y::KnetArray{$T,2}, b::KnetArray{$T})
+            m, n = size(y)
+            dz = similar(y); db = similar(b)
+            @knet8($bwd, (Cint, Cint, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}), m, n, dy, y, dz, db)
+            return dz, db
+        end
+    end
+end
+
+const _biasact_cache = IdDict{Any,Any}()   # dy => (dz, db), emptied when the second gradient is taken
+function _biasact_grads(f, dy, y, b)
+    get!(() -> biasactback(f, dy, y, b), _biasact_cache, dy)
+end
+@primitive biasact(f, z, b),dy,y  nothing  _biasact_grads(f, dy, y, b)[1]  (g = _biasact_grads(f, dy, y, b)[2]; delete!(_biasact_cache, dy); g)
+
+# relu + dropout in one pass each way: y holds U[0,1) on entry (rand!(y)), as for dropout! (src/ops20/dropout.jl:45-58).
+for (T, S) in ((Float32, 32), (Float64, 64))
+    @eval begin
+        function biasreludrop!(p, z::KnetArray{$T,2}, b::KnetArray{$T}, y::KnetArray{$T,2})
+            m, n = size(z)
+            @knet8($("biasreludrop_$S"), (Cint, Cint, $T, Ptr{$T}, Ptr{$T}, Ptr{$T}), m, n, $T(p), z, b, y)
+            return y
+        end
+        function dropreluback_biasgrad(p, dy::KnetArray{$T,2}, y::KnetArray{$T,2}, b::KnetArray{$T})
+            m, n = size(y)
+            dz = similar(y); db = similar(b)
+            @knet8($("dropreluback_biasgrad_$S"), (Cint, Cint, $T, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}), m, n, $T(p), dy, y, dz, db)
+            return dz, db
+        end
+    end
+end

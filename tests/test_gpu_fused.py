@@ -1,0 +1,158 @@
+"""GPU parity of the fused dense-layer kernels (bias + activation [+ dropout]; activation gradient + bias gradient)
+against the oracle's separate loops, through the C ABI.
+
+The fused kernels apply the same rounded operations per element as the separate launches, so y and dz are compared
+bit for bit with the oracle's chain (<= 2 ulp where the activation calls exp/tanh); db is a sum over n columns and is
+compared at 1e-5 relative to the sum of magnitudes (the bound a reordered fp summation obeys).
+"""
+import numpy as np
+import pytest
+
+from gpu_util import bits_equal, ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+ACTS = ["relu", "sigm", "tanh", "elu", "selu"]
+SHAPES = [(1, 1), (3, 5), (10, 100), (64, 100), (257, 33), (256, 1), (1000, 4096), (4096, 2048), (300, 5000), (4100, 130), (8, 70000)]
+
+
+def sfx(dt):
+    return "32" if dt == np.float32 else "64"
+
+
+def chain_forward(oracle, act, z, b, p=0.0, u=None):
+    zb = oracle.add_bias(z, b)
+    r = oracle.unary(act, zb)
+    return oracle.dropout(r, p, u) if u is not None else r, r
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("act", ACTS)
+def test_bias_act_forward_and_backward(knet, oracle, act, dt):
+    rng = np.random.default_rng(51)
+    S = sfx(dt)
+    for m, n in SHAPES:
+        if dt == np.float64 and m * n > 2_000_000:
+            continue
+        z = rng.standard_normal((m, n)).astype(dt)
+        b = rng.standard_normal((m, 1)).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        want_y, _ = chain_forward(oracle, act, z, b)
+        zd, bd, dyd = knet.KnetArray(z), knet.KnetArray(b), knet.KnetArray(dy)
+        yd = zd.similar()
+        knet.knet8("bias%s_%s" % (act, S), m, n, zd.ptr, bd.ptr, yd.ptr)
+        got_y = knet.Array(yd)
+        if act == "relu":
+            assert bits_equal(got_y, want_y), (act, m, n)
+        else:
+            # elu/selu subtract 1 from exp: the 2 ulp are measured at the magnitude of the libm result
+            scale = np.maximum(np.abs(want_y), 1.0) if act in ("elu", "selu") else None
+            assert ulp_diff(got_y, want_y, scale=scale).max(initial=0) <= 2, (act, m, n)
+        # backward from the oracle's y so that both sides start from the same bits
+        yd = knet.KnetArray(want_y)
+        dzd, dbd = zd.similar(), bd.similar()
+        knet.knet8("%sback_biasgrad_%s" % (act, S), m, n, dyd.ptr, yd.ptr, dzd.ptr, dbd.ptr)
+        want_dz = oracle.back11(act + "back", dy, want_y)
+        assert bits_equal(knet.Array(dzd), want_dz), (act, m, n)
+        ref = want_dz.astype(np.float64).sum(axis=1, keepdims=True)
+        mag = np.abs(want_dz).astype(np.float64).sum(axis=1, keepdims=True)
+        tol = 1e-5 if dt == np.float32 else 1e-13
+        assert np.all(np.abs(knet.Array(dbd).astype(np.float64) - ref) <= tol * np.maximum(mag, 1e-30)), (act, m, n)
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_bias_relu_dropout_matches_the_three_launch_chain(knet, oracle, dt):
+    rng = np.random.default_rng(52)
+    S = sfx(dt)
+    for m, n in SHAPES:
+        if dt == np.float64 and m * n > 2_000_000:
+            continue
+        for p in (0.5, 0.1):
+            z = rng.standard_normal((m, n)).astype(dt)
+            b = rng.standard_normal((m, 1)).astype(dt)
+            u = rng.random((m, n)).astype(dt)
+            dy = rng.standard_normal((m, n)).astype(dt)
+            want_y, r = chain_forward(oracle, "relu", z, b, p, u)
+            zd, bd, dyd = knet.KnetArray(z), knet.KnetArray(b), knet.KnetArray(dy)
+            yd = knet.KnetArray(u)
+            knet.knet8("biasreludrop_%s" % S, m, n, zd.ctype(p), zd.ptr, bd.ptr, yd.ptr)
+            assert bits_equal(knet.Array(yd), want_y), (m, n, p)
+            want_dz = oracle.back11("reluback", oracle.dropback(p, r, want_y, dy), r)
+            dzd, dbd = zd.similar(), bd.similar()
+            knet.knet8("dropreluback_biasgrad_%s" % S, m, n, zd.ctype(p), dyd.ptr, yd.ptr, dzd.ptr, dbd.ptr)
+            assert bits_equal(knet.Array(dzd), want_dz), (m, n, p)
+            ref = want_dz.astype(np.float64).sum(axis=1, keepdims=True)
+            mag = np.abs(want_dz).astype(np.float64).sum(axis=1, keepdims=True)
+            tol = 1e-5 if dt == np.float32 else 1e-13
+            assert np.all(np.abs(knet.Array(dbd).astype(np.float64) - ref) <= tol * np.maximum(mag, 1e-30)), (m, n, p)
+    knet.libknet8().check()
+
+
+def test_fused_kernels_on_special_values_and_empty(knet, oracle):
+    from gpu_util import SPECIALS
+    sp = np.array(SPECIALS, np.float32)
+    m = 8
+    y = np.tile(sp, (m, 1)).astype(np.float32)            # (8, 16): every special value in every row
+    dy = np.tile(sp[::-1], (m, 1)).astype(np.float32)
+    for act in ACTS:
+        yd, dyd = knet.KnetArray(y), knet.KnetArray(dy)
+        dzd, dbd = yd.similar(), knet.KnetArray(np.zeros((m, 1), np.float32))
+        knet.knet8("%sback_biasgrad_32" % act, m, y.shape[1], dyd.ptr, yd.ptr, dzd.ptr, dbd.ptr)
+        with np.errstate(all="ignore"):
+            assert bits_equal(knet.Array(dzd), oracle.back11(act + "back", dy, y)), act
+    # relu outputs (never negative, possibly NaN, +0 or Inf) through dropout with every second element dropped
+    r = np.abs(y)
+    u = np.zeros_like(r)
+    u[:, ::2] = 0.75
+    u[::2, :] = 1 - u[::2, :] - 0.25 * (u[::2, :] == 0)
+    with np.errstate(all="ignore"):
+        ypos = oracle.dropout(r, 0.5, u)
+        want = oracle.back11("reluback", oracle.dropback(0.5, r, ypos, dy), r)
+    yd, dyd = knet.KnetArray(ypos), knet.KnetArray(dy)
+    dzd, dbd = yd.similar(), knet.KnetArray(np.zeros((m, 1), np.float32))
+    knet.knet8("dropreluback_biasgrad_32", m, y.shape[1], np.float32(0.5), dyd.ptr, yd.ptr, dzd.ptr, dbd.ptr)
+    assert bits_equal(knet.Array(dzd), want)
+    # n == 0: the bias gradient of an empty batch is zero; m == 0: nothing is touched
+    dbd = knet.KnetArray(np.full((5, 1), 7.0, np.float32))
+    e = knet.KnetArray(np.zeros((5, 0), np.float32))
+    knet.knet8("reluback_biasgrad_32", 5, 0, e.ptr, e.ptr, e.ptr, dbd.ptr)
+    assert np.all(knet.Array(dbd) == 0)
+    knet.knet8("biasrelu_32", 5, 0, e.ptr, dbd.ptr, e.ptr)
+    knet.knet8("reluback_biasgrad_32", 0, 5, e.ptr, e.ptr, e.ptr, dbd.ptr)
+    knet.libknet8().check()
+
+
+def test_fused_layers_in_the_mlp_match_oracle(knet, oracle):
+    rng = np.random.default_rng(53)
+    sizes = [33, 40, 24, 17, 9]
+    ws = []
+    for i in range(4):
+        ws += [rng.standard_normal((sizes[i + 1], sizes[i])) * 0.3, rng.standard_normal((sizes[i + 1], 1)) * 0.1]
+    x = rng.random((33, 50))
+    labels = rng.integers(0, 10, size=50)
+    uni = [rng.random((sizes[i + 1], 50)) for i in range(3)]
+    loss_ref, grads_ref = oracle.mlp_backward(ws, x, labels, pdrop=0.5, uniforms=uni)
+    params = [knet.Param(knet.KnetArray(w)) for w in ws]
+    xd = knet.KnetArray(x)
+
+    def predict():
+        h = xd
+        for i in range(0, 6, 2):
+            h = knet.bias_act(knet.matmul(params[i], h), params[i + 1], act="relu", pdrop=0.5, uniform=uni[i // 2])
+        return knet.add(knet.matmul(params[6], h), params[7])
+    J = knet.diff(lambda: knet.nll(predict(), labels, fused=True))
+    assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-12 * abs(float(loss_ref))
+    for p, g in zip(params, grads_ref):
+        got = knet.Array(knet.grad(J, p)).astype(np.float64)
+        assert np.linalg.norm(got - g) <= 1e-11 * np.linalg.norm(g)
+    # outside diff() dropout is the identity
+    out = knet.Array(predict())
+    h = x
+    for i in range(0, 6, 2):
+        h = oracle.unary("relu", oracle.add_bias(oracle.gemm(ws[i], h), ws[i + 1]))
+    want = oracle.add_bias(oracle.gemm(ws[6], h), ws[7])
+    assert np.allclose(out, want, rtol=1e-12, atol=1e-12)
+    with pytest.raises(ValueError):
+        knet.bias_act(knet.KnetArray(np.zeros((4, 3))), knet.KnetArray(np.zeros((5, 1))))
+    knet.libknet8().check()
