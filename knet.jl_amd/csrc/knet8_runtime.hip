@@ -338,7 +338,7 @@ KNET8_API int knet8_version(void) { return 100; }
 KNET8_API int knet8_tune(int key, int value) {
   if (key < 0 || key >= kTuneCount) return -1;
   const int old = g_tune[key];
-  if (value > 0) g_tune[key] = value;
+  if (value >= 0) g_tune[key] = value;  // 0 restores the default
   return old;
 }
 

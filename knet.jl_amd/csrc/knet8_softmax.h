@@ -9,7 +9,8 @@
 // once and the result written once: the column is loaded with 16-byte vectors, reduced (max, then sum)
 // with wave64 butterflies (+ LDS across waves), transformed and stored.  Team size follows the column
 // length: one wave (m <= 4096), a 256-thread workgroup (m <= 16384) or a 1024-thread workgroup
-// (m <= 65536); longer columns fall back to a three-pass streaming kernel.
+// (m <= 65536 in fp32, half of each limit when two inputs are held or in fp64); longer columns fall back to a
+// two-pass streaming kernel.
 //
 // HBM roofline: forward 2*sizeof(T)*m*n; backward 3*sizeof(T)*m*n; fused nll backward 2*sizeof(T)*m*n.
 #pragma once
@@ -293,39 +294,137 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
   }
 }
 
-// ---- streaming fallback for very long columns ----------------------------------------------------------
-// One 1024-thread workgroup per column; the inputs are read once per pass (max, sum, output).
-template <typename T, typename Algo>
+// ---- streaming fallback for columns too long to hold in registers ----------------------------------------
+// One 1024-thread workgroup per column, two passes with 16-byte accesses and U of them in flight per lane.
+// Pass 1 reduces: for the max-based algorithms max and sum(exp(x - max)) are carried together as a pair that is
+// rescaled whenever the running max grows (one exp per element plus one per batch of U accesses), so x is read once
+// for both; the other algorithms just sum their terms.  Pass 2 reads the inputs again (cache hits for the part of the
+// column still resident in L2 / the memory-side cache) and writes the result.  HBM roofline: between the resident
+// kernels' bytes and one extra read of every input.
+template <typename T>
+__device__ __forceinline__ void maxsum_merge(T& m, T& s, T m2, T s2) {
+  const T mm = m > m2 ? m : m2;
+  const T s1 = (m == mm) ? s : s * dev_exp(m - mm);    // equal maxima (both -inf included): no rescale, no inf - inf
+  const T s3 = (m2 == mm) ? s2 : s2 * dev_exp(m2 - mm);
+  m = mm;
+  s = s1 + s3;
+}
+
+template <typename T, typename Algo, bool VEC>
 __global__ __launch_bounds__(1024) void softmax_col_stream_kernel(long m, long n, const T* a, const T* b, T* out, const int* labels,
                                                                   T scale, T* loss) {
-  __shared__ T lds[1024 / kWave];
+  constexpr int NV = VEC ? Vec16<T>::N : 1;
+  constexpr int U = 4;
+  constexpr bool kTwo = Algo::kInputs == 2;
+  constexpr long STEP = 1024L * NV;
+  typedef typename Vec16<T>::type V;
+  __shared__ T lds[2][1024 / kWave];
   const long col = blockIdx.x;
   const T* ac = a + col * m;
-  const T* bc = Algo::kInputs == 2 ? b + col * m : nullptr;
+  const T* bc = kTwo ? b + col * m : nullptr;
   T* oc = out + col * m;
-  T mx = T(0);
-  if (Algo::kNeedMax) {
-    mx = -INFINITY;
-    for (long r = threadIdx.x; r < m; r += 1024) { const T v = ac[r]; mx = mx > v ? mx : v; }
-    mx = block_reduce<T, 1024 / kWave>(mx, lds, MaxFn(), T(-INFINITY));
+  const T ninf = T(-INFINITY);
+  T mx = Algo::kNeedMax ? ninf : T(0), s = T(0);
+  for (long r0 = (long)threadIdx.x * NV; r0 < m; r0 += STEP * U) {
+    T va[U][NV], vb[U][NV];
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long r = r0 + q * STEP;
+      if (r < m) {
+        if (VEC) {
+          const V t = *reinterpret_cast<const V*>(ac + r);
+#pragma unroll
+          for (int e = 0; e < NV; e++) va[q][e] = t[e];
+          if (kTwo) {
+            const V t2 = *reinterpret_cast<const V*>(bc + r);
+#pragma unroll
+            for (int e = 0; e < NV; e++) vb[q][e] = t2[e];
+          }
+        } else {
+          va[q][0] = ac[r];
+          if (kTwo) vb[q][0] = bc[r];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < NV; e++) { va[q][e] = Algo::kNeedMax ? ninf : T(0); vb[q][e] = T(0); }
+      }
+    }
+    if (Algo::kNeedMax) {
+      T bm = mx;
+#pragma unroll
+      for (int q = 0; q < U; q++)
+#pragma unroll
+        for (int e = 0; e < NV; e++) bm = va[q][e] > bm ? va[q][e] : bm;
+      if (bm > mx) { s = s * dev_exp(mx - bm); mx = bm; }
+#pragma unroll
+      for (int q = 0; q < U; q++)
+#pragma unroll
+        for (int e = 0; e < NV; e++) s = s + (va[q][e] == ninf ? T(0) : dev_exp(va[q][e] - mx));
+    } else {
+#pragma unroll
+      for (int q = 0; q < U; q++)
+#pragma unroll
+        for (int e = 0; e < NV; e++) s = s + Algo::term(va[q][e], kTwo ? vb[q][e] : T(0), T(0));
+    }
   }
-  T s = T(0);
-  for (long r = threadIdx.x; r < m; r += 1024) s = s + Algo::term(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx);
-  s = block_reduce<T, 1024 / kWave>(s, lds, AddFn(), T(0));
+  if (Algo::kNeedMax) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) maxsum_merge(mx, s, __shfl_xor(mx, off), __shfl_xor(s, off));
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) { lds[0][wave] = mx; lds[1][wave] = s; }
+    __syncthreads();
+    mx = lds[0][0];
+    s = lds[1][0];
+    for (int w = 1; w < 1024 / kWave; w++) maxsum_merge(mx, s, lds[0][w], lds[1][w]);
+  } else {
+    s = block_reduce<T, 1024 / kWave>(s, lds[0], AddFn(), T(0));
+  }
   const T fin = Algo::finish(s);
   int lab = Algo::kNll ? labels[col] : 0;
   if (lab < 0 || lab > m) lab = 0;
   const T st = -scale;
-  for (long r = threadIdx.x; r < m; r += 1024) {
-    T v = Algo::out(ac[r], Algo::kInputs == 2 ? bc[r] : T(0), mx, fin);
-    if (Algo::kNll) {
-      const bool hit = (r + 1 == lab);
-      if (hit) loss[col] = -v;
-      const T dlp = hit ? st : T(0);
-      const T p = dev_exp(v) * st;
-      v = lab == 0 ? T(0) : dlp - p;
+  for (long r0 = (long)threadIdx.x * NV; r0 < m; r0 += STEP * U) {
+    T va[U][NV], vb[U][NV];
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long r = r0 + q * STEP;
+      if (r < m) {
+        if (VEC) {
+          const V t = ld_stream(reinterpret_cast<const V*>(ac + r));
+#pragma unroll
+          for (int e = 0; e < NV; e++) va[q][e] = t[e];
+          if (kTwo) {
+            const V t2 = ld_stream(reinterpret_cast<const V*>(bc + r));
+#pragma unroll
+            for (int e = 0; e < NV; e++) vb[q][e] = t2[e];
+          }
+        } else {
+          va[q][0] = ac[r];
+          if (kTwo) vb[q][0] = bc[r];
+        }
+      }
     }
-    oc[r] = v;
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long r = r0 + q * STEP;
+      if (r < m) {
+        V vo;
+#pragma unroll
+        for (int e = 0; e < NV; e++) {
+          T v = Algo::out(va[q][e], kTwo ? vb[q][e] : T(0), mx, fin);
+          if (Algo::kNll) {
+            const bool hit = (r + e + 1 == lab);
+            if (hit) loss[col] = -v;
+            const T dlp = hit ? st : T(0);
+            const T p = dev_exp(v) * st;
+            v = lab == 0 ? T(0) : dlp - p;
+          }
+          vo[e] = v;
+        }
+        if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+        else __builtin_nontemporal_store(vo[0], oc + r);
+      }
+    }
   }
   if (Algo::kNll && lab == 0 && threadIdx.x == 0) loss[col] = T(0);
 }
@@ -391,18 +490,26 @@ template <typename T, typename Algo>
 inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const T* b, T* out, const int* labels, T scale, T* loss) {
   if (m <= 0 || n <= 0) return;
   constexpr int N = Vec16<T>::N;
-  // two held inputs double the register footprint: halve the per-lane capacity
-  constexpr int kBig = (Algo::kInputs == 2 && Algo::kHoldA) ? 32 : 64;
+  // Per-lane capacity: a lane of a wave or 256-lane team may hold 64 elements (32 when two inputs are held); the
+  // 1024-lane workgroup is limited to 128 registers per lane, i.e. 64 fp32 / 32 fp64 held elements (half with two held
+  // inputs) -- more than that spills.  Longer columns stream.
+  constexpr int kHeld = (Algo::kInputs == 2 && Algo::kHoldA) ? 2 : 1;
+  constexpr int kBig = 64 / kHeld;
+  constexpr int kBig1024 = 256 / (int)(sizeof(T) * kHeld);
   const bool vec = (m % N == 0) && aligned16(a) && aligned16(out) && (Algo::kInputs == 1 || aligned16(b));
+  const long resident_cap = tuning(kTuneSoftmaxResidentRows);  // 0: no limit below the register capacity (tests lower it to reach the streaming kernel with short columns)
 #define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
+  if ((resident_cap > 0 && m > resident_cap) || m > 1024L * kBig1024) {
+    if (vec) hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, true>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
+    else hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, false>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
+    return;
+  }
   if (m <= 64 * 4) KNET8_SM(64, 4);
   else if (m <= 64 * 16) KNET8_SM(64, 16);
   else if (m <= 64 * kBig) KNET8_SM(64, kBig);
   else if (m <= 256 * kBig) KNET8_SM(256, kBig);
-  else if (m <= 1024 * 32) KNET8_SM(1024, 32);
-  else if (m <= 1024 * kBig) KNET8_SM(1024, kBig);
-  else
-    hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
+  else if (m <= 1024 * (kBig1024 / 2)) KNET8_SM(1024, kBig1024 / 2);
+  else KNET8_SM(1024, kBig1024);
 #undef KNET8_SM
 }
 

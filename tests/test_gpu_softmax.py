@@ -224,3 +224,68 @@ def test_logsumexp_value_and_gradient(knet, oracle):
             J = knet.diff(lambda: knet.sum(knet.mul(knet.logsumexp(p, dims=dims), knet.KnetArray(dy))))
             wantg = oracle.logsumexpback(x, want, dy, dims=od)
         assert close(knet.Array(knet.grad(J, p)), wantg, 2e-5), (shape, dims)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_streaming_kernel_on_short_columns_and_masked_logits(knet, oracle, dt):
+    """The two-pass streaming kernel (normally only for columns beyond the register capacity) is forced on short columns through
+    the tuning knob, so that its running (max, sum) pairs meet every column length class, -inf (masked) logits in leading,
+    trailing and whole-column positions, and all five algorithms, against the oracle's max-first evaluation."""
+    fn = knet.libknet8().fn
+    rng = np.random.default_rng(39)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    S = "32" if dt == np.float32 else "64"
+    old = fn["knet8_tune"](1, 1)
+    try:
+        for m in (2, 3, 64, 257, 1000, 4099, 4100, 16384, 20001, 40000):
+            n = 7
+            x = (rng.standard_normal((m, n)) * 3).astype(dt)
+            x[: m // 2, 1] = -np.inf          # leading masked rows: the running max starts at -inf
+            x[m // 2:, 2] = -np.inf if m > 2 else x[m // 2:, 2]
+            x[0, 2] = 5.0
+            x[:, 3] = np.sort(x[:, 3])        # ascending: the running max changes at every step
+            x[:, 4] = np.sort(x[:, 4])[::-1]  # descending: it never changes after the first element
+            dy = rng.standard_normal((m, n)).astype(dt)
+            labels = rng.integers(0, m + 1, size=n).astype(np.int32)
+            labels[1] = m  # a row that is not masked in column 1
+            xd, dyd = knet.KnetArray(x), knet.KnetArray(dy)
+            with np.errstate(all="ignore"):
+                want = oracle.logsoftmax(x, dims=1)
+                want_sm = oracle.softmax(x, dims=1)
+            got = knet.Array(knet.logsoftmax(xd, dims=1))
+            fin = np.isfinite(want)
+            assert np.array_equal(np.isneginf(got), np.isneginf(want)), m
+            assert np.abs(got[fin] - want[fin]).max() <= rtol * np.abs(want[fin]).max(), m
+            assert close(knet.Array(knet.softmax(xd, dims=1)), want_sm, rtol), m
+            y = np.where(fin, want, dt(-50))
+            got = knet.Array(knet.logsoftmaxback(knet.KnetArray(y), dyd, dims=1))
+            assert close(got, oracle.logsoftmaxback(y, dy, dims=1), rtol), m
+            got = knet.Array(knet.softmaxback(knet.KnetArray(want_sm), dyd, dims=1))
+            assert close(got, oracle.softmaxback(want_sm, dy, dims=1), rtol), m
+            dx, loss = xd.similar(), knet.KnetArray(np.zeros(n, dt))
+            knet.knet8("nll_logsoftmax_back_%s" % S, m, n, xd.ptr, knet.KnetArray(labels).ptr, xd.ctype(0.25), dx.ptr, loss.ptr)
+            onehot = np.zeros((m, n), dt)
+            cols = np.nonzero(labels)[0]
+            onehot[labels[cols] - 1, cols] = 1
+            want_dx = (want_sm - onehot) * dt(0.25)
+            want_dx[:, labels == 0] = 0
+            assert close(knet.Array(dx), want_dx, rtol), m
+            want_loss = np.zeros(n, dt)
+            want_loss[cols] = -want[labels[cols] - 1, cols]
+            gl = knet.Array(loss)
+            finl = np.isfinite(want_loss)
+            assert np.array_equal(np.isposinf(gl), np.isposinf(want_loss)), m
+            assert np.allclose(gl[finl], want_loss[finl], rtol=rtol, atol=10 * rtol), m
+    finally:
+        fn["knet8_tune"](1, old)
+    knet.libknet8().check()
+    # whole column masked: NaN everywhere in that column, as from the max-first evaluation (-inf - -inf)
+    x = (rng.standard_normal((300, 3)) * 3).astype(dt)
+    x[:, 1] = -np.inf
+    old = fn["knet8_tune"](1, 1)
+    try:
+        got = knet.Array(knet.logsoftmax(knet.KnetArray(x), dims=1))
+    finally:
+        fn["knet8_tune"](1, old)
+    assert np.all(np.isnan(got[:, 1])) and np.all(np.isfinite(got[:, [0, 2]]))
+    assert fn["knet8_tune"](1, -1) == 0  # the knob is back at its default: later tests run the register-resident kernels
