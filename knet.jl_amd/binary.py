@@ -1,8 +1,8 @@
 """Broadcasting arithmetic on ``KnetArray`` and AutoGrad's ``unbroadcast``.
 
-Mirrors the kernel selection of src/knetarrays/binary.jl:13-149 for the cases the gradient path uses:
-scalar (op) array -> ``F_S_01``; equal shapes -> ``F_S_11``; one operand a vector along a single
-dimension of the other -> ``F_S_12`` (bias add).  ``unbroadcast`` restates AutoGrad.jl's published rule
+Mirrors the kernel selection of src/knetarrays/binary.jl:13-149: scalar (op) array -> ``F_S_01``; equal shapes ->
+``F_S_11``; one operand a vector along a single dimension of the other -> ``F_S_12`` (bias add); anything else ->
+``F_S_16_3/4/5`` or ``F_S_17`` by the number of dimensions of the result.  ``unbroadcast`` restates AutoGrad.jl's published rule
 (the package is not part of the reference repository): sum the gradient over every dimension in which the
 operand had size 1 and the result did not, then reshape to the operand's size.
 """
@@ -62,8 +62,6 @@ def broadcast_op(name, x, y):
         z = x.similar(x.dims if len(x.dims) >= len(y.dims) else y.dims)
         knet8("%s_%s_11" % (name, x.suffix), z.length, x.ptr, y.ptr, z.ptr)
         return z
-    if y.length == 1 or x.length == 1:
-        raise TypeError("pass 1-element operands as numbers")
     vx, vy = _vector_dim(x.dims, y.dims), _vector_dim(y.dims, x.dims)
     if vy is not None and y.length < x.length:
         z = x.similar()
@@ -73,7 +71,50 @@ def broadcast_op(name, x, y):
         z = y.similar()
         knet8("%s_%s_12" % (name, x.suffix), z.length, x.ptr, vx[0], vx[1], y.ptr, 1, y.length, z.ptr)
         return z
-    raise ValueError("DimensionMismatch: %r, %r" % (x.dims, y.dims))
+    return _broadcast_nd(name, x, y)
+
+
+def _broadcast_nd(name, x, y):
+    """Several broadcast dimensions, or both operands broadcasting: result size as ``vbroadcast_shape``
+    (src/knetarrays/binary.jl:150-212), element strides with 0 on broadcast dimensions as ``get_strides`` (``:214-231``);
+    a 2-d result goes to ``F_S_12`` with both operands as vectors (``:71-80``), 3 to 5 dims to ``F_S_16_k`` (``:96-116``), more to
+    ``F_S_17`` with the strides in device arrays (``:117-125``)."""
+    nd = max(x.ndims, y.ndims)
+    xs = tuple(x.dims) + (1,) * (nd - x.ndims)
+    ys = tuple(y.dims) + (1,) * (nd - y.ndims)
+    dz = []
+    for a, b in zip(xs, ys):
+        if a != b and a != 1 and b != 1:
+            raise ValueError("DimensionMismatch: arrays could not be broadcast to a common size: %r, %r" % (x.dims, y.dims))
+        dz.append(b if a == 1 else a)
+    z = x.similar(tuple(dz))
+    if z.length == 0:
+        return z
+
+    def strides(dims):
+        out, st = [], 1
+        for k in range(nd):
+            out.append(0 if dims[k] != dz[k] else st)
+            st *= dims[k]
+        return out
+    sx, sy, sz = strides(xs), strides(ys), strides(dz)
+    if nd <= 2:
+        # (m,1) with (1,n): each operand is a vector along one dimension of the result; a 1-element array is read as x[0]
+        # (sx = length(z), nx = 1 in vbroadcast_shape) without the device-to-host copy the reference makes for it
+        def as_vector(a):
+            if a.length == 1:
+                return z.length, 1
+            if a.length == z.length:
+                return 1, z.length
+            return _vector_dim(a.dims, dz)
+        vx, vy = as_vector(x), as_vector(y)
+        knet8("%s_%s_12" % (name, x.suffix), z.length, x.ptr, vx[0], vx[1], y.ptr, vy[0], vy[1], z.ptr)
+    elif nd <= 5:
+        knet8("%s_%s_16_%d" % (name, x.suffix, nd), x.ptr, y.ptr, z.ptr, *(sx + sy + sz + [z.length]))
+    else:
+        dev = [KnetArray(np.asarray(v, dtype=np.int32)) for v in (sx, sy, sz)]
+        knet8("%s_%s_17" % (name, x.suffix), x.ptr, y.ptr, z.ptr, dev[0].ptr, dev[1].ptr, dev[2].ptr, z.length, nd)
+    return z
 
 
 def _squeeze(dims):

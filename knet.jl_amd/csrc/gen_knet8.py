@@ -162,6 +162,7 @@ class Out:
 
 PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_elementwise.h"
+#include "../knet8_broadcast.h"
 #include "../knet8_reduce.h"
 #include "../knet8_fused.h"
 #include "../knet8_softmax.h"
@@ -215,6 +216,24 @@ def gen_elementwise():
             o.entry("%s_%s_13_y_x" % (name, S), "void", p13,
                     "(void)nextstride; (void)multidimsize; launch_bcast12<%s>(stream, A_N, x, 1, A_N, y, dimstride, B_N, z, Op2r_%s<%s>())" % (T, name, T),
                     "src/libknet8/cuda13.jl:108-184")
+    o.decl.append("\n/* ---- general N-d broadcast: element strides per dimension, 0 for a broadcast dimension; z contiguous with N elements.\n"
+                  "   _16_3/_16_4/_16_5 take the strides by value (src/libknet8/cuda16.jl:10-88), _17 in device int arrays of length\n"
+                  "   dimlen_z (src/libknet8/cuda17.jl:25-64); caller src/knetarrays/binary.jl:96-125 ---- */")
+    for name, body, cite in BINARY_OPS:
+        for T, S in TYPES:
+            for nd in (3, 4, 5):
+                ps = [(T + "*", "x"), (T + "*", "y"), (T + "*", "z")]
+                for arr in ("x", "y", "z"):
+                    ps += [("int", "stride_%s%d" % (arr, k + 1)) for k in range(nd)]
+                ps.append(("int", "N_z"))
+                arrs = "; ".join("const int s%s[%d] = {%s}" % (arr, nd, ", ".join("stride_%s%d" % (arr, k + 1) for k in range(nd))) for arr in ("x", "y", "z"))
+                o.entry("%s_%s_16_%d" % (name, S, nd), "void", ps, None, "src/libknet8/cuda16.jl:60-86",
+                        body="  %s;\n  launch_bcast_nd<%s>(stream, %d, sx, sy, sz, N_z, x, y, z, Op2_%s<%s>());\n  knet8::check_launch(\"%s_%s_16_%d\");"
+                             % (arrs, T, nd, name, T, name, S, nd))
+            o.entry("%s_%s_17" % (name, S), "void",
+                    [(T + "*", "x"), (T + "*", "y"), (T + "*", "z"), ("int*", "stride_x"), ("int*", "stride_y"), ("int*", "stride_z"), ("int", "N_z"), ("int", "dimlen_z")],
+                    "launch_bcast17<%s>(stream, x, y, z, stride_x, stride_y, stride_z, N_z, dimlen_z, Op2_%s<%s>())" % (T, name, T),
+                    "src/libknet8/cuda17.jl:58-64")
     o.decl.append("\n/* ---- activation gradients dx[i] = f(dy[i], y[i]) -- src/libknet8/cuda11.jl:12-28 with the *back rows of ops.jl:114-121 ---- */")
     for name, body, cite in BACK11_OPS:
         s.append(functor("Op11_" + name, ["xi", "yi"], body))

@@ -66,17 +66,14 @@ def _sum_back(x, dims):
         # gradient of sum: dy broadcast back to size(x): zero(x) .+ dy  (AutoGrad's rule for sum)
         z = x.similar()
         if isinstance(dy, KnetArray):
-            k = [i for i in range(z.ndims) if dy.size(i + 1) != 1]
-            if not k:
-                raise ValueError("pass 1-element gradients as numbers")
             if dy.length == z.length:
                 knet8("add_%s_01" % z.suffix, z.length, z.ctype(0), dy.ptr, z.ptr)
             else:
-                from .binary import _vector_dim
+                from .binary import _vector_dim, broadcast_op
                 knet8("fill_%s" % z.suffix, z.length, z.ctype(0), z.ptr)
                 v = _vector_dim(dy.dims, z.dims)
-                if v is None:
-                    raise ValueError("sum gradient: unsupported dims %r" % (dims,))
+                if v is None:  # reduced over several separate dimensions (or to one element): the general broadcast
+                    return (broadcast_op("add", z, dy),)
                 knet8("add_%s_12" % z.suffix, z.length, z.ptr, 1, z.length, dy.ptr, v[0], v[1], z.ptr)
         else:
             knet8("fill_%s" % z.suffix, z.length, z.ctype(dy), z.ptr)

@@ -68,6 +68,18 @@ def test_broadcast_dispatch(knet, rec):
         knet.broadcast_op("add", x, arr((100, 64)))
     with pytest.raises(TypeError):
         knet.broadcast_op("add", x, arr((64, 100), np.float64))
+    # several broadcast dims: strides as get_strides builds them (0 on a broadcast dim), kernel by ndims of the result
+    z = knet.broadcast_op("add", arr((8, 8, 16, 4)), arr((8, 8, 1, 4)))       # test/binary.jl:21
+    assert z.dims == (8, 8, 16, 4) and calls[-1][0] == "add_32_16_4"
+    assert calls[-1][4:] == (1, 8, 64, 1024, 1, 8, 0, 64, 1, 8, 64, 1024, 4096)
+    z = knet.broadcast_op("mul", arr((7, 1, 5)), arr((1, 6, 1)))
+    assert z.dims == (7, 6, 5) and calls[-1][0] == "mul_32_16_3" and calls[-1][4:] == (1, 0, 7, 0, 1, 0, 1, 7, 42, 210)
+    z = knet.broadcast_op("div", arr((3, 1)), arr((1, 4)))                   # 2-d result: _12 with both operands as vectors
+    assert z.dims == (3, 4) and calls[-1][0] == "div_32_12" and calls[-1][3:5] == (1, 3) and calls[-1][6:8] == (3, 4)
+    z = knet.broadcast_op("add", arr((1, 1)), arr((2, 2)))                   # 1-element array: sx = length(z), nx = 1
+    assert z.dims == (2, 2) and calls[-1][0] == "add_32_12" and calls[-1][3:5] == (4, 1) and calls[-1][6:8] == (1, 4)
+    with pytest.raises(ValueError):
+        knet.broadcast_op("add", arr((3, 4, 2)), arr((3, 5, 2)))
     # unbroadcast: which dims get summed (AutoGrad's rule)
     g = knet.unbroadcast(b, x)
     assert g.dims == (64, 1) and calls[-1][0] == "sum_32_21" and calls[-1][3:5] == (1, 64)
