@@ -16,6 +16,7 @@ from .reduction import sum, prod, maximum, minimum, sumabs, sumabs2, maxabs, min
 from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
 from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback
 from .loss import nll, findindices, accuracy, getindex, ungetindex, bce, logistic
+from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat)
 from .dropout import dropout, dropback, dropout_, dropback_
 from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
 from .linalg import matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose

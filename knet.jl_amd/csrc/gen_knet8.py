@@ -415,6 +415,29 @@ def gen_softmax():
                 "launch_setents<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:349-355")
         o.entry("addents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],
                 "launch_addents<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:356-362")
+        o.entry("setent1_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T, "y")],
+                "launch_setent1<%s>(stream, n, ents, x, y)" % T, "src/libknet8/cuda1.jl:363-369")
+    o.decl.append("\n/* ---- whole columns / rows of an xrows x xcols matrix by 1-based int32 index: get (y = x[sel]), set (x[sel] = y), add (x[sel] += y,\n"
+                  "   atomic: repeated indices accumulate), set1 (x[sel] = scalar) -- src/libknet8/cuda1.jl:234-341 ---- */")
+    for T, S in TYPES:
+        for kind, sel, n in (("cols", "cols", "ncols"), ("rows", "rows", "nrows")):
+            one = kind[:-1] + "1"
+            for mode, name in enumerate(("get" + kind, "set" + kind, "add" + kind)):
+                o.entry("%s_%s" % (name, S), "void", [("int", "xrows"), ("int", "xcols"), ("int", n), ("int*", sel), (T + "*", "x"), (T + "*", "y")],
+                        "launch_%s<%s, %d>(stream, xrows, xcols, %s, %s, x, y, %s(0))" % (kind, T, mode, n, sel, T), "src/libknet8/cuda1.jl:234-341")
+            o.entry("set%s_%s" % (one, S), "void", [("int", "xrows"), ("int", "xcols"), ("int", n), ("int*", sel), (T + "*", "x"), (T, "y")],
+                    "launch_%s<%s, 3>(stream, xrows, xcols, %s, %s, x, (%s*)nullptr, y)" % (kind, T, n, sel, T), "src/libknet8/cuda1.jl:234-341")
+    o.decl.append("\n/* ---- rectangular blocks and concatenation.  xcopy counts rows and steps in BYTES, xfill in elements; icat takes a HOST array of\n"
+                  "   device pointers, concat device arrays of starts, lengths and pointers -- src/libknet8/cuda1.jl:107-207,503-530 ---- */")
+    o.entry("xcopy", "void", [("int", "nrows"), ("int", "ncols"), ("const void*", "x"), ("int", "incx"), ("void*", "y"), ("int", "incy")],
+            "launch_xcopy(stream, nrows, ncols, x, incx, y, incy)", "src/libknet8/cuda1.jl:130-165")
+    for T, S in TYPES:
+        o.entry("xfill_%s" % S, "void", [("int", "nrows"), ("int", "ncols"), (T, "x"), (T + "*", "y"), ("int", "incy")],
+                "launch_xfill<%s>(stream, nrows, ncols, x, y, incy)" % T, "src/libknet8/cuda1.jl:107-128")
+        o.entry("icat_%s" % S, "void", [("int", "nrows"), ("int", "ncols"), (T + "**", "x"), (T + "*", "y")],
+                "launch_icat<%s>(stream, nrows, ncols, x, y)" % T, "src/libknet8/cuda1.jl:167-207")
+        o.entry("concat_%s" % S, "void", [("int", "narrays"), ("int*", "starts"), ("int*", "lengths"), (T + "**", "x"), (T + "*", "y")],
+                "launch_concat<%s>(stream, narrays, starts, lengths, x, y)" % T, "src/libknet8/cuda1.jl:503-530")
     return o
 
 

@@ -107,3 +107,19 @@ def test_softmax_and_activation_dispatch(knet, rec):
     assert calls[-1][:2] == ("geluback_32_111", 32000 * 512)
     with pytest.raises(ValueError):
         knet.reluback(x, arr((5,)))
+
+
+def test_block_index_parameters_follow_indexparams(knet):
+    # src/knetarrays/getindex.jl:705-745: runs of nrows contiguous elements, astep apart, from a 1-based first linear index
+    import sys
+    ip = sys.modules["knet_jl_amd.indexing"]._indexparams
+    assert ip((37, 21), None, None) == (777, 777, 1, 1, 777, (37, 21))
+    assert ip((37, 21), None, (3, 9)) == (259, 259, 1, 75, 777, (37, 7))          # whole columns: one contiguous run
+    assert ip((37, 21), (5, 20), (3, 9)) == (112, 16, 7, 79, 37, (16, 7))          # a block: 7 runs of 16, one column apart
+    assert ip((37, 21), 7, None) == (21, 1, 21, 7, 37, (21,))                      # a row: 21 single elements
+    assert ip((37, 21), None, 4) == (37, 37, 1, 112, 777, (37,))                   # a column: a view
+    assert ip((37, 21), (4, 3), None)[0] == 0                                      # empty range
+    with pytest.raises(IndexError):
+        ip((37, 21), (0, 3), None)
+    with pytest.raises(IndexError):
+        ip((37, 21), None, 22)
