@@ -241,6 +241,12 @@ def profile_pass(torch, K):
     dxx = y.similar()
     for _ in range(3):
         K.knet8("dropback_32", n5, ctypes.c_float(0.5), y.ptr, y.ptr, dyy.ptr, dxx.ptr)
+    bias = device_randn(torch, K, 4096, f32, 11)
+    db = bias.similar()
+    for _ in range(3):
+        u = device_randn(torch, K, n5, f32, 12)
+        K.knet8("biasreludrop_32", 4096, 2048, ctypes.c_float(0.5), dyy.ptr, bias.ptr, u.ptr)
+        K.knet8("dropreluback_biasgrad_32", 4096, 2048, ctypes.c_float(0.5), dyy.ptr, u.ptr, dxx.ptr, db.ptr)
     torch.cuda.synchronize()
     K.libknet8().check()
 
