@@ -13,24 +13,25 @@ from .karray import KnetArray
 from .libknet8 import knet8
 from .reduction import sum as ksum
 
-_SWAPPED = {"sub": None, "div": None}
-
-
 def _scalar_array(name, s, y, scalar_first=True):
     z = y.similar()
     c = y.ctype
     if scalar_first:
         knet8("%s_%s_01" % (name, y.suffix), z.length, c(s), y.ptr, z.ptr)
         return z
-    # array (op) scalar: commutative ops reuse _01; a-s = a+(-s); a/s = a*(1/s) is NOT used (different rounding):
-    if name in ("add", "mul", "max", "min"):
+    # array (op) scalar: commutative ops reuse _01; a-s = a+(-s); comparisons swap sides (a>s is s<a); a/s = a*(1/s) is NOT
+    # used (different rounding): div and pow fill a temporary with the scalar and go through _11
+    swap = {"gt": "lt", "lt": "gt", "ge": "le", "le": "ge"}
+    if name in ("add", "mul", "max", "min", "eq", "ne"):
         knet8("%s_%s_01" % (name, y.suffix), z.length, c(s), y.ptr, z.ptr)
+    elif name in swap:
+        knet8("%s_%s_01" % (swap[name], y.suffix), z.length, c(s), y.ptr, z.ptr)
     elif name == "sub":
         knet8("add_%s_01" % y.suffix, z.length, c(-s), y.ptr, z.ptr)
-    else:  # div: fill a temporary with the scalar and divide elementwise
+    else:
         t = y.similar()
         knet8("fill_%s" % y.suffix, t.length, c(s), t.ptr)
-        knet8("div_%s_11" % y.suffix, z.length, y.ptr, t.ptr, z.ptr)
+        knet8("%s_%s_11" % (name, y.suffix), z.length, y.ptr, t.ptr, z.ptr)
     return z
 
 

@@ -57,6 +57,42 @@ UNARY_OPS = [
     ("one", "return T(1);", "src/libknet8/ops.jl:52"),
     ("copy", "return xi;", "the contiguous case of xcopy, src/libknet8/cuda1.jl:130-165 (also the known-size 1R+1W kernel used to calibrate HBM counters)"),
     ("zero", "return T(0);", "src/libknet8/ops.jl:67"),
+    # the plain libm rows of the same table (src/libknet8/ops.jl:6-66)
+    ("acos", "return kacos(xi);", "src/libknet8/ops.jl:6-66 (acos)"),
+    ("acosh", "return kacosh(xi);", "src/libknet8/ops.jl:6-66 (acosh)"),
+    ("asin", "return kasin(xi);", "src/libknet8/ops.jl:6-66 (asin)"),
+    ("asinh", "return kasinh(xi);", "src/libknet8/ops.jl:6-66 (asinh)"),
+    ("atan", "return katan(xi);", "src/libknet8/ops.jl:6-66 (atan)"),
+    ("atanh", "return katanh(xi);", "src/libknet8/ops.jl:6-66 (atanh)"),
+    ("cbrt", "return kcbrt(xi);", "src/libknet8/ops.jl:6-66 (cbrt)"),
+    ("ceil", "return kceil(xi);", "src/libknet8/ops.jl:6-66 (ceil)"),
+    ("cos", "return kcos(xi);", "src/libknet8/ops.jl:6-66 (cos)"),
+    ("cosh", "return kcosh(xi);", "src/libknet8/ops.jl:6-66 (cosh)"),
+    ("cospi", "return kcospi(xi);", "src/libknet8/ops.jl:6-66 (cospi)"),
+    ("erf", "return kerf(xi);", "src/libknet8/ops.jl:6-66 (erf)"),
+    ("erfc", "return kerfc(xi);", "src/libknet8/ops.jl:6-66 (erfc)"),
+    ("erfcinv", "return kerfcinv(xi);", "src/libknet8/ops.jl:6-66 (erfcinv)"),
+    ("erfcx", "return kerfcx(xi);", "src/libknet8/ops.jl:6-66 (erfcx)"),
+    ("erfinv", "return kerfinv(xi);", "src/libknet8/ops.jl:6-66 (erfinv)"),
+    ("exp10", "return kexp10(xi);", "src/libknet8/ops.jl:6-66 (exp10)"),
+    ("exp2", "return kexp2(xi);", "src/libknet8/ops.jl:6-66 (exp2)"),
+    ("expm1", "return kexpm1(xi);", "src/libknet8/ops.jl:6-66 (expm1)"),
+    ("floor", "return kfloor(xi);", "src/libknet8/ops.jl:6-66 (floor)"),
+    ("log10", "return klog10(xi);", "src/libknet8/ops.jl:6-66 (log10)"),
+    ("log1p", "return klog1p(xi);", "src/libknet8/ops.jl:6-66 (log1p)"),
+    ("log2", "return klog2(xi);", "src/libknet8/ops.jl:6-66 (log2)"),
+    ("sin", "return ksin(xi);", "src/libknet8/ops.jl:6-66 (sin)"),
+    ("sinh", "return ksinh(xi);", "src/libknet8/ops.jl:6-66 (sinh)"),
+    ("sinpi", "return ksinpi(xi);", "src/libknet8/ops.jl:6-66 (sinpi)"),
+    ("tan", "return ktan(xi);", "src/libknet8/ops.jl:6-66 (tan)"),
+    ("trunc", "return ktrunc(xi);", "src/libknet8/ops.jl:6-66 (trunc)"),
+    ("round", "return krint(xi);", "src/libknet8/ops.jl:52; ties go to the even neighbour as Julia's round does on the CPU path (the CUDA kernel rounds them away from zero)"),
+    ("j0", "return kj0(xi);", "src/libknet8/ops.jl:31 (j0)"),
+    ("j1", "return kj1(xi);", "src/libknet8/ops.jl:32 (j1)"),
+    ("y0", "return ky0(xi);", "src/libknet8/ops.jl:63 (y0)"),
+    ("y1", "return ky1(xi);", "src/libknet8/ops.jl:64 (y1)"),
+    ("lgamma", "return klgamma(xi);", "src/libknet8/ops.jl:34"),
+    ("gamma_impl", "return ktgamma(xi);", "src/libknet8/ops.jl:33 (gamma_impl, src/libknet8/gamma.jl)"),
 ]
 
 # name, body in terms of (xi, yi), citation.  Used for the _01, _11 and _12/_13 entry points.
@@ -67,12 +103,20 @@ BINARY_OPS = [
     ("div", "return xi / yi;", "src/libknet8/ops.jl:91"),
     ("max", "return xi > yi ? xi : yi;", "src/libknet8/ops.jl:93"),
     ("min", "return xi < yi ? xi : yi;", "src/libknet8/ops.jl:94"),
+    ("pow", "return kpow(xi, yi);", "src/libknet8/ops.jl:92"),
+    ("eq", "return xi == yi ? T(1) : T(0);", "src/libknet8/ops.jl:95"),
+    ("ne", "return xi != yi ? T(1) : T(0);", "src/libknet8/ops.jl:96"),
+    ("gt", "return xi > yi ? T(1) : T(0);", "src/libknet8/ops.jl:97"),
+    ("ge", "return xi >= yi ? T(1) : T(0);", "src/libknet8/ops.jl:98"),
+    ("lt", "return xi < yi ? T(1) : T(0);", "src/libknet8/ops.jl:99"),
+    ("le", "return xi <= yi ? T(1) : T(0);", "src/libknet8/ops.jl:100"),
 ]
 
 FUSED_ACTS = ["relu", "sigm", "tanh", "elu", "selu"]
 
 # Two-input gradients NAME_S_11(n, dy, y, dx): xi = dy, yi = y.
 BACK11_OPS = [
+    ("invxback", "const T a = -xi; const T b = a * yi; return b * yi;", "src/libknet8/ops.jl:115 (-dy*y*y, the gradient of the deprecated invx, src/ops20/activation.jl:60-63)"),
     ("reluback", "return yi > T(0) ? xi : T(0);", "src/ops20/activation.jl:27, src/libknet8/ops.jl:118"),
     ("sigmback", "const T a = xi * yi; const T b = T(1) - yi; return a * b;", "src/ops20/activation.jl:56, src/libknet8/ops.jl:120"),
     ("tanhback", "const T a = yi * yi; const T b = T(1) - a; return xi * b;", "src/ops20_gpu/activation.jl:11, src/libknet8/ops.jl:121"),

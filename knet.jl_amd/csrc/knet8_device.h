@@ -111,4 +111,76 @@ __device__ __forceinline__ float kerf(float x) { return erff(x); }
 __device__ __forceinline__ double kerf(double x) { return erf(x); }
 __device__ __forceinline__ float ksqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double ksqrt(double x) { return sqrt(x); }
+
+// The rest of the unary table of src/libknet8/ops.jl:6-80: one wrapper per libm routine, so that the op bodies are written once for both types.
+__device__ __forceinline__ float kacos(float x) { return acosf(x); }
+__device__ __forceinline__ double kacos(double x) { return acos(x); }
+__device__ __forceinline__ float kacosh(float x) { return acoshf(x); }
+__device__ __forceinline__ double kacosh(double x) { return acosh(x); }
+__device__ __forceinline__ float kasin(float x) { return asinf(x); }
+__device__ __forceinline__ double kasin(double x) { return asin(x); }
+__device__ __forceinline__ float kasinh(float x) { return asinhf(x); }
+__device__ __forceinline__ double kasinh(double x) { return asinh(x); }
+__device__ __forceinline__ float katan(float x) { return atanf(x); }
+__device__ __forceinline__ double katan(double x) { return atan(x); }
+__device__ __forceinline__ float katanh(float x) { return atanhf(x); }
+__device__ __forceinline__ double katanh(double x) { return atanh(x); }
+__device__ __forceinline__ float kcbrt(float x) { return cbrtf(x); }
+__device__ __forceinline__ double kcbrt(double x) { return cbrt(x); }
+__device__ __forceinline__ float kceil(float x) { return ceilf(x); }
+__device__ __forceinline__ double kceil(double x) { return ceil(x); }
+__device__ __forceinline__ float kcos(float x) { return cosf(x); }
+__device__ __forceinline__ double kcos(double x) { return cos(x); }
+__device__ __forceinline__ float kcosh(float x) { return coshf(x); }
+__device__ __forceinline__ double kcosh(double x) { return cosh(x); }
+__device__ __forceinline__ float kcospi(float x) { return cospif(x); }
+__device__ __forceinline__ double kcospi(double x) { return cospi(x); }
+__device__ __forceinline__ float kerfc(float x) { return erfcf(x); }
+__device__ __forceinline__ double kerfc(double x) { return erfc(x); }
+__device__ __forceinline__ float kerfcinv(float x) { return erfcinvf(x); }
+__device__ __forceinline__ double kerfcinv(double x) { return erfcinv(x); }
+__device__ __forceinline__ float kerfcx(float x) { return erfcxf(x); }
+__device__ __forceinline__ double kerfcx(double x) { return erfcx(x); }
+__device__ __forceinline__ float kerfinv(float x) { return erfinvf(x); }
+__device__ __forceinline__ double kerfinv(double x) { return erfinv(x); }
+__device__ __forceinline__ float kexp10(float x) { return exp10f(x); }
+__device__ __forceinline__ double kexp10(double x) { return exp10(x); }
+__device__ __forceinline__ float kexp2(float x) { return exp2f(x); }
+__device__ __forceinline__ double kexp2(double x) { return exp2(x); }
+__device__ __forceinline__ float kexpm1(float x) { return expm1f(x); }
+__device__ __forceinline__ double kexpm1(double x) { return expm1(x); }
+__device__ __forceinline__ float kfloor(float x) { return floorf(x); }
+__device__ __forceinline__ double kfloor(double x) { return floor(x); }
+__device__ __forceinline__ float kj0(float x) { return j0f(x); }
+__device__ __forceinline__ double kj0(double x) { return j0(x); }
+__device__ __forceinline__ float kj1(float x) { return j1f(x); }
+__device__ __forceinline__ double kj1(double x) { return j1(x); }
+__device__ __forceinline__ float klgamma(float x) { return lgammaf(x); }
+__device__ __forceinline__ double klgamma(double x) { return lgamma(x); }
+__device__ __forceinline__ float ktgamma(float x) { return tgammaf(x); }
+__device__ __forceinline__ double ktgamma(double x) { return tgamma(x); }
+__device__ __forceinline__ float klog10(float x) { return log10f(x); }
+__device__ __forceinline__ double klog10(double x) { return log10(x); }
+__device__ __forceinline__ float klog1p(float x) { return log1pf(x); }
+__device__ __forceinline__ double klog1p(double x) { return log1p(x); }
+__device__ __forceinline__ float klog2(float x) { return log2f(x); }
+__device__ __forceinline__ double klog2(double x) { return log2(x); }
+__device__ __forceinline__ float krint(float x) { return rintf(x); }
+__device__ __forceinline__ double krint(double x) { return rint(x); }
+__device__ __forceinline__ float ksin(float x) { return sinf(x); }
+__device__ __forceinline__ double ksin(double x) { return sin(x); }
+__device__ __forceinline__ float ksinh(float x) { return sinhf(x); }
+__device__ __forceinline__ double ksinh(double x) { return sinh(x); }
+__device__ __forceinline__ float ksinpi(float x) { return sinpif(x); }
+__device__ __forceinline__ double ksinpi(double x) { return sinpi(x); }
+__device__ __forceinline__ float ktan(float x) { return tanf(x); }
+__device__ __forceinline__ double ktan(double x) { return tan(x); }
+__device__ __forceinline__ float ktrunc(float x) { return truncf(x); }
+__device__ __forceinline__ double ktrunc(double x) { return trunc(x); }
+__device__ __forceinline__ float ky0(float x) { return y0f(x); }
+__device__ __forceinline__ double ky0(double x) { return y0(x); }
+__device__ __forceinline__ float ky1(float x) { return y1f(x); }
+__device__ __forceinline__ double ky1(double x) { return y1(x); }
+__device__ __forceinline__ float kpow(float x, float y) { return powf(x, y); }
+__device__ __forceinline__ double kpow(double x, double y) { return pow(x, y); }
 }  // namespace knet8

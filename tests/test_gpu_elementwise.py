@@ -250,3 +250,79 @@ def test_broadcast_entry_points_reject_bad_strides_and_handle_misaligned_views(k
     knet.knet8("mul_32_17", xd.ptr, yd.ptr, z2.ptr, st[0].ptr, st[1].ptr, st[2].ptr, 120, 3)
     assert bits_equal(knet.Array(z2), x * y)
     lib.check()
+
+
+# name -> (reference, sampling interval, floor, ulp bound).  The elementary functions are checked against numpy evaluated in
+# fp64 on the same T-valued inputs; the special functions against mpmath at 120 bits (scipy's fp64 erfc is itself tens of ulp
+# off in the far tail).  The error is measured at max(|result|, floor), floor being the magnitude at which the routine's absolute
+# error lives (trig and Bessel functions near their zeros, lgamma near 1 and 2).  Bounds: what the device libm delivers, measured
+# (gamma 5 ulp, erfcx 7 ulp in fp64, everything else <= 4).
+def _libm_table():
+    import mpmath as mp
+    mp.mp.prec = 120
+
+    def viamp(f):
+        return lambda x: np.array([float(mp.mpf(f(mp.mpf(float(v))).real)) for v in x])
+    return {
+        "acos": (np.arccos, (-1, 1), 1.0, 4), "acosh": (np.arccosh, (1, 50), 0, 4), "asin": (np.arcsin, (-1, 1), 0, 4), "asinh": (np.arcsinh, (-50, 50), 0, 4),
+        "atan": (np.arctan, (-50, 50), 0, 4), "atanh": (np.arctanh, (-0.999, 0.999), 0, 4), "cbrt": (np.cbrt, (-50, 50), 0, 4), "ceil": (np.ceil, (-50, 50), 0, 0),
+        "cos": (np.cos, (-20, 20), 1.0, 4), "cosh": (np.cosh, (-20, 20), 0, 4), "cospi": (lambda v: np.cos(np.pi * (v % 2)), (-20, 20), 1.0, 4),
+        "exp10": (lambda v: np.power(10.0, v), (-20, 20), 0, 4), "exp2": (np.exp2, (-50, 50), 0, 4),
+        "expm1": (np.expm1, (-20, 20), 0, 4), "floor": (np.floor, (-50, 50), 0, 0), "log10": (np.log10, (1e-3, 1e3), 0.01, 4), "log1p": (np.log1p, (-0.99, 50), 0, 4),
+        "log2": (np.log2, (1e-3, 1e3), 0.01, 4), "sin": (np.sin, (-20, 20), 1.0, 4), "sinh": (np.sinh, (-20, 20), 0, 4), "sinpi": (lambda v: np.sin(np.pi * (v % 2)), (-20, 20), 1.0, 4),
+        "tan": (np.tan, (-1.5, 1.5), 0, 4), "trunc": (np.trunc, (-50, 50), 0, 0), "round": (np.rint, (-50, 50), 0, 0),
+        "erf": (viamp(mp.erf), (-4, 4), 0, 4), "erfc": (viamp(mp.erfc), (-4, 6), 0, 4), "erfcx": (viamp(lambda v: mp.exp(v * v) * mp.erfc(v)), (-3, 30), 0, 8),
+        "erfinv": (viamp(mp.erfinv), (-0.999, 0.999), 0, 4), "erfcinv": (viamp(lambda v: mp.erfinv(1 - v)), (0.001, 1.999), 0.01, 4),
+        "j0": (viamp(lambda v: mp.besselj(0, v)), (-30, 30), 1.0, 4), "j1": (viamp(lambda v: mp.besselj(1, v)), (-30, 30), 1.0, 4),
+        "y0": (viamp(lambda v: mp.bessely(0, v)), (0.01, 30), 1.0, 4), "y1": (viamp(lambda v: mp.bessely(1, v)), (0.01, 30), 1.0, 4),
+        "lgamma": (viamp(mp.loggamma), (0.01, 50), 1.0, 4), "gamma_impl": (viamp(mp.gamma), (0.05, 30), 0, 8),
+    }
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_libm_unary_table(knet, dt):
+    """The plain libm rows of the reference's unary table (src/libknet8/ops.jl:6-66)."""
+    rng = np.random.default_rng(21)
+    for name, (ref, (lo, hi), floor, tol) in _libm_table().items():
+        x = rng.uniform(lo, hi, size=2001).astype(dt)
+        x = x[(x >= lo) & (x <= hi)]
+        if name in ("cospi", "sinpi"):
+            x = (np.round(x * 64) / 64).astype(dt)  # exactly representable arguments, so that the reduction mod 2 in the checker is exact
+        if name == "round":
+            x[:8] = dt(0.5) + np.arange(-4, 4).astype(dt)  # ties go to even, as Julia's round
+        got = knet.Array(knet.unary_op(name, knet.KnetArray(x)))
+        with np.errstate(all="ignore"):
+            want = np.asarray(ref(x.astype(np.float64)), dtype=np.float64)
+        err = ulp_diff(got, want, scale=np.maximum(np.abs(want), floor))
+        assert err.max() <= tol + 0.5, (name, float(err.max()), float(x[np.argmax(err)]))
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_pow_and_comparisons(knet, dt):
+    rng = np.random.default_rng(22)
+    x = rng.integers(-3, 4, size=(33, 17)).astype(dt)
+    y = rng.integers(-3, 4, size=(33, 17)).astype(dt)
+    b = rng.integers(-3, 4, size=(33, 1)).astype(dt)
+    xd, yd, bd = knet.KnetArray(x), knet.KnetArray(y), knet.KnetArray(b)
+    for name, f in (("eq", np.equal), ("ne", np.not_equal), ("gt", np.greater), ("ge", np.greater_equal), ("lt", np.less), ("le", np.less_equal)):
+        assert bits_equal(knet.Array(knet.broadcast_op(name, xd, yd)), f(x, y).astype(dt)), name
+        assert bits_equal(knet.Array(knet.broadcast_op(name, xd, bd)), f(x, b).astype(dt)), name
+        assert bits_equal(knet.Array(knet.broadcast_op(name, bd, xd)), f(b, x).astype(dt)), name
+        assert bits_equal(knet.Array(knet.broadcast_op(name, xd, 1.0)), f(x, dt(1)).astype(dt)), name
+        assert bits_equal(knet.Array(knet.broadcast_op(name, 1.0, xd)), f(dt(1), x).astype(dt)), name
+    p = rng.uniform(0.1, 4, size=(33, 17)).astype(dt)
+    q = rng.uniform(-3, 3, size=(33, 17)).astype(dt)
+    got = knet.Array(knet.broadcast_op("pow", knet.KnetArray(p), knet.KnetArray(q)))
+    want = np.power(p.astype(np.float64), q.astype(np.float64))
+    assert ulp_diff(got, want.astype(dt)).max() <= 4
+    got = knet.Array(knet.broadcast_op("pow", knet.KnetArray(p), 2.0))
+    assert ulp_diff(got, (p.astype(np.float64) ** 2).astype(dt)).max() <= 2
+    got = knet.Array(knet.broadcast_op("pow", 2.0, knet.KnetArray(q)))
+    assert ulp_diff(got, np.exp2(q.astype(np.float64)).astype(dt)).max() <= 2
+    # invxback: -dy*y*y in that order, exact against the same IEEE operations in numpy
+    dy = rng.standard_normal(1000).astype(dt)
+    yy = rng.standard_normal(1000).astype(dt)
+    got = knet.Array(knet.back11_op("invxback", knet.KnetArray(dy), knet.KnetArray(yy)))
+    assert bits_equal(got, ((-dy) * yy) * yy)
+    knet.libknet8().check()
