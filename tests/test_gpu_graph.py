@@ -56,3 +56,56 @@ def test_captured_mlp_step_matches_eager_on_every_replay(knet, oracle):
         lib.check()
     finally:
         lib.stream = old_stream
+
+
+def test_captured_step_with_fused_layers_dropout_and_split_reductions(knet, oracle):
+    """A deeper net whose hidden layers are the fused bias+relu+dropout launches: the backward kernels split their bias-gradient sums
+    over several workgroups (ticket counters and partial buffers live in the per-stream scratch), which a graph replays as is."""
+    rng = np.random.default_rng(82)
+    lib = knet.libknet8()
+    old_stream = lib.stream
+    try:
+        sizes = [96, 256, 512, 7]
+        batch = 300
+        ws = []
+        for i in range(3):
+            ws += [(rng.standard_normal((sizes[i + 1], sizes[i])) * 0.1).astype(np.float32), (rng.standard_normal((sizes[i + 1], 1)) * 0.1).astype(np.float32)]
+        params = [knet.Param(knet.KnetArray(w)) for w in ws]
+        xh = rng.random((96, batch), dtype=np.float32)
+        x = knet.KnetArray(xh)
+        labels_h = rng.integers(0, 8, size=batch)
+        labels = knet.KnetArray(labels_h.astype(np.int32))
+        uni_h = [rng.random((sizes[i + 1], batch), dtype=np.float32) for i in range(2)]
+        uni = [knet.KnetArray(u) for u in uni_h]
+        count = int(np.count_nonzero(labels_h))
+
+        def step():
+            def loss():
+                h = x
+                for i in range(0, 4, 2):
+                    h = knet.bias_act(knet.matmul(params[i], h), params[i + 1], act="relu", pdrop=0.5, uniform=uni[i // 2])
+                h = knet.add(knet.matmul(params[4], h), params[5])
+                return knet.nll(h, labels, fused=True, count=count)
+            J = knet.diff(loss)
+            return [J.value] + [knet.grad(J, p) for p in params]
+
+        eager = [knet.Array(o) for o in step()]
+        loss_ref, grads_ref = oracle.mlp_backward(ws, xh, labels_h, pdrop=0.5, uniforms=uni_h)
+        assert abs(float(eager[0].ravel()[0]) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
+        g = knet.capture(step)
+        for r in range(4):
+            g.replay()
+            knet.synchronize()
+            out = [knet.Array(o) for o in g.outputs]
+            assert abs(float(out[0].ravel()[0]) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref)), r
+            for got, want in zip(out[1:], grads_ref):
+                assert rel(got, want) <= 1e-4, r
+            for got, want in zip(out, eager):   # same kernels, same order: a replay repeats the eager bits
+                assert np.array_equal(got, want), r
+            # eager split reductions on the same stream between replays share the scratch with the graph's kernels
+            big = knet.KnetArray(rng.integers(-3, 4, size=(512, 4096)).astype(np.float32))
+            assert np.array_equal(knet.Array(knet.sum(big, dims=2)).ravel(), knet.Array(big).sum(axis=1))
+        del g
+        lib.check()
+    finally:
+        lib.stream = old_stream
