@@ -88,6 +88,12 @@ def primitive(fwd):
     return wrapper
 
 
+def selective(back):
+    """Marks a gradient function ``back(dy, need)`` that computes only the gradients whose ``need`` entry is true."""
+    back.selective = True
+    return back
+
+
 def addto(a, b):
     """``addto!(a,b)``: accumulate a gradient (src/autograd_gpu/addto.jl:7-10: ``axpy!(1,b,a)``)."""
     if a is None:
@@ -127,7 +133,12 @@ def diff(f):
     for node in reversed(tape.nodes):
         if node.outgrad is None or node.back is None:
             continue
-        grads = node.back(node.outgrad)
+        if getattr(node.back, "selective", False):
+            # like AutoGrad, which evaluates a primitive's gradient expression only for the arguments that are tracked:
+            # the input layer's product never computes the gradient wrt the data, a constant operand of .* is not summed
+            grads = node.back(node.outgrad, tuple(p is not None for p in node.parents))
+        else:
+            grads = node.back(node.outgrad)
         for parent, g in zip(node.parents, grads):
             if parent is not None and g is not None:
                 parent.outgrad = addto(parent.outgrad, g)

@@ -8,7 +8,7 @@ operand had size 1 and the result did not, then reshape to the operand's size.
 """
 import numpy as np
 
-from .autograd import primitive
+from .autograd import primitive, selective
 from .karray import KnetArray
 from .libknet8 import knet8
 from .reduction import sum as ksum
@@ -147,18 +147,19 @@ def _neg(a):
 @primitive
 def add(x, y):
     """``x .+ y``; gradients ``unbroadcast(x,dy)``, ``unbroadcast(y,dy)``."""
-    return broadcast_op("add", x, y), (lambda dy: (unbroadcast(x, dy), unbroadcast(y, dy)))
+    return broadcast_op("add", x, y), selective(lambda dy, need=(True, True): (unbroadcast(x, dy) if need[0] else None, unbroadcast(y, dy) if need[1] else None))
 
 
 @primitive
 def sub(x, y):
-    return broadcast_op("sub", x, y), (lambda dy: (unbroadcast(x, dy), unbroadcast(y, _neg(dy))))
+    return broadcast_op("sub", x, y), selective(lambda dy, need=(True, True): (unbroadcast(x, dy) if need[0] else None, unbroadcast(y, _neg(dy)) if need[1] else None))
 
 
 @primitive
 def mul(x, y):
     """``x .* y``; gradients ``unbroadcast(x, dy.*y)``, ``unbroadcast(y, dy.*x)``."""
-    return broadcast_op("mul", x, y), (lambda dy: (unbroadcast(x, broadcast_op("mul", dy, y)), unbroadcast(y, broadcast_op("mul", dy, x))))
+    return broadcast_op("mul", x, y), selective(lambda dy, need=(True, True): (unbroadcast(x, broadcast_op("mul", dy, y)) if need[0] else None,
+                                                                                unbroadcast(y, broadcast_op("mul", dy, x)) if need[1] else None))
 
 
 def div(x, y):

@@ -523,6 +523,8 @@ KNET8_API void knet8_meminfo(size_t* out4);
 KNET8_API int knet8_memcpy(void* dst, const void* src, size_t nbytes, int kind, hipStream_t stream);
 KNET8_API int knet8_device_count(void);
 KNET8_API int knet8_set_device(int dev);
+/* non-blocking streams; destroying one waits for its work and frees the reduction scratch the library keeps for it (destroy graphs
+   captured on it first) */
 KNET8_API hipStream_t knet8_stream_create(void);
 KNET8_API void knet8_stream_destroy(hipStream_t stream);
 KNET8_API int knet8_synchronize(hipStream_t stream);

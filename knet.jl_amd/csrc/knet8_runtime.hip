@@ -76,6 +76,11 @@ static StreamScratch& scratch_of(hipStream_t stream) {
   return g_scratch[std::make_pair(dev, stream)];
 }
 
+__global__ __launch_bounds__(256) void zero_counters_kernel(unsigned* c, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) c[i] = 0u;
+}
+
 Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   StreamScratch& s = scratch_of(stream);
@@ -93,9 +98,14 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
     size_t want = ncounters < 4096 ? 4096 : 2 * ncounters;
     s.counters = nullptr;
     s.ncounters = 0;
-    if (ok(hipMalloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned)), "hipMalloc(reduction counters)") &&
-        ok(hipMemset(s.counters, 0, want * sizeof(unsigned)), "hipMemset(reduction counters)"))
-      s.ncounters = want;
+    // Zeroed by a fill kernel on the launching stream itself, so that the zeroing is ordered before the kernel that is about to
+    // use the counters.  (A hipMemset goes to the null stream, which a non-blocking stream does not wait for: on recycled memory
+    // the first split kernel on a new stream could then count on top of garbage and leave its tickets non-zero for good.  A fill
+    // kernel is also what a stream capture can record safely.)
+    if (ok(hipMalloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned)), "hipMalloc(reduction counters)")) {
+      hipLaunchKernelGGL(zero_counters_kernel, dim3((unsigned)((want + 255) / 256)), dim3(256), 0, stream, s.counters, want);
+      if (ok(hipGetLastError(), "zero_counters_kernel")) s.ncounters = want;
+    }
   }
   Workspace w = {s.partial, s.counters};
   return w;
@@ -246,7 +256,27 @@ KNET8_API hipStream_t knet8_stream_create(void) {
 }
 
 KNET8_API void knet8_stream_destroy(hipStream_t stream) {
-  if (stream) ok(hipStreamDestroy(stream), "hipStreamDestroy");
+  if (!stream) return;
+  // The stream's reduction scratch goes with it (a later stream may get the same handle and must start from its own, freshly
+  // zeroed counters).  Graphs captured on the stream hold the scratch addresses: destroy them first.
+  ok(hipStreamSynchronize(stream), "hipStreamSynchronize");
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    auto it = g_scratch.find(std::make_pair(dev, stream));
+    if (it != g_scratch.end()) {
+      StreamScratch& s = it->second;
+      if (s.partial) (void)hipFree(s.partial);
+      if (s.counters) (void)hipFree(s.counters);
+      if (s.scalar) (void)hipFree(s.scalar);
+      for (void* p : s.retired) (void)hipFree(p);
+      if (s.t0) (void)hipEventDestroy(s.t0);
+      if (s.t1) (void)hipEventDestroy(s.t1);
+      g_scratch.erase(it);
+    }
+  }
+  ok(hipStreamDestroy(stream), "hipStreamDestroy");
 }
 
 KNET8_API int knet8_synchronize(hipStream_t stream) { return ok(hipStreamSynchronize(stream), "hipStreamSynchronize") ? 0 : -1; }

@@ -4,7 +4,7 @@ Mirrors src/knetarrays/linalg.jl: ``A*B``, the transposition-free gradient forms
 (``:11-18``), ``gemm!`` (``:26-52``, cuBLAS there, hipBLASLt here through ``gemm_S``), ``axpy!`` (``:58-73``)
 and ``scal!`` (``:75-90``).
 """
-from .autograd import primitive
+from .autograd import primitive, selective
 from .karray import KnetArray
 from .libknet8 import knet8, libknet8
 
@@ -49,7 +49,7 @@ def At_mul_B(A, B):
 @primitive
 def matmul(x1, x2):
     """``x1*x2`` with ``@primitive1 *(x1,x2),dy  A_mul_Bt(dy,x2)  At_mul_B(x1,dy)`` (src/knetarrays/linalg.jl:15)."""
-    return A_mul_B(x1, x2), (lambda dy: (A_mul_Bt(dy, x2), At_mul_B(x1, dy)))
+    return A_mul_B(x1, x2), selective(lambda dy, need=(True, True): (A_mul_Bt(dy, x2) if need[0] else None, At_mul_B(x1, dy) if need[1] else None))
 
 
 def mat(x):

@@ -150,3 +150,27 @@ def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
     with pytest.raises(ValueError):
         knet.gemm("N", "N", 1, knet.KnetArray(np.zeros((3, 4), dt)), knet.KnetArray(np.zeros((5, 2), dt)), 0, knet.KnetArray(np.zeros((3, 2), dt)))
     knet.libknet8().check()
+
+
+def test_first_split_reduction_on_a_new_stream_over_recycled_memory(knet):
+    """The ticket counters of a stream are allocated at its first split reduction and must be zero before that kernel counts on
+    them, whatever the driver's memory held before: they are zeroed on the launching stream itself.  (A non-blocking stream does
+    not wait for null-stream work, so zeroing there would race with the first kernel.)"""
+    fn = knet.libknet8().fn
+    rng = np.random.default_rng(7)
+    x = rng.integers(-3, 4, size=(512, 4096)).astype(np.float32)
+    d = knet.KnetArray(x)
+    want = x.sum(axis=1)
+    for _ in range(6):
+        # dirty a spread of small and medium device blocks and hand them back to the driver
+        junk = [knet.KnetArray(np.full(n, np.float32(np.nan))) for n in (1024, 4096, 16384, 65536) for _ in range(8)]
+        del junk
+        fn["knet8_trim"]()
+        s = fn["knet8_stream_create"]()
+        y = knet.KnetArray(np.zeros(512, np.float32))
+        for _ in range(3):
+            fn["sum_32_21_stream"](x.size, d.ptr, 1, 512, y.ptr, s)
+            fn["knet8_synchronize"](s)
+            assert np.array_equal(knet.Array(y), want)
+        fn["knet8_stream_destroy"](s)
+    knet.libknet8().check()

@@ -123,3 +123,24 @@ def test_block_index_parameters_follow_indexparams(knet):
         ip((37, 21), (0, 3), None)
     with pytest.raises(IndexError):
         ip((37, 21), None, 22)
+
+
+def test_tape_computes_only_the_gradients_that_are_needed(knet, rec, monkeypatch):
+    # AutoGrad evaluates a primitive's gradient expression only for tracked arguments: the input layer's product has no
+    # gradient wrt the data (src/knetarrays/linalg.jl:15 declares one expression per argument)
+    calls, arr = rec
+    gemms = []
+    lib = knet.libknet8()
+    monkeypatch.setattr(lib, "call", lambda fun, *a: gemms.append((fun, a[0], a[1])) or 0)
+    w1, b1, w2, b2 = (knet.Param(arr(d)) for d in ((64, 784), (64, 1), (10, 64), (10, 1)))
+    x, c = arr((784, 100)), arr((10, 100))
+
+    def loss():
+        h = knet.relu(knet.add(knet.matmul(w1, x), b1))
+        return knet.sum(knet.mul(knet.add(knet.matmul(w2, h), b2), c))
+    n0 = len(calls)
+    J = knet.diff(loss)
+    assert [g[1:] for g in gemms if g[0].startswith("gemm")] == [(b"N", b"N"), (b"N", b"N"), (b"N", b"T"), (b"T", b"N"), (b"N", b"T")]  # no dx for layer 1
+    assert all(knet.grad(J, p) is not None for p in (w1, b1, w2, b2))
+    names = [c_[0] for c_ in calls[n0:]]
+    assert names.count("mul_32_11") == 2  # forward product and the gradient wrt its tracked operand only
