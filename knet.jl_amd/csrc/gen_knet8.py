@@ -547,7 +547,8 @@ KNET8_API void knet8_graph_destroy(void* graph);
 KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
-   device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity) */
+   device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
+   key 2: small products with 16 to this many 32x32 output tiles and k >= 97 split k inside one workgroup per tile (default 256; 1: never) */
 KNET8_API int knet8_tune(int key, int value);
 /* replaces cublasSgemm_v2 / cublasDgemm_v2 at src/knetarrays/linalg.jl:26-52 (column-major, transa/transb in 'N','T'): hipBLASLt */
 KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc, hipStream_t stream);

@@ -93,6 +93,99 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T 
     }
 }
 
+// ---- k split inside the workgroup ------------------------------------------------------------------------------
+// For the very small products (a few output tiles, k in the tens to hundreds) the cross-workgroup ticket costs more than the
+// arithmetic: three dependent memory round trips after the last product.  Here one wave owns the whole 32x32 tile for a slice
+// of k (4x4 outputs per lane) and the KS waves of a workgroup take KS slices; their partial tiles meet in LDS.  Every wave runs
+// the same number of k steps (loads beyond its slice or beyond k read zeros), so the workgroup barriers line up.
+template <typename T, bool TA, bool TB, int KS>
+__global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda,
+                                                              const T* __restrict__ B, int ldb, T beta, T* C, int ldc, int kslice) {
+  __shared__ T As[KS][kGsTile][kGsTile + 1];  // As[w][kk][i] = op(A)(i0+i, k0+kk) of wave w's current step
+  __shared__ T Bs[KS][kGsTile][kGsTile + 1];
+  const int tiles_m = (m + kGsTile - 1) / kGsTile;
+  const int tile = blockIdx.x;
+  const int i0 = (tile % tiles_m) * kGsTile, j0 = (tile / tiles_m) * kGsTile;
+  const int w = threadIdx.x / kWave, l = threadIdx.x & (kWave - 1);
+  const int tx = l & 7, ty = l >> 3;  // outputs (tx + 8a, ty + 8b), a, b = 0..3
+  const int lo = l & 31, hi = l >> 5;  // loader coordinates: `lo` along the operand's contiguous axis
+  const int kbeg = w * kslice;
+  int kend = kbeg + kslice;
+  if (kend > k) kend = k;
+  T acc[4][4];
+#pragma unroll
+  for (int a = 0; a < 4; a++)
+#pragma unroll
+    for (int b = 0; b < 4; b++) acc[a][b] = T(0);
+  T ga[16], gb[16];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int h = hi + 2 * r;
+      if (!TA) { const int i = i0 + lo, kk = k0 + h; ga[r] = (i < m && kk < kend) ? A[i + (long)kk * lda] : T(0); }
+      else     { const int kk = k0 + lo, i = i0 + h; ga[r] = (i < m && kk < kend) ? A[kk + (long)i * lda] : T(0); }
+      if (!TB) { const int kk = k0 + lo, j = j0 + h; gb[r] = (j < n && kk < kend) ? B[kk + (long)j * ldb] : T(0); }
+      else     { const int j = j0 + lo, kk = k0 + h; gb[r] = (j < n && kk < kend) ? B[j + (long)kk * ldb] : T(0); }
+    }
+  };
+  fetch(kbeg);
+  for (int k0 = kbeg; k0 < kbeg + kslice; k0 += kGsTile) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int h = hi + 2 * r;
+      if (!TA) As[w][h][lo] = ga[r]; else As[w][lo][h] = ga[r];
+      if (!TB) Bs[w][lo][h] = gb[r]; else Bs[w][h][lo] = gb[r];
+    }
+    __syncthreads();
+    if (k0 + kGsTile < kbeg + kslice) fetch(k0 + kGsTile);
+#pragma unroll 8
+    for (int kk = 0; kk < kGsTile; kk++) {
+      T av[4], bv[4];
+#pragma unroll
+      for (int a = 0; a < 4; a++) av[a] = As[w][kk][tx + 8 * a];
+#pragma unroll
+      for (int b = 0; b < 4; b++) bv[b] = Bs[w][kk][ty + 8 * b];
+#pragma unroll
+      for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = kfma(av[a], bv[b], acc[a][b]);
+    }
+    __syncthreads();
+  }
+  if (KS > 1) {
+    // partial tiles into LDS (each wave reuses its own staging area: 32*33 >= 1024 elements), summed in wave order
+    T* mine = &As[w][0][0];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+      for (int b = 0; b < 4; b++) mine[(ty + 8 * b) * kGsTile + tx + 8 * a] = acc[a][b];
+    __syncthreads();
+    for (int o = threadIdx.x; o < kGsTile * kGsTile; o += KS * kWave) {
+      T sum = T(0);
+#pragma unroll
+      for (int q = 0; q < KS; q++) sum += (&As[q][0][0])[o];
+      const int i = i0 + (o & (kGsTile - 1)), j = j0 + o / kGsTile;
+      if (i < m && j < n) {
+        T* c = C + i + (long)j * ldc;
+        const T v = alpha * sum;
+        *c = beta == T(0) ? v : v + beta * *c;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+      for (int b = 0; b < 4; b++) {
+        const int i = i0 + tx + 8 * a, j = j0 + ty + 8 * b;
+        if (i < m && j < n) {
+          T* c = C + i + (long)j * ldc;
+          const T v = alpha * acc[a][b];
+          *c = beta == T(0) ? v : v + beta * *c;
+        }
+      }
+  }
+}
+
 // True if this product should use the small kernel.
 inline bool gemm_is_small(int m, int n, int k) { return 2.0 * m * n * (double)k <= 1.0e8 && (long)m * n <= 262144; }
 
@@ -101,6 +194,28 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
                               T beta, T* C, int ldc) {
   const long tiles = (long)((m + kGsTile - 1) / kGsTile) * ((n + kGsTile - 1) / kGsTile);
   const long ksteps = (k + kGsTile - 1) / kGsTile;
+  if (ksteps >= 4 && tiles >= 16 && tiles <= tuning(kTuneGemmWaveTiles)) {
+    // Enough tiles to occupy a fair share of the CUs and a k long enough that walking it serially would dominate: one wave per k
+    // slice inside the workgroup, no cross-workgroup combine.  Measured (us per call, back-to-back launches, this kernel vs the
+    // one below): 128^3 6.1/7.1, 256^3 6.3/9.9, 512x300x256 6.4/10.0, 512x256x300 NT 9.2/12.4, 256x300x512 TN 10.4/17.3.  With fewer
+    // tiles (64x100x784: 15.4/11.8) one CU's LDS bandwidth limits a 16-wave workgroup and the cross-workgroup split wins; with
+    // short k (256x300x96: 6.7/5.1) the 256-lane tiles win.
+    constexpr int kMaxKs = sizeof(T) == 4 ? 16 : 8;  // 2 * 32*33 elements of LDS per wave
+    int ks = 1;
+    while (ks < kMaxKs && ks < ksteps) ks *= 2;
+    const int kslice = (int)((ksteps + ks - 1) / ks) * kGsTile;
+    const dim3 grid((unsigned)tiles);
+#define KNET8_GW1(TA, TB, KS) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KS>), grid, dim3(KS * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kslice)
+#define KNET8_GW(TA, TB) do { if (ks == 1) KNET8_GW1(TA, TB, 1); else if (ks == 2) KNET8_GW1(TA, TB, 2); else if (ks == 4) KNET8_GW1(TA, TB, 4); \
+                              else if (ks == 8) KNET8_GW1(TA, TB, 8); else { if constexpr (kMaxKs >= 16) KNET8_GW1(TA, TB, kMaxKs); } } while (0)
+    if (!ta && !tb) KNET8_GW(false, false);
+    else if (ta && !tb) KNET8_GW(true, false);
+    else if (!ta && tb) KNET8_GW(false, true);
+    else KNET8_GW(true, true);
+#undef KNET8_GW
+#undef KNET8_GW1
+    return;
+  }
   long P = 1;
   const long ncu = tuning(kTuneNumCUs);
   if (tiles * 8 <= ncu) P = ncu / (2 * tiles);  // measured: splitting pays only when the tiles cover a small fraction of the CUs

@@ -28,7 +28,7 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
 void* scalar_slot(hipStream_t stream);
 void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes);
 
-enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneCount = 8 };
+enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneGemmWaveTiles = 2, kTuneCount = 8 };
 int tuning(int key);
 
 }  // namespace knet8

@@ -54,6 +54,7 @@ int tuning(int key) {
       g_tune[key] = 256;
     }
   }
+  if (key == kTuneGemmWaveTiles && g_tune[key] == 0) g_tune[key] = 256;  // at most this many output tiles (and at least 16): k is split inside the workgroup (1 switches that kernel off)
   return g_tune[key];
 }
 
