@@ -41,32 +41,34 @@ template <> __device__ __forceinline__ double dev_log<double>(double x) { return
 // ---- algorithms -------------------------------------------------------------------------------------
 // a, b: the (up to) two inputs.  kInputs==1: a = x.  kInputs==2: a = y, b = dy.
 // kHoldA: a must stay in registers between the reduction and the output pass (false: it is only needed in
-// the output pass and is streamed there).  term(): summand of the column sum.  out(): the result.
+// the output pass and is streamed there).  term(): summand of the column sum.  out(): the result.  kKeepTerm: the summand
+// replaces a in its register and the result is out_kept(term, fin) -- one exp per element instead of two, same bits.
 
 // y = (x - max) - log(sum(exp(x - max)))                      src/ops20/softmax.jl:42-47
 template <typename T> struct AlgoLogSoftmax {
-  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false;
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false, kKeepTerm = false;
   __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
   __device__ static T finish(T s) { return dev_log(s); }
   __device__ static T out(T a, T, T mx, T fin) { return (a - mx) - fin; }
 };
 // y = exp(x - max) / sum(exp(x - max))                          src/ops20/softmax.jl:53-59
 template <typename T> struct AlgoSoftmax {
-  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false;
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = false, kKeepTerm = true;
   __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
   __device__ static T finish(T s) { return s; }
   __device__ static T out(T a, T, T mx, T fin) { return dev_exp(a - mx) / fin; }
+  __device__ static T out_kept(T t, T fin) { return t / fin; }
 };
 // dx = dy - exp(y)*sum(dy)                                      src/ops20/softmax.jl:49-51
 template <typename T> struct AlgoLogSoftmaxBack {
-  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = false, kNll = false;
+  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = false, kNll = false, kKeepTerm = false;
   __device__ static T term(T, T b, T) { return b; }
   __device__ static T finish(T s) { return s; }
   __device__ static T out(T a, T b, T, T fin) { const T e = dev_exp(a); const T p = e * fin; return b - p; }
 };
 // dx = y*dy - y*sum(y*dy)                                       src/ops20/softmax.jl:61-63
 template <typename T> struct AlgoSoftmaxBack {
-  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = true, kNll = false;
+  static constexpr int kInputs = 2; static constexpr bool kNeedMax = false, kHoldA = true, kNll = false, kKeepTerm = false;
   __device__ static T term(T a, T b, T) { return a * b; }
   __device__ static T finish(T s) { return s; }
   __device__ static T out(T a, T b, T, T fin) { const T p = a * b; const T q = a * fin; return p - q; }
@@ -76,7 +78,7 @@ template <typename T> struct AlgoSoftmaxBack {
 // src/ops20/loss.jl:37-41 and src/ops20/softmax.jl:49-51 -- and loss[col] = -lsm[label].  Label 0 skips
 // the column (dx = 0, loss = 0), as findindices does (src/ops20/loss.jl:125).
 template <typename T> struct AlgoNll {
-  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = true;
+  static constexpr int kInputs = 1; static constexpr bool kNeedMax = true, kHoldA = true, kNll = true, kKeepTerm = false;
   __device__ static T term(T a, T, T mx) { return dev_exp(a - mx); }
   __device__ static T finish(T s) { return dev_log(s); }
   __device__ static T out(T a, T, T mx, T fin) { return (a - mx) - fin; }  // lsm; the kernel finishes the job
@@ -155,7 +157,11 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
     for (int i = 0; i < ITEMS; i++)
       if (colok && i < cnt) {
 #pragma unroll
-        for (int e = 0; e < NV; e++) s = s + Algo::term(kHold ? ra[c][i][e] : T(0), kTwo ? rb[c][i][e] : T(0), mx);
+        for (int e = 0; e < NV; e++) {
+          const T t = Algo::term(kHold ? ra[c][i][e] : T(0), kTwo ? rb[c][i][e] : T(0), mx);
+          if constexpr (Algo::kKeepTerm && kHold) ra[c][i][e] = t;
+          s = s + t;
+        }
       }
     s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
     const T fin = Algo::finish(s);
@@ -170,7 +176,10 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
       }
       V vo;
 #pragma unroll
-      for (int e = 0; e < NV; e++) vo[e] = Algo::out(kHold ? ra[c][i][e] : va[e], kTwo ? rb[c][i][e] : T(0), mx, fin);
+      for (int e = 0; e < NV; e++) {
+        if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(ra[c][i][e], fin);
+        else vo[e] = Algo::out(kHold ? ra[c][i][e] : va[e], kTwo ? rb[c][i][e] : T(0), mx, fin);
+      }
       if (VEC) st_stream(reinterpret_cast<V*>(out + base + r), vo);
       else __builtin_nontemporal_store(vo[0], out + base + r);
     }
