@@ -316,6 +316,35 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=F
     return {"steps_per_sec": steps / dt, "ms_per_step": dt / steps * 1e3, "loss": lossv}
 
 
+def c_host_steps(K, steps=5000):
+    """The config-1 step driven by a compiled C99 host through the C ABI (tests/c_host/mlp_step.c), eager, no graph: what a host
+    with ccall-like call overhead (the reference's Julia) reaches.  None if no C compiler is at hand."""
+    import shutil
+    import subprocess
+    import tempfile
+    if shutil.which("gcc") is None:
+        return None
+    here = os.path.dirname(os.path.abspath(__file__))
+    libdir = os.path.dirname(K.LIB_PATH)
+    rng = np.random.default_rng(0)
+    with tempfile.TemporaryDirectory() as tmp:
+        exe, fin, fout = os.path.join(tmp, "mlp_step"), os.path.join(tmp, "in.bin"), os.path.join(tmp, "out.bin")
+        subprocess.check_call(["gcc", "-std=c99", "-D_POSIX_C_SOURCE=199309L", "-O2", "-I", os.path.join(here, "include"),
+                               os.path.join(here, "tests", "c_host", "mlp_step.c"), "-o", exe, "-L", libdir, "-lknet8",
+                               "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
+        with open(fin, "wb") as f:
+            for shape, scale in (((64, 784), 0.01), ((64, 1), 0.0), ((10, 64), 0.01), ((10, 1), 0.0)):
+                f.write((rng.standard_normal(shape) * scale).astype(np.float32).tobytes(order="F"))
+            f.write(rng.random((784, 100), dtype=np.float32).tobytes(order="F"))
+            f.write(rng.integers(1, 11, size=100).astype(np.int32).tobytes())
+        r = subprocess.run([exe, fin, fout, str(steps)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+        if r.returncode != 0:
+            raise RuntimeError("mlp_step failed: " + r.stderr)
+        rate = float(r.stdout.split()[-1])
+        loss = float(np.fromfile(fout, dtype=np.float32, count=1)[0])
+    return {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "loss": loss}
+
+
 def cpu_side_table():
     """The oracle's loops for the config 3-5 kernels, one thread, full shapes (each takes well under a second)."""
     from oracle import knet_oracle as ko
@@ -436,6 +465,7 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
             "config1 same graph with fused bias+relu layers": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
+            "config1 same step from a compiled C99 host through the C ABI (eager, 10 launches, fused layer kernels)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),

@@ -1,0 +1,105 @@
+/* A compiled host driving the C ABI directly, the way Knet's Julia code does through ccall: one forward + backward step of the
+ * MLP of examples/mnist-mlp/mlp.jl:25-35 (784-64-10, batch 100), every device operation an entry point of knet8.h.
+ *
+ *   mlp_step IN OUT [steps]
+ *
+ * IN holds, as raw little-endian data in this order: float W1[64*784], b1[64], W2[10*64], b2[10], x[784*100] (all column-major),
+ * int32 labels[100] (1-based).  OUT receives float loss, dW1[64*784], db1[64], dW2[10*64], db2[10].  With `steps` the step is then
+ * repeated that many times on a stream without host synchronisation and the rate is printed ("steps_per_sec N").
+ * Test infrastructure: the parity test compares OUT with the CPU oracle. */
+#include <stdio.h>
+#include <stdlib.h>
+#include <time.h>
+#include "knet8.h"
+
+enum { D0 = 784, D1 = 64, D2 = 10, NB = 100 };
+
+static float *dev(size_t n) {
+  float *p = (float *)knet8_malloc(n * sizeof(float));
+  if (!p) { fprintf(stderr, "knet8_malloc failed: %s\n", knet8_last_error()); exit(2); }
+  return p;
+}
+
+static void up(void *d, const void *h, size_t bytes) {
+  if (knet8_memcpy(d, h, bytes, 1, 0) != 0) { fprintf(stderr, "upload failed\n"); exit(2); }
+}
+
+struct net {
+  float *W1, *b1, *W2, *b2, *x, *z1, *y1, *z2, *s, *dx, *lossv, *db2, *dW2, *dy1, *dz1, *db1, *dW1;
+  int *labels;
+};
+
+static void step(struct net *n, hipStream_t st) {
+  /* forward: y1 = relu(W1*x .+ b1); s = W2*y1 .+ b2 */
+  gemm_32_stream('N', 'N', D1, NB, D0, 1.0f, n->W1, D1, n->x, D0, 0.0f, n->z1, D1, st);
+  biasrelu_32_stream(D1, NB, n->z1, n->b1, n->y1, st);
+  gemm_32_stream('N', 'N', D2, NB, D1, 1.0f, n->W2, D2, n->y1, D1, 0.0f, n->z2, D2, st);
+  add_32_12_stream(D2 * NB, n->z2, 1, D2 * NB, n->b2, 1, D2, n->s, st);
+  /* loss and its gradient wrt the scores in one pass */
+  nll_logsoftmax_back_32_stream(D2, NB, n->s, n->labels, 1.0f / NB, n->dx, n->lossv, st);
+  /* backward */
+  sum_32_21_stream(D2 * NB, n->dx, 1, D2, n->db2, st);                                              /* db2 = sum(dx; dims=2) */
+  gemm_32_stream('N', 'T', D2, D1, NB, 1.0f, n->dx, D2, n->y1, D1, 0.0f, n->dW2, D2, st);             /* dW2 = dx * y1'      */
+  gemm_32_stream('T', 'N', D1, NB, D2, 1.0f, n->W2, D2, n->dx, D2, 0.0f, n->dy1, D1, st);             /* dy1 = W2' * dx      */
+  reluback_biasgrad_32_stream(D1, NB, n->dy1, n->y1, n->dz1, n->db1, st);                             /* dz1, db1            */
+  gemm_32_stream('N', 'T', D1, D0, NB, 1.0f, n->dz1, D1, n->x, D0, 0.0f, n->dW1, D1, st);             /* dW1 = dz1 * x'      */
+}
+
+int main(int argc, char **argv) {
+  if (argc < 3) { fprintf(stderr, "usage: %s IN OUT [steps]\n", argv[0]); return 2; }
+  const long steps = argc > 3 ? atol(argv[3]) : 0;
+  const size_t nW1 = (size_t)D1 * D0, nW2 = (size_t)D2 * D1, nx = (size_t)D0 * NB;
+  const size_t nin = nW1 + D1 + nW2 + D2 + nx;
+  float *h = (float *)malloc(nin * sizeof(float));
+  int hl[NB];
+  FILE *f = fopen(argv[1], "rb");
+  if (!f || fread(h, sizeof(float), nin, f) != nin || fread(hl, sizeof(int), NB, f) != NB) { fprintf(stderr, "cannot read %s\n", argv[1]); return 2; }
+  fclose(f);
+  if (knet8_device_count() < 1) { fprintf(stderr, "no device\n"); return 3; }
+  struct net n;
+  n.W1 = dev(nW1); n.b1 = dev(D1); n.W2 = dev(nW2); n.b2 = dev(D2); n.x = dev(nx);
+  n.z1 = dev(D1 * NB); n.y1 = dev(D1 * NB); n.z2 = dev(D2 * NB); n.s = dev(D2 * NB); n.dx = dev(D2 * NB); n.lossv = dev(NB);
+  n.db2 = dev(D2); n.dW2 = dev(nW2); n.dy1 = dev(D1 * NB); n.dz1 = dev(D1 * NB); n.db1 = dev(D1); n.dW1 = dev(nW1);
+  n.labels = (int *)knet8_malloc(NB * sizeof(int));
+  const float *p = h;
+  up(n.W1, p, nW1 * 4); p += nW1;
+  up(n.b1, p, D1 * 4); p += D1;
+  up(n.W2, p, nW2 * 4); p += nW2;
+  up(n.b2, p, D2 * 4); p += D2;
+  up(n.x, p, nx * 4);
+  up(n.labels, hl, NB * sizeof(int));
+
+  hipStream_t st = knet8_stream_create();
+  step(&n, st);
+  const float loss = sum_32_20_stream(NB, n.lossv, st) / NB; /* blocks; the kernel leaves -logp of the labelled class per column */
+  const char *err = knet8_last_error();
+  if (err) { fprintf(stderr, "libknet8: %s\n", err); return 4; }
+
+  const size_t nout = 1 + nW1 + D1 + nW2 + D2;
+  float *o = (float *)malloc(nout * sizeof(float));
+  float *q = o;
+  *q++ = loss;
+  knet8_memcpy(q, n.dW1, nW1 * 4, 2, st); q += nW1;
+  knet8_memcpy(q, n.db1, D1 * 4, 2, st); q += D1;
+  knet8_memcpy(q, n.dW2, nW2 * 4, 2, st); q += nW2;
+  knet8_memcpy(q, n.db2, D2 * 4, 2, st);
+  f = fopen(argv[2], "wb");
+  if (!f || fwrite(o, sizeof(float), nout, f) != nout) { fprintf(stderr, "cannot write %s\n", argv[2]); return 2; }
+  fclose(f);
+
+  if (steps > 0) {
+    for (int i = 0; i < 20; i++) step(&n, st);
+    knet8_synchronize(st);
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (long i = 0; i < steps; i++) step(&n, st);
+    knet8_synchronize(st);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    const double dt = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+    printf("steps_per_sec %.1f\n", (double)steps / dt);
+    err = knet8_last_error();
+    if (err) { fprintf(stderr, "libknet8: %s\n", err); return 4; }
+  }
+  knet8_stream_destroy(st);
+  return 0;
+}
