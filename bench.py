@@ -270,6 +270,9 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=F
     def loss():
         h = x
         for i in range(0, len(params), 2):
+            if layers and pdrop == 0:
+                h = K.dense(params[i], h, params[i + 1], act="relu" if i < len(params) - 2 else None)
+                continue
             if layers and i < len(params) - 2:
                 h = K.bias_act(K.matmul(params[i], h), params[i + 1], act="relu", pdrop=pdrop, uniform=uni[i // 2] if pdrop > 0 else None)
                 continue
@@ -340,9 +343,10 @@ def c_host_steps(K, steps=5000):
         r = subprocess.run([exe, fin, fout, str(steps)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
         if r.returncode != 0:
             raise RuntimeError("mlp_step failed: " + r.stderr)
-        rate = float(r.stdout.split()[-1])
+        rates = dict(line.split() for line in r.stdout.strip().splitlines())
+        rate = float(rates["steps_per_sec"])
         loss = float(np.fromfile(fout, dtype=np.float32, count=1)[0])
-    return {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "loss": loss}
+    return {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "graph_replay_steps_per_sec": float(rates["graph_steps_per_sec"]), "loss": loss}
 
 
 def cpu_side_table():
@@ -464,8 +468,8 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager, fused nll)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, True),
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
-            "config1 same graph with fused bias+relu layers": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
-            "config1 same step from a compiled C99 host through the C ABI (eager, 10 launches, fused layer kernels)": c_host_steps(K),
+            "config1 same graph with dense layers (product, bias and relu in one launch)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
+            "config1 same step from a compiled C99 host through the C ABI (eager, 8 launches, fused layer kernels)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),

@@ -555,6 +555,13 @@ KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, floa
 KNET8_API int gemm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc);
 KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc, hipStream_t stream);
 KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc);
+/* dense layer in one call: C = act(alpha*op(A)*op(B) + bias[i]) with bias of length m and act 0 (none) or 1 (relu).  No counterpart in
+   the reference, which runs gemm!, the bias broadcast (src/knetarrays/binary.jl:61-95) and relu (src/ops20_gpu/activation.jl:17-29) as
+   three launches; same bits as that chain.  Small products fold bias and relu into the product kernel's output stage. */
+KNET8_API int gemm_bias_act_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc, hipStream_t stream);
+KNET8_API int gemm_bias_act_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc);
+KNET8_API int gemm_bias_act_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias, int act, double* C, int ldc, hipStream_t stream);
+KNET8_API int gemm_bias_act_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias, int act, double* C, int ldc);
 """
 
 HEADER_BOTTOM = """

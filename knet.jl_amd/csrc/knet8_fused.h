@@ -9,6 +9,7 @@
 // Every element goes through the same rounded operations as the separate launches, so dz and y are bit-identical
 // to the chain; db differs from the chain's sum only by summation order.
 #pragma once
+#include "knet8_elementwise.h"
 #include "knet8_reduce.h"
 
 namespace knet8 {

@@ -16,10 +16,21 @@ constexpr int kGsTile = 32;
 __device__ __forceinline__ float kfma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double kfma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
+// Output stage shared by the kernels below: v = alpha*acc [+ beta*C] [+ bias[i]] [relu].  Each step is one rounded operation, so
+// a product with bias and relu folded in gives the bits of the product followed by the separate bias-add and relu launches.
+template <typename T>
+__device__ __forceinline__ void gemm_store(T* c, T acc, T alpha, T beta, const T* bias, int i, int act) {
+  T v = alpha * acc;
+  if (beta != T(0)) v = v + beta * *c;
+  if (bias) v = v + bias[i];
+  if (act == 1) v = v != v ? v : (v > T(0) ? v : T(0));
+  *c = v;
+}
+
 template <typename T, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda,
-                                                         const T* __restrict__ B, int ldb, T beta, T* C, int ldc, int kchunk,
-                                                         unsigned P, T* partial, unsigned* counters) {
+                                                         const T* __restrict__ B, int ldb, T beta, T* C, int ldc, const T* bias, int act,
+                                                         int kchunk, unsigned P, T* partial, unsigned* counters) {
   __shared__ T As[kGsTile][kGsTile + 1];  // As[kk][i] = op(A)(i0+i, k0+kk)
   __shared__ T Bs[kGsTile][kGsTile + 1];  // Bs[kk][j] = op(B)(k0+kk, j0+j)
   __shared__ unsigned flag;
@@ -85,11 +96,7 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T 
 #pragma unroll
     for (int b = 0; b < 2; b++) {
       const int i = i0 + tx + 16 * a, j = j0 + ty + 16 * b;
-      if (i < m && j < n) {
-        T* c = C + i + (long)j * ldc;
-        const T v = alpha * acc[a][b];
-        *c = beta == T(0) ? v : v + beta * *c;
-      }
+      if (i < m && j < n) gemm_store(C + i + (long)j * ldc, acc[a][b], alpha, beta, bias, i, act);
     }
 }
 
@@ -100,7 +107,7 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T 
 // the same number of k steps (loads beyond its slice or beyond k read zeros), so the workgroup barriers line up.
 template <typename T, bool TA, bool TB, int KS>
 __global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda,
-                                                              const T* __restrict__ B, int ldb, T beta, T* C, int ldc, int kslice) {
+                                                              const T* __restrict__ B, int ldb, T beta, T* C, int ldc, const T* bias, int act, int kslice) {
   __shared__ T As[KS][kGsTile][kGsTile + 1];  // As[w][kk][i] = op(A)(i0+i, k0+kk) of wave w's current step
   __shared__ T Bs[KS][kGsTile][kGsTile + 1];
   const int tiles_m = (m + kGsTile - 1) / kGsTile;
@@ -165,11 +172,7 @@ __global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int
 #pragma unroll
       for (int q = 0; q < KS; q++) sum += (&As[q][0][0])[o];
       const int i = i0 + (o & (kGsTile - 1)), j = j0 + o / kGsTile;
-      if (i < m && j < n) {
-        T* c = C + i + (long)j * ldc;
-        const T v = alpha * sum;
-        *c = beta == T(0) ? v : v + beta * *c;
-      }
+      if (i < m && j < n) gemm_store(C + i + (long)j * ldc, sum, alpha, beta, bias, i, act);
     }
   } else {
 #pragma unroll
@@ -177,11 +180,7 @@ __global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int
 #pragma unroll
       for (int b = 0; b < 4; b++) {
         const int i = i0 + tx + 8 * a, j = j0 + ty + 8 * b;
-        if (i < m && j < n) {
-          T* c = C + i + (long)j * ldc;
-          const T v = alpha * acc[a][b];
-          *c = beta == T(0) ? v : v + beta * *c;
-        }
+        if (i < m && j < n) gemm_store(C + i + (long)j * ldc, acc[a][b], alpha, beta, bias, i, act);
       }
   }
 }
@@ -191,7 +190,7 @@ inline bool gemm_is_small(int m, int n, int k) { return 2.0 * m * n * (double)k 
 
 template <typename T>
 inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb,
-                              T beta, T* C, int ldc) {
+                              T beta, T* C, int ldc, const T* bias = nullptr, int act = 0) {
   const long tiles = (long)((m + kGsTile - 1) / kGsTile) * ((n + kGsTile - 1) / kGsTile);
   const long ksteps = (k + kGsTile - 1) / kGsTile;
   if (ksteps >= 4 && tiles >= 16 && tiles <= tuning(kTuneGemmWaveTiles)) {
@@ -205,7 +204,7 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
     while (ks < kMaxKs && ks < ksteps) ks *= 2;
     const int kslice = (int)((ksteps + ks - 1) / ks) * kGsTile;
     const dim3 grid((unsigned)tiles);
-#define KNET8_GW1(TA, TB, KS) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KS>), grid, dim3(KS * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kslice)
+#define KNET8_GW1(TA, TB, KS) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KS>), grid, dim3(KS * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
 #define KNET8_GW(TA, TB) do { if (ks == 1) KNET8_GW1(TA, TB, 1); else if (ks == 2) KNET8_GW1(TA, TB, 2); else if (ks == 4) KNET8_GW1(TA, TB, 4); \
                               else if (ks == 8) KNET8_GW1(TA, TB, 8); else { if constexpr (kMaxKs >= 16) KNET8_GW1(TA, TB, kMaxKs); } } while (0)
     if (!ta && !tb) KNET8_GW(false, false);
@@ -229,7 +228,7 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
   if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)tiles * P * kGsTile * kGsTile, (size_t)tiles);
   const dim3 grid((unsigned)(tiles * P)), block(256);
   T* partial = static_cast<T*>(ws.partial);
-#define KNET8_GS(TA, TB) hipLaunchKernelGGL((gemm_small_kernel<T, TA, TB>), grid, block, 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kchunk, (unsigned)P, partial, ws.counters)
+#define KNET8_GS(TA, TB) hipLaunchKernelGGL((gemm_small_kernel<T, TA, TB>), grid, block, 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kchunk, (unsigned)P, partial, ws.counters)
   if (!ta && !tb) KNET8_GS(false, false);
   else if (ta && !tb) KNET8_GS(true, false);
   else if (!ta && tb) KNET8_GS(false, true);

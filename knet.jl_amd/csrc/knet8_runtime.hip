@@ -2,6 +2,7 @@
 // storage, copies, stream/timer helpers and the hipBLASLt GEMM entry points.
 #include "knet8_runtime.h"
 #include "knet8_gemm_small.h"
+#include "knet8_fused.h"
 
 #include <hipblaslt/hipblaslt.h>
 
@@ -405,15 +406,34 @@ static bool lt_ok(hipblasStatus_t s, const char* what) {
   return false;
 }
 
+// bias != nullptr / act != 0: the dense-layer form C = act(alpha*op(A)*op(B) + bias[i]) (beta must be 0).  Small products fold it
+// into the output stage of the product kernel; large ones run the vendor product and then one in-place bias+activation pass.
+struct EpiNone { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb; } };
+struct EpiRelu { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb != zb ? zb : (zb > T(0) ? zb : T(0)); } };
+
 template <typename T>
 static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
-                hipStream_t stream) {
+                hipStream_t stream, const T* bias = nullptr, int act = 0) {
   if (m <= 0 || n <= 0) return 0;
   const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
   const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
   if (gemm_is_small(m, n, k)) {
-    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act);
     check_launch("gemm (small)");
+    return 0;
+  }
+  if (bias || act) {
+    if (ldc != m) { record_error("gemm_bias_act: ldc must equal m for large products"); return -1; }
+    const int rc = gemm<T>(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+    if (rc != 0) return rc;
+    if (bias) {
+      if (act == 1) launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiRelu());
+      else launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiNone());
+    } else {
+      record_error("gemm_bias_act: an activation without a bias is not provided");
+      return -1;
+    }
+    check_launch("gemm_bias_act (bias pass)");
     return 0;
   }
   const hipDataType dt = sizeof(T) == 4 ? HIP_R_32F : HIP_R_64F;
@@ -500,5 +520,29 @@ KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, doub
 KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta,
                       double* C, int ldc) {
   return gemm_64_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, 0);
+}
+
+static int check_epilogue(int act) {
+  if (act == 0 || act == 1) return 0;
+  knet8::record_error("gemm_bias_act: act must be 0 (none) or 1 (relu)");
+  return -1;
+}
+KNET8_API int gemm_bias_act_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias,
+                                      int act, float* C, int ldc, hipStream_t stream) {
+  if (check_epilogue(act) != 0) return -1;
+  return knet8::gemm<float>(transa, transb, m, n, k, alpha, A, lda, B, ldb, 0.0f, C, ldc, stream, bias, act);
+}
+KNET8_API int gemm_bias_act_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act,
+                               float* C, int ldc) {
+  return gemm_bias_act_32_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, bias, act, C, ldc, 0);
+}
+KNET8_API int gemm_bias_act_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias,
+                                      int act, double* C, int ldc, hipStream_t stream) {
+  if (check_epilogue(act) != 0) return -1;
+  return knet8::gemm<double>(transa, transb, m, n, k, alpha, A, lda, B, ldb, 0.0, C, ldc, stream, bias, act);
+}
+KNET8_API int gemm_bias_act_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias, int act,
+                               double* C, int ldc) {
+  return gemm_bias_act_64_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, bias, act, C, ldc, 0);
 }
 }

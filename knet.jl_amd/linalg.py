@@ -52,6 +52,37 @@ def matmul(x1, x2):
     return A_mul_B(x1, x2), selective(lambda dy, need=(True, True): (A_mul_Bt(dy, x2) if need[0] else None, At_mul_B(x1, dy) if need[1] else None))
 
 
+@primitive
+def dense(w, x, b, act=None):
+    """``f.(w*x .+ b)`` with ``b`` of shape (size(w,1), 1) and ``f`` relu or nothing, as ONE launch forward (``gemm_bias_act_S``: small products
+    fold bias and relu into the product kernel) and the fused activation-gradient + bias-gradient launch backward.  The reference
+    runs the same arithmetic as gemm!, a broadcast add and relu (src/knetarrays/linalg.jl:26-52, binary.jl:61-95,
+    src/ops20_gpu/activation.jl:17-29) and, backward, reluback and sum(dz;dims=2); the results carry the same bits."""
+    if act not in (None, "relu"):
+        raise ValueError("dense: act must be None or 'relu'")
+    x2 = mat(x)
+    m, k, n = _size2(w, 1), _size2(w, 2), x2.size(2)
+    if x2.size(1) != k or b.length != m or w.dtype != x2.dtype or b.dtype != w.dtype:
+        raise ValueError("DimensionMismatch: %r" % ((w.dims, x2.dims, b.dims),))
+    y = w.similar((m, n))
+    lib = libknet8()
+    c = w.ctype
+    rc = lib.call("gemm_bias_act_%s" % w.suffix, b"N", b"N", m, n, k, c(1), w.ptr, m, x2.ptr, k, b.ptr, 1 if act == "relu" else 0, y.ptr, m)
+    if rc != 0:
+        lib.check()
+        raise RuntimeError("gemm_bias_act failed")
+
+    def back(dy, need=(True, True, True)):
+        if act == "relu":
+            dz, db = y.similar(), b.similar()
+            knet8("reluback_biasgrad_%s" % w.suffix, m, n, dy.ptr, y.ptr, dz.ptr, db.ptr)
+        else:
+            from .reduction import reduce_op
+            dz, db = dy, (reduce_op("sum", dy, 2).reshape(b.dims) if need[2] else None)
+        return (A_mul_Bt(dz, x2) if need[0] else None, At_mul_B(w, dz).reshape(x.dims) if need[1] else None, db)
+    return y, selective(back)
+
+
 def mat(x):
     """``mat(x)``: reshape to a matrix keeping the last dimension as columns (used by the MLP example)."""
     from .autograd import Node

@@ -5,7 +5,8 @@
  *
  * IN holds, as raw little-endian data in this order: float W1[64*784], b1[64], W2[10*64], b2[10], x[784*100] (all column-major),
  * int32 labels[100] (1-based).  OUT receives float loss, dW1[64*784], db1[64], dW2[10*64], db2[10].  With `steps` the step is then
- * repeated that many times on a stream without host synchronisation and the rate is printed ("steps_per_sec N").
+ * repeated that many times on a stream without host synchronisation and the rate is printed ("steps_per_sec N"), then captured
+ * into a graph and replayed as often ("graph_steps_per_sec N").
  * Test infrastructure: the parity test compares OUT with the CPU oracle. */
 #include <stdio.h>
 #include <stdlib.h>
@@ -25,16 +26,14 @@ static void up(void *d, const void *h, size_t bytes) {
 }
 
 struct net {
-  float *W1, *b1, *W2, *b2, *x, *z1, *y1, *z2, *s, *dx, *lossv, *db2, *dW2, *dy1, *dz1, *db1, *dW1;
+  float *W1, *b1, *W2, *b2, *x, *y1, *s, *dx, *lossv, *db2, *dW2, *dy1, *dz1, *db1, *dW1;
   int *labels;
 };
 
 static void step(struct net *n, hipStream_t st) {
   /* forward: y1 = relu(W1*x .+ b1); s = W2*y1 .+ b2 */
-  gemm_32_stream('N', 'N', D1, NB, D0, 1.0f, n->W1, D1, n->x, D0, 0.0f, n->z1, D1, st);
-  biasrelu_32_stream(D1, NB, n->z1, n->b1, n->y1, st);
-  gemm_32_stream('N', 'N', D2, NB, D1, 1.0f, n->W2, D2, n->y1, D1, 0.0f, n->z2, D2, st);
-  add_32_12_stream(D2 * NB, n->z2, 1, D2 * NB, n->b2, 1, D2, n->s, st);
+  gemm_bias_act_32_stream('N', 'N', D1, NB, D0, 1.0f, n->W1, D1, n->x, D0, n->b1, 1, n->y1, D1, st);
+  gemm_bias_act_32_stream('N', 'N', D2, NB, D1, 1.0f, n->W2, D2, n->y1, D1, n->b2, 0, n->s, D2, st);
   /* loss and its gradient wrt the scores in one pass */
   nll_logsoftmax_back_32_stream(D2, NB, n->s, n->labels, 1.0f / NB, n->dx, n->lossv, st);
   /* backward */
@@ -58,7 +57,7 @@ int main(int argc, char **argv) {
   if (knet8_device_count() < 1) { fprintf(stderr, "no device\n"); return 3; }
   struct net n;
   n.W1 = dev(nW1); n.b1 = dev(D1); n.W2 = dev(nW2); n.b2 = dev(D2); n.x = dev(nx);
-  n.z1 = dev(D1 * NB); n.y1 = dev(D1 * NB); n.z2 = dev(D2 * NB); n.s = dev(D2 * NB); n.dx = dev(D2 * NB); n.lossv = dev(NB);
+  n.y1 = dev(D1 * NB); n.s = dev(D2 * NB); n.dx = dev(D2 * NB); n.lossv = dev(NB);
   n.db2 = dev(D2); n.dW2 = dev(nW2); n.dy1 = dev(D1 * NB); n.dz1 = dev(D1 * NB); n.db1 = dev(D1); n.dW1 = dev(nW1);
   n.labels = (int *)knet8_malloc(NB * sizeof(int));
   const float *p = h;
@@ -97,6 +96,22 @@ int main(int argc, char **argv) {
     clock_gettime(CLOCK_MONOTONIC, &t1);
     const double dt = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
     printf("steps_per_sec %.1f\n", (double)steps / dt);
+    err = knet8_last_error();
+    if (err) { fprintf(stderr, "libknet8: %s\n", err); return 4; }
+    /* the same step captured once into a graph and replayed */
+    if (knet8_graph_begin(st) != 0) { fprintf(stderr, "capture failed: %s\n", knet8_last_error()); return 4; }
+    step(&n, st);
+    void *g = knet8_graph_end(st);
+    if (!g) { fprintf(stderr, "capture failed: %s\n", knet8_last_error()); return 4; }
+    for (int i = 0; i < 20; i++) knet8_graph_launch(g, st);
+    knet8_synchronize(st);
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (long i = 0; i < steps; i++) knet8_graph_launch(g, st);
+    knet8_synchronize(st);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    const double dg = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+    printf("graph_steps_per_sec %.1f\n", (double)steps / dg);
+    knet8_graph_destroy(g);
     err = knet8_last_error();
     if (err) { fprintf(stderr, "libknet8: %s\n", err); return 4; }
   }

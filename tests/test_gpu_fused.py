@@ -156,3 +156,51 @@ def test_fused_layers_in_the_mlp_match_oracle(knet, oracle):
     with pytest.raises(ValueError):
         knet.bias_act(knet.KnetArray(np.zeros((4, 3))), knet.KnetArray(np.zeros((5, 1))))
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gemm_bias_act_carries_the_bits_of_the_three_launch_chain(knet, dt):
+    """C = act(alpha*op(A)*op(B) + bias) in one call against gemm, add_12 and relu through the same library: identical bits, over
+    the product kernels' plans (cross-workgroup split, in-workgroup k slices, plain tiles) and a vendor-library size."""
+    rng = np.random.default_rng(55)
+    S = sfx(dt)
+    lib = knet.libknet8()
+    shapes = [(64, 100, 784), (10, 100, 64), (33, 17, 5), (130, 131, 129), (512, 300, 256), (256, 300, 96), (1000, 700, 300)]
+    for (m, n, k) in shapes:
+        for ta, tb in (("N", "N"), ("T", "N"), ("N", "T")):
+            a = rng.standard_normal((m, k) if ta == "N" else (k, m)).astype(dt)
+            b = rng.standard_normal((k, n) if tb == "N" else (n, k)).astype(dt)
+            bias = rng.standard_normal((m, 1)).astype(dt)
+            A, B, bd = knet.KnetArray(a), knet.KnetArray(b), knet.KnetArray(bias)
+            z = knet.gemm(ta, tb, 1, A, B, 0, knet.KnetArray(np.zeros((m, n), dt)))
+            zb = knet.add(z, bd)
+            for act, want in ((0, knet.Array(zb)), (1, knet.Array(knet.relu(zb)))):
+                C = knet.KnetArray(np.full((m, n), np.nan, dt))
+                rc = lib.call("gemm_bias_act_%s" % S, ta.encode(), tb.encode(), m, n, k, A.ctype(1), A.ptr, a.shape[0], B.ptr, b.shape[0],
+                              bd.ptr, act, C.ptr, m)
+                assert rc == 0
+                assert bits_equal(knet.Array(C), want), (m, n, k, ta, tb, act)
+    lib.call("gemm_bias_act_%s" % S, b"N", b"N", 4, 4, 4, A.ctype(1), A.ptr, 4, B.ptr, 4, bd.ptr, 7, C.ptr, 4)
+    with pytest.raises(RuntimeError):
+        lib.check()
+
+
+def test_dense_primitive_in_the_mlp_matches_oracle(knet, oracle):
+    rng = np.random.default_rng(56)
+    ws = [(rng.standard_normal((64, 784)) * 0.01).astype(np.float32), (rng.standard_normal((64, 1)) * 0.1).astype(np.float32),
+          (rng.standard_normal((10, 64)) * 0.1).astype(np.float32), (rng.standard_normal((10, 1)) * 0.1).astype(np.float32)]
+    x = rng.random((784, 100), dtype=np.float32)
+    labels = rng.integers(1, 11, size=100)
+    loss_ref, grads_ref = oracle.mlp_backward(ws, x, labels)
+    params = [knet.Param(knet.KnetArray(w)) for w in ws]
+    xd = knet.KnetArray(x.reshape(28, 28, 1, 100, order="F"))   # the images as the example feeds them: mat() inside dense
+    J = knet.diff(lambda: knet.nll(knet.dense(params[2], knet.dense(params[0], xd, params[1], act="relu"), params[3]), labels, fused=True))
+    assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
+    for p, g in zip(params, grads_ref):
+        got = knet.Array(knet.grad(J, p))
+        assert got.shape == g.shape and np.linalg.norm(got - g) <= 1e-4 * np.linalg.norm(g)
+    # the data gradient, when asked for, has the data's shape
+    px = knet.Param(xd)
+    J = knet.diff(lambda: knet.nll(knet.dense(params[2], knet.dense(params[0], px, params[1], act="relu"), params[3]), labels, fused=True))
+    assert knet.grad(J, px).dims == (28, 28, 1, 100)
+    knet.libknet8().check()
