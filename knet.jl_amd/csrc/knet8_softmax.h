@@ -473,26 +473,17 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
   constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   const dim3 block(BT);
-  // COLS (columns per team, all loads issued up front) is always 1: measured on (32000,512), two columns per
-  // workgroup brought nothing for the fused nll kernel (23.0 us either way) and cost 8 % on the forward kernels --
-  // both phases are limited by HBM itself, not by the bubbles between them.
-  constexpr bool kCanTwo = false;
-  const bool two = false;
-#define KNET8_GRID(COLS) dim3((unsigned)((n + (long)TEAMS * COLS - 1) / ((long)TEAMS * COLS)))
+  // COLS (columns per team, all loads issued up front) is 1: measured on (32000,512), two columns per workgroup brought
+  // nothing for the fused nll kernel (23.0 us either way) and cost 8 % on the forward kernels -- both phases are limited by
+  // HBM itself, not by the bubbles between them.  The kernels keep the parameter for that measurement.
+  const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS));
   if constexpr (Algo::kNll) {
-#define KNET8_NLL(COLS) do { \
-      if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, out, labels, scale, loss); \
-      else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, out, labels, scale, loss); } while (0)
-    if constexpr (kCanTwo) { if (two) KNET8_NLL(2); else KNET8_NLL(1); } else { KNET8_NLL(1); }
-#undef KNET8_NLL
+    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, 1>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, 1>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
   } else {
-#define KNET8_COL(COLS) do { \
-      if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, b, out); \
-      else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false, COLS>), KNET8_GRID(COLS), block, 0, stream, m, n, a, b, out); } while (0)
-    if constexpr (kCanTwo) { if (two) KNET8_COL(2); else KNET8_COL(1); } else { KNET8_COL(1); }
-#undef KNET8_COL
+    if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true, 1>), grid, block, 0, stream, m, n, a, b, out);
+    else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false, 1>), grid, block, 0, stream, m, n, a, b, out);
   }
-#undef KNET8_GRID
 }
 
 template <typename T, typename Algo>
