@@ -60,7 +60,7 @@ def dense(w, x, b, act=None):
     src/ops20_gpu/activation.jl:17-29) and, backward, reluback and sum(dz;dims=2); the results carry the same bits."""
     if act not in (None, "relu"):
         raise ValueError("dense: act must be None or 'relu'")
-    x2 = mat(x)
+    x2 = x if x.ndims == 2 else x.reshape(x.length // x.size(x.ndims), x.size(x.ndims))
     m, k, n = _size2(w, 1), _size2(w, 2), x2.size(2)
     if x2.size(1) != k or b.length != m or w.dtype != x2.dtype or b.dtype != w.dtype:
         raise ValueError("DimensionMismatch: %r" % ((w.dims, x2.dims, b.dims),))
@@ -83,12 +83,18 @@ def dense(w, x, b, act=None):
     return y, selective(back)
 
 
-def mat(x):
-    """``mat(x)``: reshape to a matrix keeping the last dimension as columns (used by the MLP example)."""
-    from .autograd import Node
-    if isinstance(x, KnetArray) and x.ndims != 2:
-        return x.reshape(x.length // x.size(x.ndims), x.size(x.ndims))
-    return x
+@primitive
+def mat(x, dims=None):
+    """``mat(x; dims=ndims(x)-1)``: reshape to a matrix whose rows are the first ``dims`` dimensions (src/ops20/conv.jl:222; the MLP example
+    flattens its image batches with it).  Shares the memory; the gradient is the reshape back."""
+    nd = x.ndims
+    dims = nd - 1 if dims is None else int(dims)
+    rows = 1
+    for d in x.dims[:max(dims, 0)]:
+        rows *= d
+    cols = x.length // rows if rows else 0
+    y = x if (nd == 2 and x.dims == (rows, cols)) else x.reshape(rows, cols)
+    return y, (lambda dy: (dy.reshape(x.dims),))
 
 
 def axpy(alpha, x, y):

@@ -82,7 +82,23 @@ def _make(kernel, backkernel):
                 knet8("%s_strided_%s" % (backkernel, y.suffix), inner, d, outer, y.ptr, dy.ptr, dx.ptr)
                 return (dx,)
             return y, back
-        raise NotImplementedError("softmax over non-adjacent dims=%r of a %d-d array" % (dims, x.ndims))
+        # dims that are not adjacent (e.g. (1,3) of a 3-d array, test/loss.jl:46): the generic formulation of
+        # src/ops20/softmax.jl:42-63 from reductions and broadcasts
+        from .activation import unary_op
+        from .binary import broadcast_op as bc
+        d = sorted(set(int(i) for i in dims))
+        x1 = bc("sub", x, R.reduce_op("maximum", x, d))
+        e = unary_op("exp", x1)
+        ssum = R.reduce_op("sum", e, d)
+        if kernel == "logsoftmax":
+            y = bc("sub", x1, unary_op("log", ssum))
+            return y, (lambda dy: (bc("sub", dy, bc("mul", unary_op("exp", y), R.reduce_op("sum", dy, d))),))
+        y = bc("div", e, ssum)
+
+        def back_generic(dy):
+            yd = bc("mul", y, dy)
+            return (bc("sub", yd, bc("mul", y, R.reduce_op("sum", yd, d))),)
+        return y, back_generic
 
     f.__name__ = kernel
     return f

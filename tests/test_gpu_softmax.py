@@ -289,3 +289,32 @@ def test_streaming_kernel_on_short_columns_and_masked_logits(knet, oracle, dt):
         fn["knet8_tune"](1, old)
     assert np.all(np.isnan(got[:, 1])) and np.all(np.isfinite(got[:, [0, 2]]))
     assert fn["knet8_tune"](1, -1) == 0  # the knob is back at its default: later tests run the register-resident kernels
+
+
+def test_every_dims_choice_of_the_reference_test(knet, oracle):
+    """test/loss.jl:46-56: softmax == exp.(logsoftmax) and sums to one for dims in 1, 2, 3, (1,2), (1,3), [2,3], [1,2,3] of a
+    (10,10,10) array -- (1,3) is not a run of adjacent dims and goes through the generic reductions-and-broadcasts formulation --
+    plus values and gradients against the oracle."""
+    rng = np.random.default_rng(40)
+    a = rng.random((10, 10, 10)).astype(np.float32)
+    dy = rng.standard_normal((10, 10, 10)).astype(np.float32)
+    def adjacent(fun, dims, *arrays):
+        # the oracle takes runs of adjacent dims: for (1,3) permute the array to (1,3,2), use dims (1,2), permute back
+        if dims in ((1, 3), (3, 1)):
+            perm = (0, 2, 1)
+            out = fun(*[np.ascontiguousarray(np.transpose(x, perm)) for x in arrays], dims=(1, 2))
+            return np.transpose(out, perm)
+        return fun(*arrays, dims=dims)
+    for d in [1, 2, 3, (1, 2), (1, 3), [2, 3], [1, 2, 3], (3, 1)]:
+        od = tuple(d) if not isinstance(d, int) else d
+        k = knet.KnetArray(a)
+        sm, lsm = knet.Array(knet.softmax(k, dims=d)), knet.Array(knet.logsoftmax(k, dims=d))
+        assert np.allclose(sm, np.exp(lsm), rtol=1e-5, atol=1e-7), d
+        axes = tuple(i - 1 for i in ([d] if isinstance(d, int) else d))
+        assert np.allclose(sm.sum(axis=axes), 1, atol=1e-5), d
+        assert close(lsm, adjacent(oracle.logsoftmax, od, a)) and close(sm, adjacent(oracle.softmax, od, a)), d
+        for f, fo, bo in ((knet.logsoftmax, oracle.logsoftmax, oracle.logsoftmaxback), (knet.softmax, oracle.softmax, oracle.softmaxback)):
+            p = knet.Param(knet.KnetArray(a))
+            J = knet.diff(lambda: knet.sum(knet.mul(f(p, dims=d), knet.KnetArray(dy))))
+            assert close(knet.Array(knet.grad(J, p)), adjacent(bo, od, adjacent(fo, od, a), dy), 2e-5), d
+    knet.libknet8().check()

@@ -144,3 +144,17 @@ def test_tape_computes_only_the_gradients_that_are_needed(knet, rec, monkeypatch
     assert all(knet.grad(J, p) is not None for p in (w1, b1, w2, b2))
     names = [c_[0] for c_ in calls[n0:]]
     assert names.count("mul_32_11") == 2  # forward product and the gradient wrt its tracked operand only
+
+
+def test_mat_dims_as_the_reference_tests_them(knet, rec):
+    # test/ops20.jl:86-94 on an (8,8,2,3) array
+    calls, arr = rec
+    x = arr((8, 8, 2, 3))
+    assert knet.mat(x).dims == (128, 3)
+    assert knet.mat(x, dims=4).dims == (384, 1)
+    assert knet.mat(x, dims=3).dims == (128, 3)
+    assert knet.mat(x, dims=2).dims == (64, 6)
+    assert knet.mat(x, dims=1).dims == (8, 48)
+    assert knet.mat(x, dims=0).dims == (1, 384)
+    m = arr((5, 7))
+    assert knet.mat(m) is m
