@@ -86,32 +86,41 @@ def sum(x, dims=None):
     return reduce_op("sum", x, dims), _sum_back(x, dims)
 
 
-def prod(x, dims=None):
-    return reduce_op("prod", x, dims)
+def _reduction_with_gradient(name, grad):
+    """A reduction as a tape primitive.  ``grad(x, y, dy)`` is the gradient expression AutoGrad.jl (not part of the reference
+    repository) attaches to the Base function: the standard ones, pinned here the way test/reduction.jl:44-58 pins them -- by
+    finite differences."""
+    @primitive
+    def f(x, dims=None):
+        y = reduce_op(name, x, dims)
+        return y, (lambda dy: (grad(x, y, dy),))
+
+    f.__name__ = name
+    return f
 
 
-def maximum(x, dims=None):
-    return reduce_op("maximum", x, dims)
+def _bc(op, a, b):
+    from .binary import broadcast_op
+    return broadcast_op(op, a, b)
 
 
-def minimum(x, dims=None):
-    return reduce_op("minimum", x, dims)
+def _sign(x):
+    from .activation import unary_op
+    return unary_op("sign", x)
 
 
-def sumabs(x, dims=None):
-    return reduce_op("sumabs", x, dims)
+def _abs(x):
+    from .activation import unary_op
+    return unary_op("abs", x)
 
 
-def sumabs2(x, dims=None):
-    return reduce_op("sumabs2", x, dims)
-
-
-def maxabs(x, dims=None):
-    return reduce_op("maxabs", x, dims)
-
-
-def minabs(x, dims=None):
-    return reduce_op("minabs", x, dims)
+prod = _reduction_with_gradient("prod", lambda x, y, dy: _bc("mul", _bc("div", y, x), dy))
+maximum = _reduction_with_gradient("maximum", lambda x, y, dy: _bc("mul", _bc("eq", x, y), dy))
+minimum = _reduction_with_gradient("minimum", lambda x, y, dy: _bc("mul", _bc("eq", x, y), dy))
+sumabs = _reduction_with_gradient("sumabs", lambda x, y, dy: _bc("mul", _sign(x), dy))
+sumabs2 = _reduction_with_gradient("sumabs2", lambda x, y, dy: _bc("mul", _bc("mul", 2, x), dy))
+maxabs = _reduction_with_gradient("maxabs", lambda x, y, dy: _bc("mul", _bc("mul", _bc("eq", _abs(x), y), _sign(x)), dy))
+minabs = _reduction_with_gradient("minabs", lambda x, y, dy: _bc("mul", _bc("mul", _bc("eq", _abs(x), y), _sign(x)), dy))
 
 
 def countnz(x, dims=None):

@@ -190,3 +190,49 @@ def test_ticket_protocol_under_repetition(knet):
         for sh, y, want in outs:
             assert np.array_equal(knet.Array(y), want), (rep, sh)
     knet.libknet8().check()
+
+
+def test_gradients_of_every_reduction_by_finite_differences(knet):
+    """What test/reduction.jl:44-58 does with gradcheck: d/dx of sum(w .* f(x; dims)) through the tape against central differences in
+    fp64, for every reduction with a gradient, the reference's shapes (1, (1,1), 2, (2,1), (1,2), (2,2)) and a 3-d array with dims
+    lists.  Data as the reference draws it: distinct magnitudes for max/min-like ops (no ties), near-1 factors for prod."""
+    rng = np.random.default_rng(71)
+    fns = {"sum": np.sum, "prod": np.prod, "maximum": np.max, "minimum": np.min, "sumabs": lambda a, **k: np.sum(np.abs(a), **k),
+           "sumabs2": lambda a, **k: np.sum(a * a, **k), "maxabs": lambda a, **k: np.max(np.abs(a), **k), "minabs": lambda a, **k: np.min(np.abs(a), **k)}
+    cases = [((1,), None), ((1, 1), None), ((2,), None), ((2, 1), 1), ((1, 2), 2), ((2, 2), 1), ((2, 2), 2), ((2, 2), None),
+             ((3, 4, 5), None), ((3, 4, 5), 2), ((3, 4, 5), [1, 3]), ((3, 4, 5), [1, 2]), ((6, 7), 1), ((6, 7), 2)]
+    for name, ref in fns.items():
+        for shape, dims in cases:
+            n = int(np.prod(shape))
+            if name in ("maximum", "minimum", "maxabs", "minabs", "sumabs2"):
+                x = (0.01 * rng.permutation(np.arange(1, n + 1))).reshape(shape) * rng.choice([-1.0, 1.0], size=shape)
+            elif name == "prod":
+                x = np.exp(0.01 * rng.standard_normal(shape))
+            else:
+                x = rng.standard_normal(shape)
+            axes = None if dims is None else tuple(d - 1 for d in ([dims] if isinstance(dims, int) else dims))
+
+            def host(a):
+                return ref(a) if axes is None else ref(a, axis=axes, keepdims=True)
+            w = rng.standard_normal(np.shape(host(x)))
+            p = knet.Param(knet.KnetArray(x))
+            f = getattr(knet, name)
+            if dims is None:
+                J = knet.diff(lambda: f(p))
+                wgt = 1.0
+            else:
+                J = knet.diff(lambda: knet.sum(knet.mul(f(p, dims=dims), knet.KnetArray(w))))
+                wgt = w
+            assert np.isclose(float(knet.value(J)), float(np.sum(host(x) * wgt)), rtol=1e-12, atol=1e-14), (name, shape, dims)
+            got = knet.Array(knet.grad(J, p))
+            num = np.zeros_like(x)
+            h = 1e-6
+            it = np.nditer(x, flags=["multi_index"])
+            for _ in it:
+                i = it.multi_index
+                xp, xm = x.copy(), x.copy()
+                xp[i] += h
+                xm[i] -= h
+                num[i] = (np.sum(host(xp) * wgt) - np.sum(host(xm) * wgt)) / (2 * h)
+            assert np.allclose(got, num, rtol=1e-5, atol=1e-7), (name, shape, dims)
+    knet.libknet8().check()
