@@ -79,3 +79,30 @@ def test_special_cases(oracle):
     for t in range(1, 4001):
         (m, v), x = oracle.optimizer_update("adam", 2 * x, [m, v], x, t=t, lr=0.01, beta1=0.9, beta2=0.999, eps=1e-8)
     assert np.abs(x).max() < 1e-2
+
+
+def test_rosenbrock_converges_with_the_reference_tests_settings(oracle):
+    """test/update.jl:10-60 minimises the 6-dimensional Rosenbrock function with every optimizer at fixed hyper-parameters until
+    f <= 0.1 (at most 10000 steps; the reference notes the outcome depends on the random start).  The same run with the oracle's
+    update rules from two fixed starts: a dropped term or a wrong sign in a rule does not get there."""
+    def f(x):
+        return np.sum((1 - x[:-1]) ** 2 + 100 * (x[1:] - x[:-1] ** 2) ** 2)
+
+    def grad(x):
+        d = np.zeros_like(x)
+        d[:-1] += -2 * (1 - x[:-1]) - 400 * x[:-1] * (x[1:] - x[:-1] ** 2)
+        d[1:] += 200 * (x[1:] - x[:-1] ** 2)
+        return d
+    opts = [("momentum", dict(lr=0.00025, gamma=0.95), 1), ("nesterov", dict(lr=0.00025, gamma=0.95), 1),
+            ("adam", dict(lr=0.005, beta1=0.9, beta2=0.95, eps=1e-8), 2), ("adagrad", dict(lr=0.4, eps=1e-6), 1),
+            ("adadelta", dict(lr=0.4, rho=0.5, eps=1e-6), 2), ("rmsprop", dict(lr=0.005, rho=0.9, eps=1e-6), 1)]
+    for seed in (0, 5):
+        w0 = np.random.default_rng(seed).standard_normal(6)
+        for kind, hp, nstate in opts:
+            w, st = w0.copy(), [np.zeros(6) for _ in range(nstate)]
+            prev, cur, i = 0.0, 1.0, 1
+            while i <= 10000 and abs(cur - prev) > 1e-10 and cur > 0.1:
+                prev, cur = cur, f(w)
+                st, w = oracle.optimizer_update(kind, grad(w), st, w, t=i, **hp)
+                i += 1
+            assert cur <= 0.1, (kind, seed, cur, i)
