@@ -111,9 +111,17 @@ def scal(alpha, x):
     return x
 
 
-def transpose(x):
-    """``permutedims(x)`` for a matrix (src/knetarrays/reshape.jl:18) -> ``transpose_S``."""
+def _transpose(x):
     m, n = x.size(1), x.size(2)
     y = x.similar((n, m))
     knet8("transpose_%s" % x.suffix, m, n, x.ptr, y.ptr)
     return y
+
+
+@primitive
+def transpose(x):
+    """``permutedims(x)`` / ``transpose(x)`` for a matrix (src/knetarrays/reshape.jl:18, linalg.jl:92-113) -> ``transpose_S``; the gradient is
+    the transpose of the incoming gradient."""
+    if x.ndims > 2:
+        raise ValueError("transpose needs a vector or a matrix")
+    return _transpose(x), (lambda dy: (_transpose(dy),))

@@ -148,3 +148,20 @@ def test_backward_sweep_releases_intermediates(knet):
     expect = 6 * 256 * 256 * 4 * 2 + 256 * 512 * 4   # weights + their gradients + the input batch
     assert live <= expect + 64 * 1024, (live, expect)
     assert all(knet.grad(J, w) is not None for w in ws)
+
+
+def test_matmul_and_transpose_gradients_as_the_reference_checks_them(knet):
+    """test/linalg.jl:12-31,43: gradcheck of w[1]*w[2] on (3,5)x(5,2) and of transpose -- here against the closed forms
+    d(sum(W .* (A*B)))/dA = W*B', /dB = A'*W and d(sum(W .* A'))/dA = W'."""
+    rng = np.random.default_rng(44)
+    for dt, tol in ((np.float32, 1e-5), (np.float64, 1e-13)):
+        a, b = rng.random((3, 5)).astype(dt), rng.random((5, 2)).astype(dt)
+        w = rng.standard_normal((3, 2)).astype(dt)
+        pa, pb = knet.Param(knet.KnetArray(a)), knet.Param(knet.KnetArray(b))
+        J = knet.diff(lambda: knet.sum(knet.mul(knet.matmul(pa, pb), knet.KnetArray(w))))
+        assert np.allclose(knet.Array(knet.grad(J, pa)), w @ b.T, rtol=tol, atol=tol)
+        assert np.allclose(knet.Array(knet.grad(J, pb)), a.T @ w, rtol=tol, atol=tol)
+        wt = rng.standard_normal((5, 3)).astype(dt)
+        J = knet.diff(lambda: knet.sum(knet.mul(knet.transpose(pa), knet.KnetArray(wt))))
+        assert np.array_equal(knet.Array(knet.grad(J, pa)), wt.T)
+    knet.libknet8().check()
