@@ -71,7 +71,16 @@ def device_randn(torch, K, n, dtype, seed, dims=None, scale=1.0):
     t = torch.randn(n, device="cuda", dtype=dtype, generator=g)
     if scale != 1.0:
         t.mul_(scale)
-    return K.KnetArray.from_torch(t, dims=dims or (n,))
+    # into memory from the library's own pool, as every KnetArray of a real run is (the pool places large blocks so that arrays
+    # allocated one after the other do not start at the same offset modulo the memory-channel interleave)
+    dt = {torch.float32: np.float32, torch.float64: np.float64}[dtype]
+    k = K.KnetArray(dtype=dt, dims=dims or (n,))
+    lib = K.libknet8()
+    lib.fn["knet8_memcpy"](k.ptr, t.data_ptr(), n * t.element_size(), 3, lib.stream)
+    torch.cuda.synchronize()
+    lib.fn["knet8_synchronize"](lib.stream)
+    del t
+    return k
 
 
 def config2(torch, K, steps, warmup):

@@ -131,13 +131,47 @@ void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes
 // reference's KnetPtr pool does (src/knetarrays/kptr.jl:105-142; an uncached allocation costs ~0.5 ms there,
 // kptr.jl:187).  Sizes are rounded up to {1, 1.25, 1.5, 1.75} x 2^k (>= 256 bytes), so at most 25 % is lost
 // to rounding.  When hipMalloc fails the free lists are released and the allocation retried once.
+//
+// Placement of large blocks.  Measured on MI355X with the 2R+1W gradient kernels on 1 GiB operands (a 16 x 16 map of the start
+// offsets of y and dx relative to dy, in KB): the time depends on where the three arrays start relative to each other modulo
+// 16 KB -- 499-513 us when the output starts at the same residue as dy (what page-aligned allocations give; 522-529 us at odd
+// multiples of 16 KB), 480-485 us when it starts 5-7 KB later and y 1-5 KB later: same-index accesses of the streams then do not
+// meet in the same memory channel and bank.  Blocks of 1 MB and more are therefore handed out at a start address whose residue
+// modulo 16 KB advances by 21*256 bytes (5.25 KB) from one new block to the next (all 64 multiples of 256 come up before any
+// repeats), so arrays allocated one after the other -- a layer's dy and then its dx -- sit in the good region of that map.
 struct Pool {
   std::mutex mutex;
-  std::unordered_map<size_t, std::vector<void*>> free_lists;  // rounded size -> blocks
+  std::unordered_map<size_t, std::vector<void*>> free_lists;  // rounded size -> blocks (as handed out)
   std::unordered_map<void*, size_t> live;                     // block -> rounded size
+  std::unordered_map<void*, void*> base_of;                   // block handed out at an offset -> what hipMalloc returned
   size_t bytes_live = 0, bytes_cached = 0, nmalloc = 0, nhit = 0;
+  unsigned next_color = 0;
 };
 static Pool g_pool;
+constexpr size_t kColorPeriod = 16384, kColorStep = 21 * 256, kColorMinBytes = size_t(1) << 20;
+
+static hipError_t pool_device_malloc(Pool& pool, void** out, size_t sz) {
+  if (sz < kColorMinBytes) return hipMalloc(out, sz);
+  void* base = nullptr;
+  const hipError_t e = hipMalloc(&base, sz + kColorPeriod);
+  if (e != hipSuccess) return e;
+  const size_t want = (pool.next_color++ * kColorStep) % kColorPeriod;
+  const size_t have = reinterpret_cast<uintptr_t>(base) % kColorPeriod;
+  const size_t off = ((want + kColorPeriod - have) % kColorPeriod + 255) / 256 * 256 % kColorPeriod;
+  *out = static_cast<char*>(base) + off;
+  if (off) pool.base_of[*out] = base;
+  return hipSuccess;
+}
+
+static void pool_device_free(Pool& pool, void* p) {
+  auto it = pool.base_of.find(p);
+  if (it != pool.base_of.end()) {
+    (void)hipFree(it->second);
+    pool.base_of.erase(it);
+  } else {
+    (void)hipFree(p);
+  }
+}
 
 static size_t round_size(size_t n) {
   if (n <= 256) return 256;
@@ -153,7 +187,7 @@ static size_t trim_locked(Pool& pool) {
   size_t released = 0;
   for (auto& kv : pool.free_lists) {
     for (void* p : kv.second) {
-      (void)hipFree(p);
+      pool_device_free(pool, p);
       released += kv.first;
     }
     kv.second.clear();
@@ -179,11 +213,11 @@ KNET8_API void* knet8_malloc(size_t nbytes) {
     g_pool.bytes_cached -= sz;
     g_pool.nhit++;
   } else {
-    hipError_t e = hipMalloc(&p, sz);
+    hipError_t e = pool_device_malloc(g_pool, &p, sz);
     if (e != hipSuccess) {
       (void)hipGetLastError();
       trim_locked(g_pool);
-      e = hipMalloc(&p, sz);
+      e = pool_device_malloc(g_pool, &p, sz);
     }
     if (e != hipSuccess) {
       (void)hipGetLastError();
