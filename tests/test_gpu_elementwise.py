@@ -326,3 +326,33 @@ def test_pow_and_comparisons(knet, dt):
     got = knet.Array(knet.back11_op("invxback", knet.KnetArray(dy), knet.KnetArray(yy)))
     assert bits_equal(got, ((-dy) * yy) * yy)
     knet.libknet8().check()
+
+
+def test_largest_length_the_abi_can_express(knet):
+    """n = 2^31 - 1 elements (the `int n` of the entry points at its maximum): 8 GiB per fp32 array.  reluback on a +1/-1 pattern and
+    the whole-array sum over it; sizes and offsets inside the kernels must not wrap."""
+    n = (1 << 31) - 1
+    fn = knet.libknet8().fn
+    y = np.empty(n, np.float32)
+    y[0::2] = 1.0
+    y[1::2] = -1.0
+    y[12345::1000003] = 0.5          # a sprinkle of other values so that a shifted or repeated block cannot pass
+    yd = knet.KnetArray(y)
+    dx = yd.similar()
+    knet.knet8("reluback_32_11", n, yd.ptr, yd.ptr, dx.ptr)       # dx = y > 0 ? y : 0
+    got = knet.Array(dx)
+    step = 1 << 27
+    for a in range(0, n, step):
+        assert np.array_equal(got[a:a + step], np.maximum(y[a:a + step], 0)), a
+    del got
+    # sum: +1 and -1 cancel pairwise; the sprinkled elements replace some +1/-1 by 0.5 -- all partial sums are exact in fp32
+    want = float(np.sum(y, dtype=np.float64))
+    assert float(knet.sum(yd)) == want
+    # column sums of a (2^15, 2^15) prefix of the same memory through the _21 form
+    rows, cols = 1 << 15, 1 << 15
+    ycol = knet.KnetArray(np.zeros(cols, np.float32))
+    knet.knet8("sum_32_21", rows * cols, yd.ptr, rows, cols, ycol.ptr)
+    assert np.array_equal(knet.Array(ycol), y[: rows * cols].reshape(cols, rows).sum(axis=1, dtype=np.float64).astype(np.float32))
+    del yd, dx
+    fn["knet8_trim"]()
+    knet.libknet8().check()
