@@ -236,3 +236,28 @@ def test_gradients_of_every_reduction_by_finite_differences(knet):
                 num[i] = (np.sum(host(xp) * wgt) - np.sum(host(xm) * wgt)) / (2 * h)
             assert np.allclose(got, num, rtol=1e-5, atol=1e-7), (name, shape, dims)
     knet.libknet8().check()
+
+
+def test_split_reductions_are_bit_reproducible(knet):
+    """Partial results are combined in a fixed order by the last workgroup to finish (no floating-point atomics), so repeated launches
+    on the same data give the same bits whatever the arrival order -- for the strided and run views, the fused bias-gradient
+    kernel, the split small GEMM and the whole-array sum."""
+    rng = np.random.default_rng(72)
+    x = rng.standard_normal((4096, 1024)).astype(np.float32)
+    d = knet.KnetArray(x)
+    dy = knet.KnetArray(rng.standard_normal((4096, 1024)).astype(np.float32))
+    a = knet.KnetArray(rng.standard_normal((64, 784)).astype(np.float32))
+    b = knet.KnetArray(rng.standard_normal((784, 100)).astype(np.float32))
+    first = None
+    for r in range(12):
+        outs = [knet.Array(knet.sum(d, dims=2)), knet.Array(knet.sum(d, dims=1)), np.float32(knet.sum(d)),
+                knet.Array(knet.matmul(a, b))]
+        dz, db = d.similar(), knet.KnetArray(np.zeros((4096, 1), np.float32))
+        knet.knet8("reluback_biasgrad_32", 4096, 1024, dy.ptr, d.ptr, dz.ptr, db.ptr)
+        outs.append(knet.Array(db))
+        if first is None:
+            first = outs
+        else:
+            for got, want in zip(outs, first):
+                assert np.array_equal(np.asarray(got).view(np.uint32), np.asarray(want).view(np.uint32)), r
+    knet.libknet8().check()
