@@ -48,3 +48,17 @@ for (T, S) in ((Float32, 32), (Float64, 64))
         end
     end
 end
+
+# The whole layer in one call: y = f.(w*x .+ b) with f = relu or identity (gemm_bias_act_S folds bias and relu into the product's
+# output stage for small products; large ones run hipBLASLt followed by one in-place pass).  `act`: 0 none, 1 relu.
+for (T, S) in ((Float32, 32), (Float64, 64))
+    @eval function dense!(y::KnetArray{$T,2}, w::KnetArray{$T,2}, x::KnetArray{$T,2}, b::KnetArray{$T}; act::Integer=1)
+        m, k = size(w); n = size(x, 2)
+        @assert size(x, 1) == k && size(y) == (m, n) && length(b) == m
+        rc = ccall(($("gemm_bias_act_$(S)_stream"), LibKnet8.libknet8), Cint,
+                   (UInt8, UInt8, Cint, Cint, Cint, $T, Ptr{$T}, Cint, Ptr{$T}, Cint, Ptr{$T}, Cint, Ptr{$T}, Cint, Ptr{Cvoid}),
+                   'N', 'N', m, n, k, one($T), w, m, x, k, b, act, y, m, LibKnet8.knet8_stream())
+        rc == 0 || LibKnet8.knet8_check()
+        return y
+    end
+end
