@@ -31,9 +31,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of reluback_32_11 on 2^28 elements from the two `rocprofv3 --pmc` runs summarised in
-# profiles/libknet8_kernels_profile_pass.txt: FETCH_SIZE 1048576 KiB x 2.0000 + WRITE_SIZE 1048600 KiB x 0.9991, each scaled by
+# profiles/libknet8_kernels_profile_pass.txt: FETCH_SIZE x 2.0000 -> 2048.0 MiB + WRITE_SIZE x 0.9996 -> 1023.6 MiB, each scaled by
 # what the same counter reads for the 1 GiB + 1 GiB copy kernel of that run.  (Algorithmic: 3 * 4 * 2^28 = 3221225472.)
-RELUBACK_32_TRAFFIC_BYTES = int((2048.0 + 1023.1) * (1 << 20))
+RELUBACK_32_TRAFFIC_BYTES = int((2048.0 + 1023.6) * (1 << 20))
 OPS = [("reluback", "relu"), ("sigmback", "sigm"), ("tanhback", "tanh"), ("eluback", "elu"), ("seluback", "selu")]
 
 
