@@ -175,3 +175,54 @@ def test_first_split_reduction_on_a_new_stream_over_recycled_memory(knet):
             assert np.array_equal(knet.Array(y), want)
         fn["knet8_stream_destroy"](s)
     knet.libknet8().check()
+
+
+def test_threads_with_their_own_streams(knet):
+    """The reference builds its library with per-thread default streams and calls it from Julia tasks (src/libknet8/build.jl:5,
+    LibKnet8.jl:50-55): entry points must be re-entrant.  Four host threads, each with its own stream, run split reductions,
+    small split products, pool allocations and frees at the same time; every result is exact (integer-valued data)."""
+    import threading
+    fn = knet.libknet8().fn
+    rng = np.random.default_rng(8)
+    errors = []
+
+    def worker(seed):
+        try:
+            r = np.random.default_rng(seed)
+            s = fn["knet8_stream_create"]()
+            x = r.integers(-3, 4, size=(768, 2048)).astype(np.float32)
+            a = r.integers(-2, 3, size=(40, 300)).astype(np.float32)
+            b = r.integers(-2, 3, size=(300, 50)).astype(np.float32)
+            nbytes = x.nbytes
+            for it in range(15):
+                dx = fn["knet8_malloc"](nbytes)
+                dy = fn["knet8_malloc"](768 * 4)
+                dc = fn["knet8_malloc"](40 * 50 * 4)
+                da, db = fn["knet8_malloc"](a.nbytes), fn["knet8_malloc"](b.nbytes)
+                xf, af, bf = np.asfortranarray(x), np.asfortranarray(a), np.asfortranarray(b)
+                fn["knet8_memcpy"](dx, xf.ctypes.data, nbytes, 1, s)
+                fn["knet8_memcpy"](da, af.ctypes.data, a.nbytes, 1, s)
+                fn["knet8_memcpy"](db, bf.ctypes.data, b.nbytes, 1, s)
+                fn["sum_32_21_stream"](x.size, dx, 1, 768, dy, s)          # dims=2: split over workgroups, per-stream scratch
+                fn["gemm_32_stream"](b"N", b"N", 40, 50, 300, np.float32(1), da, 40, db, 300, np.float32(0), dc, 40, s)
+                tot = fn["sum_32_20_stream"](x.size, dx, s)                # blocks on this stream only
+                out = np.empty(768, np.float32)
+                c = np.empty((40, 50), np.float32, order="F")
+                fn["knet8_memcpy"](out.ctypes.data, dy, out.nbytes, 2, s)
+                fn["knet8_memcpy"](c.ctypes.data, dc, c.nbytes, 2, s)
+                assert np.array_equal(out, x.sum(axis=1)), ("sum dims=2", seed, it)
+                assert float(tot) == float(x.sum()), ("sum", seed, it)
+                assert np.array_equal(c, a @ b), ("gemm", seed, it)
+                for p in (dx, dy, dc, da, db):
+                    fn["knet8_free"](p)
+            fn["knet8_stream_destroy"](s)
+        except Exception as e:  # noqa: BLE001 -- reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(100 + i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    knet.libknet8().check()
