@@ -110,13 +110,15 @@ inline void launch_ew(hipStream_t stream, long n, const T* a, const T* b, const 
 template <typename T, typename F>
 __global__ __launch_bounds__(kEwBlock) void ew_bcast12_kernel(long n, const T* x, int sx, int nx, const T* y, int sy, int ny,
                                                               T* z, F f) {
-  const long base = (long)blockIdx.x * (kEwBlock * 4) + threadIdx.x;
+  // n is a 32-bit int at the ABI: index arithmetic in 32 bits (a 64-bit division costs several times more than the memory access)
+  const unsigned base = blockIdx.x * (kEwBlock * 4) + threadIdx.x;
+  const unsigned un = (unsigned)n, unx = (unsigned)nx, uny = (unsigned)ny, usx = (unsigned)sx, usy = (unsigned)sy;
 #pragma unroll
   for (int u = 0; u < 4; u++) {
-    const long i = base + u * kEwBlock;
-    if (i < n) {
-      const T xi = (nx == n ? x[i] : sx == 1 ? x[i % nx] : nx == 1 ? x[0] : x[(i / sx) % nx]);
-      const T yi = (ny == n ? y[i] : sy == 1 ? y[i % ny] : ny == 1 ? y[0] : y[(i / sy) % ny]);
+    const unsigned i = base + u * kEwBlock;
+    if (i < un) {
+      const T xi = (unx == un ? x[i] : usx == 1 ? x[i % unx] : unx == 1 ? x[0] : x[(i / usx) % unx]);
+      const T yi = (uny == un ? y[i] : usy == 1 ? y[i % uny] : uny == 1 ? y[0] : y[(i / usy) % uny]);
       z[i] = f(xi, yi);
     }
   }
