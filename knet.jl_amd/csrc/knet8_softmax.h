@@ -95,10 +95,23 @@ __device__ __forceinline__ T team_reduce(T v, T* lds, Merge merge, T identity) {
 
 // ---- register-resident column kernel -----------------------------------------------------------------
 // TEAM lanes per column (64: four columns per 256-thread workgroup; 256 or 1024: the whole workgroup),
-// E elements of each held input per lane, VEC: 16-byte accesses (m % N == 0 and 16-byte aligned operands),
-// COLS: columns a team handles one after the other with the loads of all of them issued up front (an experiment in
-// hiding the reduce phase behind the next column's loads; the launcher explains why it always passes 1).
-template <typename T, typename Algo, int TEAM, int E, bool VEC, int COLS>
+// E elements of each held input per lane, VEC: 16-byte accesses.
+//
+// Columns need not start on a 16-byte boundary (m odd: vocabularies of 50257 or 10001 classes): with VEC each column is
+// cut into `head` elements up to its first aligned address, `nb` whole vectors and `tail` elements.  Lane tl of the team owns
+// vectors tl, tl+TEAM, ...; the at most N-1 head and N-1 tail elements live in one extra register each of lanes 0..N-2.  All
+// operands of a call must be congruent modulo 16 bytes (they then are in every column, the column length being common).
+template <typename T, int NV>
+__device__ __forceinline__ void cut_column(const T* p, int m, int& head, int& nb, int& tail) {
+  if (NV == 1) { head = 0; nb = m; tail = 0; return; }
+  const int mis = (int)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) % NV);
+  head = (NV - mis) % NV;
+  if (head > m) head = m;
+  nb = (m - head) / NV;
+  tail = m - head - nb * NV;
+}
+
+template <typename T, typename Algo, int TEAM, int E, bool VEC>
 __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
   // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
   // output pass, so the dependent chain is one memory round trip instead of two.
@@ -111,78 +124,88 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   typedef typename Vec16<T>::type V;
   __shared__ T lds[BT / kWave];
   const int tl = threadIdx.x % TEAM;
-  const long col0 = ((long)blockIdx.x * TEAMS + threadIdx.x / TEAM) * COLS;
-  // lane tl owns accesses tl, tl+TEAM, ... of the m/NV accesses of a column: the first `cnt` of its ITEMS slots
-  int cnt = (m / NV - tl + TEAM - 1) / TEAM;
-  cnt = cnt < 0 ? 0 : cnt;
+  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
+  const bool colok = col < n;  // only wave teams can be out of range
+  const long base = colok ? col * (long)m : 0;
+  const T* ac = a + base;
+  const T* bc = kTwo ? b + base : nullptr;
+  T* oc = out + base;
+  int head, nb, tail;
+  cut_column<T, NV>(ac, m, head, nb, tail);
+  int cnt = (nb - tl + TEAM - 1) / TEAM;  // this lane's share of the nb vectors: the first `cnt` of its ITEMS slots
+  cnt = !colok || cnt < 0 ? 0 : cnt;
+  const bool hv = NV > 1 && colok && tl < head, tv = NV > 1 && colok && tl < tail;  // this lane holds a head / a tail element
+  const int tpos = head + nb * NV + tl;                                         // where its tail element sits
 
-  V ra[kHold ? COLS : 1][kHold ? ITEMS : 1], rb[kTwo ? COLS : 1][kTwo ? ITEMS : 1];
+  V ra[kHold ? ITEMS : 1], rb[kTwo ? ITEMS : 1];
+  T ah = T(0), at = T(0), bh = T(0), bt = T(0);
 #pragma unroll
-  for (int c = 0; c < COLS; c++) {
-    const long col = col0 + c;
-    const bool colok = col < n;  // only wave teams and the last of COLS can be out of range
-    const long base = colok ? col * (long)m : 0;
-#pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-      const long r = (long)(tl + i * TEAM) * NV;
-      if (colok && i < cnt) {
-        if (VEC) {
-          if (kHold) ra[c][i] = ld_stream(reinterpret_cast<const V*>(a + base + r));
-          if (kTwo) rb[c][i] = ld_stream(reinterpret_cast<const V*>(b + base + r));
-        } else {
-          if (kHold) ra[c][i][0] = __builtin_nontemporal_load(a + base + r);
-          if (kTwo) rb[c][i][0] = __builtin_nontemporal_load(b + base + r);
-        }
+  for (int i = 0; i < ITEMS; i++) {
+    const long r = head + (long)(tl + i * TEAM) * NV;
+    if (i < cnt) {
+      if (VEC) {
+        if (kHold) ra[i] = ld_stream(reinterpret_cast<const V*>(ac + r));
+        if (kTwo) rb[i] = ld_stream(reinterpret_cast<const V*>(bc + r));
+      } else {
+        if (kHold) ra[i][0] = __builtin_nontemporal_load(ac + r);
+        if (kTwo) rb[i][0] = __builtin_nontemporal_load(bc + r);
       }
     }
   }
-#pragma unroll
-  for (int c = 0; c < COLS; c++) {
-    const long col = col0 + c;
-    const bool colok = col < n;
-    const long base = colok ? col * (long)m : 0;
-    T mx = T(0);
-    if (Algo::kNeedMax) {
-      mx = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < ITEMS; i++)
-        if (colok && i < cnt) {
-#pragma unroll
-          for (int e = 0; e < NV; e++) mx = mx > ra[c][i][e] ? mx : ra[c][i][e];
-        }
-      mx = team_reduce<T, TEAM>(mx, lds, MaxFn(), T(-INFINITY));
-    }
-    T s = T(0);
+  if (NV > 1) {
+    if (hv) { ah = ac[tl]; if (kTwo) bh = bc[tl]; }
+    if (tv) { at = ac[tpos]; if (kTwo) bt = bc[tpos]; }
+  }
+  T mx = T(0);
+  if (Algo::kNeedMax) {
+    mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < ITEMS; i++)
-      if (colok && i < cnt) {
+      if (i < cnt) {
 #pragma unroll
-        for (int e = 0; e < NV; e++) {
-          const T t = Algo::term(kHold ? ra[c][i][e] : T(0), kTwo ? rb[c][i][e] : T(0), mx);
-          if constexpr (Algo::kKeepTerm && kHold) ra[c][i][e] = t;
-          s = s + t;
-        }
+        for (int e = 0; e < NV; e++) mx = mx > ra[i][e] ? mx : ra[i][e];
       }
-    s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
-    const T fin = Algo::finish(s);
+    if (hv) mx = mx > ah ? mx : ah;
+    if (tv) mx = mx > at ? mx : at;
+    mx = team_reduce<T, TEAM>(mx, lds, MaxFn(), T(-INFINITY));
+  }
+  T s = T(0);
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-      if (!(colok && i < cnt)) continue;
-      const long r = (long)(tl + i * TEAM) * NV;
-      V va = {};
-      if (!kHold) {
-        if (VEC) va = ld_stream(reinterpret_cast<const V*>(a + base + r));
-        else va[0] = __builtin_nontemporal_load(a + base + r);
-      }
-      V vo;
+  for (int i = 0; i < ITEMS; i++)
+    if (i < cnt) {
 #pragma unroll
       for (int e = 0; e < NV; e++) {
-        if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(ra[c][i][e], fin);
-        else vo[e] = Algo::out(kHold ? ra[c][i][e] : va[e], kTwo ? rb[c][i][e] : T(0), mx, fin);
+        const T t = Algo::term(kHold ? ra[i][e] : T(0), kTwo ? rb[i][e] : T(0), mx);
+        if constexpr (Algo::kKeepTerm && kHold) ra[i][e] = t;
+        s = s + t;
       }
-      if (VEC) st_stream(reinterpret_cast<V*>(out + base + r), vo);
-      else __builtin_nontemporal_store(vo[0], out + base + r);
     }
+  if (hv) { const T t = Algo::term(ah, bh, mx); if constexpr (Algo::kKeepTerm) ah = t; s = s + t; }
+  if (tv) { const T t = Algo::term(at, bt, mx); if constexpr (Algo::kKeepTerm) at = t; s = s + t; }
+  s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
+  const T fin = Algo::finish(s);
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    if (i >= cnt) continue;
+    const long r = head + (long)(tl + i * TEAM) * NV;
+    V va = {};
+    if (!kHold) {
+      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+      else va[0] = __builtin_nontemporal_load(ac + r);
+    }
+    V vo;
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(ra[i][e], fin);
+      else vo[e] = Algo::out(kHold ? ra[i][e] : va[e], kTwo ? rb[i][e] : T(0), mx, fin);
+    }
+    if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+    else __builtin_nontemporal_store(vo[0], oc + r);
+  }
+  if (NV > 1) {
+    // a streamed (not held) first input was read above as ah/at all the same: the extras are always held
+    if (hv) { if constexpr (Algo::kKeepTerm) oc[tl] = Algo::out_kept(ah, fin); else oc[tl] = Algo::out(ah, bh, mx, fin); }
+    if (tv) { if constexpr (Algo::kKeepTerm) oc[tpos] = Algo::out_kept(at, fin); else oc[tpos] = Algo::out(at, bt, mx, fin); }
   }
 }
 
@@ -211,10 +234,9 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
   return v;
 }
 
-// COLS: as in softmax_col_kernel.
 // The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
-// fished out of the register that happens to hold it.
-template <typename T, int TEAM, int E, bool VEC, int COLS>
+// fished out of the register that happens to hold it.  Columns are cut into head / vectors / tail as in softmax_col_kernel.
+template <typename T, int TEAM, int E, bool VEC>
 __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
                                                                             T scale, T* loss) {
   constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
@@ -223,83 +245,87 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
   constexpr int NV = VEC ? Vec16<T>::N : 1;
   constexpr int ITEMS = E / NV;
   typedef typename Vec16<T>::type V;
-  __shared__ T lds_m[COLS][BT / kWave], lds_s[COLS][BT / kWave];
+  __shared__ T lds_m[BT / kWave], lds_s[BT / kWave];
   const int tl = threadIdx.x % TEAM;
-  const long col0 = ((long)blockIdx.x * TEAMS + threadIdx.x / TEAM) * COLS;
-  // lane tl owns accesses tl, tl+TEAM, ... of the m/NV accesses of a column: the first `cnt` of its ITEMS slots
-  const int macc = m / NV;  // VEC implies m % NV == 0
-  int cnt = (macc - tl + TEAM - 1) / TEAM;
-  cnt = cnt < 0 ? 0 : cnt;
+  const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
+  const bool colok = col < n;
+  const T* ac = a + (colok ? col * (long)m : 0);
+  T* oc = out + (colok ? col * (long)m : 0);
+  int head, nb, tail;
+  cut_column<T, NV>(ac, m, head, nb, tail);
+  int cnt = (nb - tl + TEAM - 1) / TEAM;
+  cnt = !colok || cnt < 0 ? 0 : cnt;
+  const bool hv = NV > 1 && colok && tl < head, tv = NV > 1 && colok && tl < tail;
+  const int tpos = head + nb * NV + tl;
+  const T ninf = T(-INFINITY);
 
-  V rv[COLS][ITEMS];
-  int lab[COLS];
-  T alab[COLS];
+  int lab = colok ? labels[col] : 0;
+  if (lab < 0 || lab > m) lab = 0;  // callers check labels on the host; an out-of-range one is skipped, never dereferenced
+  const T alab = (tl == 0 && lab > 0) ? ac[lab - 1] : T(0);
+  V rv[ITEMS];
 #pragma unroll
-  for (int c = 0; c < COLS; c++) {
-    const long col = col0 + c;
-    const bool colok = col < n;
-    const T* ac = a + (colok ? col * (long)m : 0);
-    lab[c] = colok ? labels[col] : 0;
-    if (lab[c] < 0 || lab[c] > m) lab[c] = 0;  // callers check labels on the host; an out-of-range one is skipped, never dereferenced
-    alab[c] = (tl == 0 && lab[c] > 0) ? ac[lab[c] - 1] : T(0);
+  for (int i = 0; i < ITEMS; i++) {
+    if (i < cnt) {
+      if (VEC) rv[i] = ld_stream(reinterpret_cast<const V*>(ac + head + (long)(tl + i * TEAM) * NV));
+      else rv[i][0] = __builtin_nontemporal_load(ac + (tl + i * TEAM));
+    } else {
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-      if (colok && i < cnt) {
-        if (VEC) rv[c][i] = ld_stream(reinterpret_cast<const V*>(ac + (long)(tl + i * TEAM) * NV));
-        else rv[c][i][0] = __builtin_nontemporal_load(ac + (tl + i * TEAM));
-      } else {
-#pragma unroll
-        for (int e = 0; e < NV; e++) rv[c][i][e] = T(-INFINITY);
-      }
+      for (int e = 0; e < NV; e++) rv[i][e] = ninf;
     }
   }
+  T xh = hv ? ac[tl] : ninf, xt = tv ? ac[tpos] : ninf;  // -inf padding contributes exp(-inf) = 0
+
+  T mt = ninf;
 #pragma unroll
-  for (int c = 0; c < COLS; c++) {
-    const long col = col0 + c;
-    const bool colok = col < n;
-    T* oc = out + (colok ? col * (long)m : 0);
-    T mt = -INFINITY;
+  for (int i = 0; i < ITEMS; i++)
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++)
+    for (int e = 0; e < NV; e++) mt = mt > rv[i][e] ? mt : rv[i][e];
+  if (NV > 1) { mt = mt > xh ? mt : xh; mt = mt > xt ? mt : xt; }
+  T st = T(0);
+  const T mref = mt == ninf ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
 #pragma unroll
-      for (int e = 0; e < NV; e++) mt = mt > rv[c][i][e] ? mt : rv[c][i][e];
-    T st = T(0);
-    const T mref = mt == T(-INFINITY) ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
+  for (int i = 0; i < ITEMS; i++)
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++)
-#pragma unroll
-      for (int e = 0; e < NV; e++) {
-        const T ex = dev_exp(rv[c][i][e] - mref);
-        rv[c][i][e] = ex;
-        st = st + ex;
-      }
-    MaxSum<T> ms = {mt, st};
-    ms = ms_wave_reduce(ms);
-    if (NW > 1) {
-      const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-      if (lane == 0) { lds_m[c][wave] = ms.m; lds_s[c][wave] = ms.s; }
-      __syncthreads();
-      MaxSum<T> t = {lane < NW ? lds_m[c][lane] : T(-INFINITY), lane < NW ? lds_s[c][lane] : T(0)};
-      ms = ms_wave_reduce(t);
+    for (int e = 0; e < NV; e++) {
+      const T ex = dev_exp(rv[i][e] - mref);
+      rv[i][e] = ex;
+      st = st + ex;
     }
-    const T logS = dev_log(ms.s);
-    // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
-    const T f = (mt == T(-INFINITY) ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
-    if (colok && tl == 0) loss[col] = lab[c] > 0 ? -((alab[c] - ms.m) - logS) : T(0);
+  if (NV > 1) {
+    xh = dev_exp(xh - mref);
+    xt = dev_exp(xt - mref);
+    st = st + xh + xt;
+  }
+  MaxSum<T> ms = {mt, st};
+  ms = ms_wave_reduce(ms);
+  if (NW > 1) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (lane == 0) { lds_m[wave] = ms.m; lds_s[wave] = ms.s; }
+    __syncthreads();
+    MaxSum<T> t = {lane < NW ? lds_m[lane] : ninf, lane < NW ? lds_s[lane] : T(0)};
+    ms = ms_wave_reduce(t);
+  }
+  const T logS = dev_log(ms.s);
+  // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
+  const T f = (mt == ninf ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
+  if (colok && tl == 0) loss[col] = lab > 0 ? -((alab - ms.m) - logS) : T(0);
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++) {
-      if (!(colok && i < cnt)) continue;
-      const int r = (tl + i * TEAM) * NV;
-      V vo;
+  for (int i = 0; i < ITEMS; i++) {
+    if (i >= cnt) continue;
+    const int r = head + (tl + i * TEAM) * NV;
+    V vo;
 #pragma unroll
-      for (int e = 0; e < NV; e++) {
-        const T p = rv[c][i][e] * f;
-        const T dlp = (r + e + 1 == lab[c]) ? -scale : T(0);
-        vo[e] = lab[c] == 0 ? T(0) : dlp + p;
-      }
-      if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
-      else __builtin_nontemporal_store(vo[0], oc + r);
+    for (int e = 0; e < NV; e++) {
+      const T p = rv[i][e] * f;
+      const T dlp = (r + e + 1 == lab) ? -scale : T(0);
+      vo[e] = lab == 0 ? T(0) : dlp + p;
     }
+    if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+    else __builtin_nontemporal_store(vo[0], oc + r);
+  }
+  if (NV > 1) {
+    if (hv) oc[tl] = lab == 0 ? T(0) : ((tl + 1 == lab) ? -scale : T(0)) + xh * f;
+    if (tv) oc[tpos] = lab == 0 ? T(0) : ((tpos + 1 == lab) ? -scale : T(0)) + xt * f;
   }
 }
 
@@ -473,16 +499,16 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
   constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   const dim3 block(BT);
-  // COLS (columns per team, all loads issued up front) is 1: measured on (32000,512), two columns per workgroup brought
-  // nothing for the fused nll kernel (23.0 us either way) and cost 8 % on the forward kernels -- both phases are limited by
-  // HBM itself, not by the bubbles between them.  The kernels keep the parameter for that measurement.
+  // (Handling two columns per team with the loads of both issued up front was measured on (32000,512): nothing for the fused nll
+  // kernel, 23.0 us either way, and 8 % slower forward kernels -- both phases are limited by HBM itself, not by the bubbles
+  // between them.)
   const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS));
   if constexpr (Algo::kNll) {
-    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true, 1>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
-    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false, 1>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
   } else {
-    if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true, 1>), grid, block, 0, stream, m, n, a, b, out);
-    else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false, 1>), grid, block, 0, stream, m, n, a, b, out);
+    if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out);
+    else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out);
   }
 }
 
@@ -496,11 +522,16 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   constexpr int kHeld = (Algo::kInputs == 2 && Algo::kHoldA) ? 2 : 1;
   constexpr int kBig = 64 / kHeld;
   constexpr int kBig1024 = 256 / (int)(sizeof(T) * kHeld);
-  const bool vec = (m % N == 0) && aligned16(a) && aligned16(out) && (Algo::kInputs == 1 || aligned16(b));
+  // resident kernels: vectors whenever the operands are congruent modulo 16 bytes (each column is cut at its own aligned address);
+  // streaming kernel: whole columns of vectors only
+  const uintptr_t ma = reinterpret_cast<uintptr_t>(a) % 16, mo = reinterpret_cast<uintptr_t>(out) % 16;
+  const uintptr_t mb = Algo::kInputs == 2 ? reinterpret_cast<uintptr_t>(b) % 16 : ma;
+  const bool vec = ma == mo && ma == mb && ma % sizeof(T) == 0;
+  const bool vec_stream = (m % N == 0) && ma == 0 && mo == 0 && mb == 0;
   const long resident_cap = tuning(kTuneSoftmaxResidentRows);  // 0: no limit below the register capacity (tests lower it to reach the streaming kernel with short columns)
 #define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
   if ((resident_cap > 0 && m > resident_cap) || m > 1024L * kBig1024) {
-    if (vec) hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, true>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
+    if (vec_stream) hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, true>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     else hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, false>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     return;
   }
