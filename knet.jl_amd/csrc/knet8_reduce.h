@@ -111,15 +111,28 @@ __global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x,
 // lane; the four waves of a workgroup take k = k0+wave, k0+wave+4, ...; P workgroups split the k range.
 // The same walk (rows `stride` apart, this wave's share of [k0,k1)) combines the P partial tiles at the end
 // (ITEM=false: partials are merged as they are, the item map was applied when they were made).
-template <typename T, typename Op, int NV, bool ITEM, int NW, int U>
-__device__ __forceinline__ void strided_walk(const T* base, long stride, long k0, long k1, int wave, T (&acc)[NV]) {
+// SC ("scalar, coalesced"): for rows that do not start on 16-byte boundaries (s1 odd) the lane's NV elements are the columns
+// lane, lane+64, ... of the tile instead of NV neighbours, each fetched with its own 4-byte load: a wave instruction still reads
+// 256 contiguous bytes and a lane keeps as many bytes in flight as on the vector path.  `livemask` bit e: column e of this lane exists.
+template <typename T, typename Op, int NV, bool ITEM, int NW, int U, bool SC = false>
+__device__ __forceinline__ void strided_walk(const T* base, long stride, long k0, long k1, int wave, T (&acc)[NV], unsigned livemask = ~0u) {
   for (long k = k0 + wave; k < k1; k += NW * U) {
     T v[U][NV];
 #pragma unroll
     for (int q = 0; q < U; q++) {
       const long kk = k + q * NW;
       if (kk < k1) {
-        if (NV > 1) {
+        if (SC) {
+#pragma unroll
+          for (int e = 0; e < NV; e++) {
+            if (livemask & (1u << e)) {
+              const T t = __builtin_nontemporal_load(base + kk * stride + e * kWave);
+              v[q][e] = ITEM ? Op::item(t) : t;
+            } else {
+              v[q][e] = Op::init();
+            }
+          }
+        } else if (NV > 1) {
           typedef typename Vec16<T>::type V;
           V t = ld_stream(reinterpret_cast<const V*>(base + kk * stride));
 #pragma unroll
@@ -140,7 +153,7 @@ __device__ __forceinline__ void strided_walk(const T* base, long stride, long k0
   }
 }
 
-template <typename T, typename Op, int NV, int BT, int U>
+template <typename T, typename Op, int NV, int BT, int U, bool SC = false>
 __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
                                                                    unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
   constexpr int TILE = kWave * NV;
@@ -153,19 +166,23 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
   const unsigned p = blockIdx.x % P;
   const long b = group / atiles, at = group % atiles;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const long a0 = at * TILE + (long)lane * NV;
-  const bool live = a0 < s1;           // on the vector path s1 % NV == 0, so a live lane is fully in range
+  // element e of this lane is column a0 + e (vector path: NV neighbours) or a0 + e*64 (SC: interleaved); `slot` is where it sits in the tile
+  const long a0 = at * TILE + (SC ? (long)lane : (long)lane * NV);
+  unsigned livemask = 0;
+#pragma unroll
+  for (int e = 0; e < NV; e++)
+    if (a0 + (SC ? e * kWave : e) < s1) livemask |= 1u << e;   // on the vector path s1 % NV == 0: all or nothing
   const long k0 = (long)p * kchunk;
   long k1 = k0 + kchunk;
   if (k1 > d) k1 = d;
   T acc[NV];
 #pragma unroll
   for (int e = 0; e < NV; e++) acc[e] = Op::init();
-  if (live) strided_walk<T, Op, NV, true, NW, U>(x + b * s1 * d + a0, s1, k0, k1, wave, acc);
+  if (livemask) strided_walk<T, Op, NV, true, NW, U, SC>(x + b * s1 * d + a0, s1, k0, k1, wave, acc, livemask);
   if (P > 1) {
     // partial tile p of this group = this workgroup's reduction over its k range
 #pragma unroll
-    for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+    for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
     __syncthreads();
     if (threadIdx.x < TILE) {
       T r = Op::init();
@@ -176,11 +193,11 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
     if (!last_block_ticket(counters + group, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
-    strided_walk<T, Op, NV, false, NW, U>(partial + group * P * TILE + lane * NV, TILE, 0, P, wave, acc);
+    strided_walk<T, Op, NV, false, NW, U, SC>(partial + group * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
     if (threadIdx.x == 0) st_coherent(counters + group, 0u);
   }
 #pragma unroll
-  for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+  for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
   __syncthreads();
   const long a = at * TILE + threadIdx.x;
   if (threadIdx.x < TILE && a < s1) {
@@ -281,8 +298,10 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   const dim3 grid((unsigned)(ny * P));
 #define KNET8_RUN(NV, SINGLE, BT, U) \
   hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE, BT, U>), grid, dim3(BT), 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters)
+  // (the scalar path, for runs that do not start on 16-byte boundaries, keeps four times as many loads in flight per lane to move the same bytes)
 #define KNET8_RUN_BT(NV, SINGLE) \
-  do { if (bt == 64) KNET8_RUN(NV, SINGLE, 64, 8); else if (bt == 256) KNET8_RUN(NV, SINGLE, 256, 4); else KNET8_RUN(NV, SINGLE, 512, 4); } while (0)
+  do { if (bt == 64) KNET8_RUN(NV, SINGLE, 64, (NV == 1 ? 16 : 8)); else if (bt == 256) KNET8_RUN(NV, SINGLE, 256, (NV == 1 ? 16 : 4)); \
+       else KNET8_RUN(NV, SINGLE, 512, (NV == 1 ? 16 : 4)); } while (0)
   if (vec) { if (no == 1) KNET8_RUN_BT(N, true); else KNET8_RUN_BT(N, false); }
   else     { if (no == 1) KNET8_RUN_BT(1, true); else KNET8_RUN_BT(1, false); }
 #undef KNET8_RUN_BT
@@ -307,8 +326,8 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
     return;
   }
   const bool vec = aligned16(x) && (s1 % N == 0);
-  const int nv = vec ? N : 1;
-  const long tile = (long)kWave * nv;
+  // rows that do not start on 16-byte boundaries: the same tile width from N interleaved 4- or 8-byte loads per lane
+  const long tile = (long)kWave * N;
   const long atiles = ceil_div(s1, tile);
   const long groups = atiles * nb;
   unsigned P = plan_parts(groups, d, 64);
@@ -320,10 +339,10 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   const dim3 grid((unsigned)(groups * P));
   T* partial = static_cast<T*>(ws.partial);
   const bool big = kchunk >= 128;  // sixteen waves share a tile when each still gets >= 8 rows
-#define KNET8_STR(NV, BT, U) \
-  hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters)
-  if (vec) { if (big) KNET8_STR(N, 1024, 2); else KNET8_STR(N, 256, 8); }
-  else     { if (big) KNET8_STR(1, 1024, 2); else KNET8_STR(1, 256, 8); }
+#define KNET8_STR(NV, BT, U, SC) \
+  hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U, SC>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters)
+  if (vec) { if (big) KNET8_STR(N, 1024, 2, false); else KNET8_STR(N, 256, 8, false); }
+  else     { if (big) KNET8_STR(N, 1024, 2, true); else KNET8_STR(N, 256, 8, true); }
 #undef KNET8_STR
 }
 
