@@ -58,7 +58,9 @@ inline void launch_bias_act(hipStream_t stream, long m, long n, const T* z, cons
 // P workgroups split the columns of a tile and the last one to finish adds their partial sums (same ticket
 // scheme as the strided reduction).  F(dy, y) is the element gradient.  dz may be dy or y itself (each element is read
 // before the same lane writes it).
-template <typename T, typename F, int NV, int BT, int U>
+// SC: rows that do not start on 16-byte boundaries (m odd) -- the lane's NV elements are the rows lane, lane+64, ... of the tile,
+// each moved with its own 4- or 8-byte access (see strided_walk).
+template <typename T, typename F, int NV, int BT, int U, bool SC>
 __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const T* yv, long m, long n, long jchunk, unsigned P, T* dz, T* __restrict__ db,
                                                               T* partial, unsigned* counters, F f) {
   constexpr int TILE = kWave * NV;
@@ -68,15 +70,18 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
   const long at = blockIdx.x / P;
   const unsigned p = blockIdx.x % P;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const long a0 = at * TILE + (long)lane * NV;
-  const bool live = a0 < m;
+  const long a0 = at * TILE + (SC ? (long)lane : (long)lane * NV);
+  unsigned livemask = 0;
+#pragma unroll
+  for (int e = 0; e < NV; e++)
+    if (a0 + (SC ? e * kWave : e) < m) livemask |= 1u << e;   // vector path: m % NV == 0, all or nothing
   const long j0 = (long)p * jchunk;
   long j1 = j0 + jchunk;
   if (j1 > n) j1 = n;
   T acc[NV];
 #pragma unroll
   for (int e = 0; e < NV; e++) acc[e] = T(0);
-  if (live) {
+  if (livemask) {
     for (long j = j0 + wave; j < j1; j += NW * U) {
       T g[U][NV];
 #pragma unroll
@@ -84,7 +89,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
         const long jj = j + q * NW;
         if (jj < j1) {
           const long off = jj * m + a0;
-          if (NV > 1) {
+          if (!SC && NV > 1) {
             typedef typename Vec16<T>::type V;
             const V d = ld_stream(reinterpret_cast<const V*>(dy + off));
             const V o = ld_stream(reinterpret_cast<const V*>(yv + off));
@@ -93,9 +98,16 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
             for (int e = 0; e < NV; e++) { r[e] = f(d[e], o[e]); g[q][e] = r[e]; }
             st_stream(reinterpret_cast<V*>(dz + off), r);
           } else {
-            const T r = f(__builtin_nontemporal_load(dy + off), __builtin_nontemporal_load(yv + off));
-            g[q][0] = r;
-            __builtin_nontemporal_store(r, dz + off);
+#pragma unroll
+            for (int e = 0; e < NV; e++) {
+              if (livemask & (1u << e)) {
+                const T r = f(__builtin_nontemporal_load(dy + off + e * kWave), __builtin_nontemporal_load(yv + off + e * kWave));
+                g[q][e] = r;
+                __builtin_nontemporal_store(r, dz + off + e * kWave);
+              } else {
+                g[q][e] = T(0);
+              }
+            }
           }
         } else {
 #pragma unroll
@@ -110,7 +122,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
   }
   if (P > 1) {
 #pragma unroll
-    for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+    for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
     __syncthreads();
     if (threadIdx.x < TILE) {
       T r = T(0);
@@ -121,11 +133,11 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
     if (!last_block_ticket(counters + at, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = T(0);
-    strided_walk<T, RedSum<T>, NV, false, NW, U>(partial + at * P * TILE + lane * NV, TILE, 0, P, wave, acc);
+    strided_walk<T, RedSum<T>, NV, false, NW, U, SC>(partial + at * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
     if (threadIdx.x == 0) st_coherent(counters + at, 0u);
   }
 #pragma unroll
-  for (int e = 0; e < NV; e++) lds[wave][lane * NV + e] = acc[e];
+  for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
   __syncthreads();
   const long a = at * TILE + threadIdx.x;
   if (threadIdx.x < TILE && a < m) {
@@ -141,8 +153,7 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   if (m <= 0) return;
   constexpr int N = Vec16<T>::N;
   const bool vec = (m % N == 0) && aligned16(dy) && aligned16(y) && aligned16(dz);
-  const int nv = vec ? N : 1;
-  const long tile = (long)kWave * nv;
+  const long tile = (long)kWave * N;
   const long atiles = ceil_div(m, tile);
   unsigned P = n > 0 ? plan_parts(atiles, n, 32) : 1;
   long jchunk = ceil_div(n, P);
@@ -153,10 +164,10 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   const dim3 grid((unsigned)(atiles * P));
   T* partial = static_cast<T*>(ws.partial);
   const bool big = jchunk >= 64;
-#define KNET8_ABG(NV, BT, U) \
-  hipLaunchKernelGGL((actback_biasgrad_kernel<T, F, NV, BT, U>), grid, dim3(BT), 0, stream, dy, y, m, n, jchunk, P, dz, db, partial, ws.counters, f)
-  if (vec) { if (big) KNET8_ABG(N, 1024, 2); else KNET8_ABG(N, 256, 4); }
-  else     { if (big) KNET8_ABG(1, 1024, 2); else KNET8_ABG(1, 256, 4); }
+#define KNET8_ABG(BT, U, SC) \
+  hipLaunchKernelGGL((actback_biasgrad_kernel<T, F, N, BT, U, SC>), grid, dim3(BT), 0, stream, dy, y, m, n, jchunk, P, dz, db, partial, ws.counters, f)
+  if (vec) { if (big) KNET8_ABG(1024, 2, false); else KNET8_ABG(256, 4, false); }
+  else     { if (big) KNET8_ABG(1024, 2, true); else KNET8_ABG(256, 4, true); }
 #undef KNET8_ABG
 }
 
