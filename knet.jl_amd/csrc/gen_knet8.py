@@ -451,6 +451,9 @@ def gen_softmax():
     for T, S in TYPES:
         o.entry("transpose_%s" % S, "void", [("int", "m"), ("int", "n"), (T + "*", "x"), (T + "*", "y")],
                 "launch_transpose<%s>(stream, m, n, x, y)" % T, "permutedims(x) for matrices, src/ops20_gpu/softmax.jl:19-20")
+        o.entry("permute213_%s" % S, "void", [("int", "m"), ("int", "n"), ("int", "batch"), (T + "*", "x"), (T + "*", "y")],
+                "launch_transpose<%s>(stream, m, n, x, y, batch)" % T,
+                "permutedims(x, (2,1,3)) of an (m, n, batch) array (CUDA.jl's permutedims in the reference, src/knetarrays/reshape.jl:18)")
     o.decl.append("\n/* ---- gather / scatter on 1-based int32 linear indices -- src/libknet8/cuda1.jl:342-362 ---- */")
     for T, S in TYPES:
         o.entry("getents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],

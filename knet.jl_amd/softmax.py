@@ -53,6 +53,16 @@ def _bwd(kernel, y, dy, m, n):
     return dx
 
 
+_STRIDED_MAX = 1 << 14  # elements; above this the lane-per-slice kernel has too few lanes or too long walks
+
+
+def _permute213(x, m, n, batch):
+    """``permutedims(reshape(x, m, n, batch), (2,1,3))`` -> ``permute213_S``."""
+    y = x.similar((n, m, batch))
+    knet8("permute213_%s" % x.suffix, m, n, batch, x.ptr, y.ptr)
+    return y
+
+
 def permutedims(x):
     """2-d transpose (the reference uses CUDA.jl's permutedims, src/knetarrays/reshape.jl:18)."""
     from .linalg import transpose
@@ -72,7 +82,24 @@ def _make(kernel, backkernel):
             y = _fwd(kernel, x, m, n)
             return y, (lambda dy: (_bwd(backkernel, y, dy, m, n),))  # @primitive1 _cudnnSoftmaxForward(x),dy,y _cudnnSoftmaxBackward(y,dy)
         v3 = _view3(x, dims)
-        if v3 is not None:  # a run of adjacent non-leading dims: one strided kernel instead of the reference's transposes/broadcast chain
+        if v3 is not None and v3[0] == 1:  # leading dims of size 1: the slices are contiguous columns after all
+            _, d, outer = v3
+            y = _fwd(kernel, x, d, outer)
+            return y, (lambda dy: (_bwd(backkernel, y, dy, d, outer),))
+        if v3 is not None and x.length > _STRIDED_MAX:
+            # A run of adjacent non-leading dims of a large array: permute (inner, d, outer) -> (d, inner, outer), run the column kernels
+            # on contiguous columns of length d, permute back -- the reference's route for 2-d dims=2 (src/ops20_gpu/softmax.jl:19-20),
+            # batched over the trailing dims.  The transposed result is kept for the backward pass, which needs exactly that.
+            inner, d, outer = v3
+            xt = _permute213(x, inner, d, outer)
+            yt = _fwd(kernel, xt, d, inner * outer)
+            y = _permute213(yt, d, inner, outer).reshape(x.dims)
+
+            def back_t(dy):
+                dxt = _bwd(backkernel, yt, _permute213(dy, inner, d, outer), d, inner * outer)
+                return (_permute213(dxt, d, inner, outer).reshape(x.dims),)
+            return y, back_t
+        if v3 is not None:  # small arrays: one strided kernel (a lane per slice) instead of three launches
             inner, d, outer = v3
             y = x.similar()
             knet8("%s_strided_%s" % (kernel, x.suffix), inner, d, outer, x.ptr, y.ptr)

@@ -226,3 +226,26 @@ def test_threads_with_their_own_streams(knet):
         t.join()
     assert not errors, errors
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt,S", [(np.float32, "32"), (np.float64, "64")])
+def test_transpose_and_batched_permutation(knet, dt, S):
+    """transpose_S and permute213_S against numpy, over the tile kernel (both sides > 32), the skinny kernel (one side <= 32, either
+    one), ragged edges and batches."""
+    rng = np.random.default_rng(57)
+    for (m, n, batch) in [(1, 1, 1), (3, 5, 1), (64, 64, 1), (65, 130, 3), (8, 1000, 4), (1000, 8, 4), (1, 5000, 2), (5000, 1, 2), (32, 4097, 1),
+                          (4097, 32, 2), (33, 70, 5), (300, 257, 2), (7, 64, 3), (2, 70000, 1)]:
+        x = rng.standard_normal((batch, n, m)).astype(dt)      # numpy (batch, n, m) C-order == column-major (m, n, batch)
+        xd = knet.KnetArray(dtype=dt, dims=(m, n, batch))
+        fn = knet.libknet8().fn
+        fn["knet8_memcpy"](xd.ptr, np.ascontiguousarray(x).ctypes.data, x.nbytes, 1, knet.libknet8().stream)
+        yd = knet.KnetArray(dtype=dt, dims=(n, m, batch))
+        knet.knet8("permute213_%s" % S, m, n, batch, xd.ptr, yd.ptr)
+        got = knet.Array(yd)                                      # column-major (n, m, batch)
+        want = np.transpose(x, (0, 2, 1))                         # (batch, m, n) C-order == column-major (n, m, batch)
+        assert bits_equal(np.ascontiguousarray(np.transpose(got, (2, 1, 0))), np.ascontiguousarray(want)), (m, n, batch)
+        if batch == 1:
+            y2 = knet.KnetArray(dtype=dt, dims=(n, m))
+            knet.knet8("transpose_%s" % S, m, n, xd.ptr, y2.ptr)
+            assert bits_equal(knet.Array(y2), knet.Array(yd).reshape(n, m)), (m, n)
+    knet.libknet8().check()
