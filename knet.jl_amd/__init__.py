@@ -11,7 +11,7 @@ from .autograd import Param, diff, grad, value, recording
 from .activation import (bias_act, relu, sigm, tanh, elu, selu, reluback, sigmback, tanhback, eluback, seluback,
                          gelu, hardsigmoid, hardswish, swish, tanh_, geluback, hardsigmoidback, hardswishback,
                          swishback, tanh_back, eluback21, seluback21, sigmback21, relu_kw, relu_kw_back,
-                         unary_op, back11_op, back111_op)
+                         unary_op, unary_op_with_degree, back11_op, back111_op)
 from .reduction import sum, prod, maximum, minimum, sumabs, sumabs2, maxabs, minabs, countnz, reduce_op
 from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
 from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback

@@ -36,6 +36,15 @@ def unary_op(name, x):
     return y
 
 
+def unary_op_with_degree(name, d, x):
+    """``y = similar(x); @knet8(F_S, (Cint,Cint,Ptr,Ptr), length(y), d, x, y)``: ``besselj.(d,x)`` -> ``jn``, ``bessely.(d,x)`` ->
+    ``yn`` (src/knetarrays/unary.jl:47-60)."""
+    _check(x)
+    y = x.similar()
+    knet8("%s_%s" % (name, x.suffix), x.length, int(d), x.ptr, y.ptr)
+    return y
+
+
 def back11_op(name, dy, y):
     """``z = similar(x); @knet8(Fback_S_11, ..., length(z), dy, y, z)`` (src/ops20_gpu/activation.jl:33-37)."""
     _check(dy, y)

@@ -93,6 +93,14 @@ UNARY_OPS = [
     ("y1", "return ky1(xi);", "src/libknet8/ops.jl:64 (y1)"),
     ("lgamma", "return klgamma(xi);", "src/libknet8/ops.jl:34"),
     ("gamma_impl", "return ktgamma(xi);", "src/libknet8/ops.jl:33 (gamma_impl, src/libknet8/gamma.jl)"),
+    ("digamma_impl", "return kdigamma<T>(xi);", "src/libknet8/ops.jl:35, src/libknet8/gamma.jl:72-124 (poles return the largest finite T)"),
+    ("trigamma_impl", "return ktrigamma<T>(xi);", "src/libknet8/ops.jl:36, src/libknet8/gamma.jl:221-239 (zeta(2,x); poles return the largest finite T)"),
+]
+
+# Unary ops with an integer degree NAME_S(n, d, x, y): name, device routine, citation (src/libknet8/ops.jl:138-141).
+INT_DEGREE_OPS = [
+    ("jn", "kbesselj", "src/libknet8/ops.jl:139, src/libknet8/cuda1.jl:49-79 (besselj(d,x), any integer d)"),
+    ("yn", "kbessely", "src/libknet8/ops.jl:140, src/libknet8/cuda1.jl:49-79 (bessely(d,x); NaN for x < 0)"),
 ]
 
 # name, body in terms of (xi, yi), citation.  Used for the _01, _11 and _12/_13 entry points.
@@ -125,6 +133,13 @@ BACK11_OPS = [
      "src/ops20/activation.jl:40, src/libknet8/ops.jl:119"),
 ]
 
+# The reference's binary table also carries geluback and swishback with xi = x, yi = dy (src/libknet8/ops.jl:110,116): same
+# arithmetic as the three-input forms below.
+def _back_as_binary(name):
+    body = [b for n, b, _ in BACK111_OPS if n == name][0]
+    return "const T x = xi; const T dy = yi; " + body
+
+
 # Three-input gradients NAME_S_111(n, x, y, dy, dx).
 BACK111_OPS = [
     ("eluback", "if (y >= T(0)) return dy; const T b = T(1) + y; return dy * b;", "src/ops21/activation.jl:17, src/libknet8/ops.jl:126"),
@@ -143,6 +158,13 @@ BACK111_OPS = [
                   "else { const T z = kexp(x); const T s = (x + z) + T(1); const T num = z * s; const T d = z + T(1); g = num / (d * d); } return dy * g;",
      "src/ops21/activation.jl:171, src/libknet8/ops.jl:135"),
 ]
+
+BACKBIN_OPS = [("geluback", _back_as_binary("geluback"), "src/libknet8/ops.jl:110 (xi = x, yi = dy)"),
+               ("swishback", _back_as_binary("swishback"), "src/libknet8/ops.jl:116 (xi = x, yi = dy)")]
+
+# Every row of the reference's binary table: the generators of the scalar and broadcast forms loop over all of them
+# (src/libknet8/cuda01.jl:32, cuda12.jl:40, cuda13.jl:190, cuda16.jl:105, cuda17.jl:70), the gradient rows included.
+ALL_BINARY_OPS = BINARY_OPS + BACK11_OPS + BACKBIN_OPS
 
 # Fused optimizer updates: name, scalar parameters (all of type T, derived on the host exactly as the Julia code derives
 # them: T(-lr), T(1-rho), T(1-beta1^t) ...), arrays (in order), write mask, body on v[...], citation.  Each body is the
@@ -206,6 +228,7 @@ class Out:
 
 PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_elementwise.h"
+#include "../knet8_special.h"
 #include "../knet8_broadcast.h"
 #include "../knet8_reduce.h"
 #include "../knet8_fused.h"
@@ -222,31 +245,24 @@ def functor(name, args, body, extra_fields=""):
             % (name, extra_fields, ", ".join("T " + a for a in args), body))
 
 
-def gen_elementwise():
+def binary_functors():
+    out = []
+    for name, body, cite in BINARY_OPS + BACKBIN_OPS:
+        out.append(functor("Op2_" + name, ["xi", "yi"], body))
+    for name, body, cite in BACK11_OPS:
+        out.append(functor("Op11_" + name, ["xi", "yi"], body))
+        out.append("template <typename T> using Op2_%s = Op11_%s<T>;\n" % (name, name))
+    return "\n".join(out)
+
+
+def gen_broadcast():
     o = Out()
     s = o.src
     s.append(PRELUDE)
-    o.decl.append("\n/* ---- elementwise forward: y[i] = f(x[i]) -- src/libknet8/cuda1.jl:13-38 ---- */")
-    for name, body, cite in UNARY_OPS:
-        s.append(functor("Op_" + name, ["xi"], body))
-        for T, S in TYPES:
-            o.entry("%s_%s" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y")],
-                    "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, y, Op_%s<%s>())" % (T, T, T, name, T), cite)
-    o.decl.append("\n/* ---- scalar (op) array: z[i] = f(xi, y[i]) -- src/libknet8/cuda01.jl:11-25 ---- */")
-    for name, body, cite in BINARY_OPS:
-        s.append(functor("Op2_" + name, ["xi", "yi"], body))
-        s.append("template <typename T> struct Op01_%s { T xi; __device__ __forceinline__ T operator()(T yi) const { return Op2_%s<T>()(xi, yi); } };\n" % (name, name))
-        for T, S in TYPES:
-            o.entry("%s_%s_01" % (name, S), "void", [("int", "n"), (T, "xi"), (T + "*", "y"), (T + "*", "z")],
-                    "launch_ew<%s, 1>(stream, n, y, (const %s*)nullptr, (const %s*)nullptr, z, Op01_%s<%s>{xi})" % (T, T, T, name, T), cite)
-    o.decl.append("\n/* ---- same-shape binary: z[i] = f(x[i], y[i]) -- src/libknet8/cuda11.jl:12-28 ---- */")
-    for name, body, cite in BINARY_OPS:
-        for T, S in TYPES:
-            o.entry("%s_%s_11" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y"), (T + "*", "z")],
-                    "launch_ew<%s, 2>(stream, n, x, y, (const %s*)nullptr, z, Op2_%s<%s>())" % (T, T, name, T), cite)
+    s.append(binary_functors())
     o.decl.append("\n/* ---- vector broadcast: operand k is full size or a vector along one dim, read as v[(i/s)%n]\n"
                   "   -- src/libknet8/cuda12.jl:18-34; the _13 forms (src/libknet8/cuda13.jl:44-184) take the full array first ---- */")
-    for name, body, cite in BINARY_OPS:
+    for name, body, cite in ALL_BINARY_OPS:
         s.append("template <typename T> struct Op2r_%s { __device__ __forceinline__ T operator()(T full, T vec) const { return Op2_%s<T>()(vec, full); } };\n" % (name, name))
         for T, S in TYPES:
             o.entry("%s_%s_12" % (name, S), "void",
@@ -263,7 +279,7 @@ def gen_elementwise():
     o.decl.append("\n/* ---- general N-d broadcast: element strides per dimension, 0 for a broadcast dimension; z contiguous with N elements.\n"
                   "   _16_3/_16_4/_16_5 take the strides by value (src/libknet8/cuda16.jl:10-88), _17 in device int arrays of length\n"
                   "   dimlen_z (src/libknet8/cuda17.jl:25-64); caller src/knetarrays/binary.jl:96-125 ---- */")
-    for name, body, cite in BINARY_OPS:
+    for name, body, cite in ALL_BINARY_OPS:
         for T, S in TYPES:
             for nd in (3, 4, 5):
                 ps = [(T + "*", "x"), (T + "*", "y"), (T + "*", "z")]
@@ -278,9 +294,40 @@ def gen_elementwise():
                     [(T + "*", "x"), (T + "*", "y"), (T + "*", "z"), ("int*", "stride_x"), ("int*", "stride_y"), ("int*", "stride_z"), ("int", "N_z"), ("int", "dimlen_z")],
                     "launch_bcast17<%s>(stream, x, y, z, stride_x, stride_y, stride_z, N_z, dimlen_z, Op2_%s<%s>())" % (T, name, T),
                     "src/libknet8/cuda17.jl:58-64")
+    return o
+
+
+def gen_elementwise():
+    o = Out()
+    s = o.src
+    s.append(PRELUDE)
+    o.decl.append("\n/* ---- elementwise forward: y[i] = f(x[i]) -- src/libknet8/cuda1.jl:13-38 ---- */")
+    for name, body, cite in UNARY_OPS:
+        s.append(functor("Op_" + name, ["xi"], body))
+        for T, S in TYPES:
+            o.entry("%s_%s" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y")],
+                    "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, y, Op_%s<%s>())" % (T, T, T, name, T), cite)
+    # functors of every row of the binary table: Op2_NAME(xi, yi); the gradient rows keep their Op11_ names (xi = dy, yi = y)
+    s.append(binary_functors())
+    o.decl.append("\n/* ---- scalar (op) array: z[i] = f(xi, y[i]) -- src/libknet8/cuda01.jl:11-25 ---- */")
+    for name, body, cite in ALL_BINARY_OPS:
+        s.append("template <typename T> struct Op01_%s { T xi; __device__ __forceinline__ T operator()(T yi) const { return Op2_%s<T>()(xi, yi); } };\n" % (name, name))
+        for T, S in TYPES:
+            o.entry("%s_%s_01" % (name, S), "void", [("int", "n"), (T, "xi"), (T + "*", "y"), (T + "*", "z")],
+                    "launch_ew<%s, 1>(stream, n, y, (const %s*)nullptr, (const %s*)nullptr, z, Op01_%s<%s>{xi})" % (T, T, T, name, T), cite)
+    o.decl.append("\n/* ---- same-shape binary: z[i] = f(x[i], y[i]) -- src/libknet8/cuda11.jl:12-28 ---- */")
+    for name, body, cite in BINARY_OPS + BACKBIN_OPS:
+        for T, S in TYPES:
+            o.entry("%s_%s_11" % (name, S), "void", [("int", "n"), (T + "*", "x"), (T + "*", "y"), (T + "*", "z")],
+                    "launch_ew<%s, 2>(stream, n, x, y, (const %s*)nullptr, z, Op2_%s<%s>())" % (T, T, name, T), cite)
+    o.decl.append("\n/* ---- unary functions with an integer degree: y[i] = f(d, x[i]) -- src/libknet8/cuda1.jl:49-79 ---- */")
+    for name, fn, cite in INT_DEGREE_OPS:
+        s.append("template <typename T> struct OpDeg_%s { int d; __device__ __forceinline__ T operator()(T xi) const { return %s<T>(d, xi); } };\n" % (name, fn))
+        for T, S in TYPES:
+            o.entry("%s_%s" % (name, S), "void", [("int", "n"), ("int", "d"), (T + "*", "x"), (T + "*", "y")],
+                    "launch_ew<%s, 1>(stream, n, x, (const %s*)nullptr, (const %s*)nullptr, y, OpDeg_%s<%s>{d})" % (T, T, T, name, T), cite)
     o.decl.append("\n/* ---- activation gradients dx[i] = f(dy[i], y[i]) -- src/libknet8/cuda11.jl:12-28 with the *back rows of ops.jl:114-121 ---- */")
     for name, body, cite in BACK11_OPS:
-        s.append(functor("Op11_" + name, ["xi", "yi"], body))
         for T, S in TYPES:
             o.entry("%s_%s_11" % (name, S), "void", [("int", "n"), (T + "*", "dy"), (T + "*", "y"), (T + "*", "dx")],
                     "launch_ew<%s, 2>(stream, n, dy, y, (const %s*)nullptr, dx, Op11_%s<%s>())" % (T, T, name, T), cite)
@@ -576,7 +623,7 @@ HEADER_BOTTOM = """
 
 
 def generate(write=True):
-    units = {"knet8_elementwise_gen.hip": gen_elementwise(), "knet8_reduce_gen.hip": gen_reduce(), "knet8_softmax_gen.hip": gen_softmax()}
+    units = {"knet8_elementwise_gen.hip": gen_elementwise(), "knet8_broadcast_gen.hip": gen_broadcast(), "knet8_reduce_gen.hip": gen_reduce(), "knet8_softmax_gen.hip": gen_softmax()}
     files = {}
     for fn, o in units.items():
         files[os.path.join(GEN, fn)] = "\n".join(o.src) + "\n"

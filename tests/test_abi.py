@@ -45,6 +45,18 @@ def test_library_exports_every_declared_symbol(built_lib):
         assert needed in decls, needed
 
 
+def test_every_symbol_of_the_reference_library_is_exported(built_lib):
+    """tests/golden/libknet8_symbols.txt lists what the reference's generator scripts export (op tables of
+    src/libknet8/ops.jl x the patterns of the scripts src/libknet8/build.jl:43-55 builds): a drop-in libknet8.so has them all."""
+    names = open(os.path.join(ROOT, "tests", "golden", "libknet8_symbols.txt")).read().split()
+    assert len(names) > 1200
+    lk = _load("lk_for_test2", "knet.jl_amd/libknet8.py")
+    decls = lk.parse_header()
+    lib = ctypes.CDLL(built_lib)
+    assert not [n for n in names if n not in decls]
+    assert not [n for n in names if not hasattr(lib, n)]
+
+
 def test_no_undefined_device_runtime_surprises(built_lib):
     # the product must not link the oracle or anything outside HIP / hipBLASLt / the C++ runtime
     out = subprocess.check_output(["readelf", "-d", built_lib], text=True)

@@ -299,6 +299,94 @@ def test_libm_unary_table(knet, dt):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_digamma_trigamma_and_integer_order_bessel(knet, dt):
+    """digamma_impl / trigamma_impl (src/libknet8/ops.jl:35-36, src/libknet8/gamma.jl) and jn / yn with an integer degree
+    (src/libknet8/ops.jl:139-140; the reference tests besselj.(2,x) and bessely.(2,x), test/unary.jl:31-32) against mpmath.
+    The library evaluates them in fp64 and rounds once: fp32 within 1 ulp; fp64 within 16 ulp at max(|f|, 1) -- the routines'
+    absolute error lives at the size of the cancelling terms (log x against the recurrence sum; the oscillating Bessel values)."""
+    import mpmath as mp
+    mp.mp.prec = 160
+    rng = np.random.default_rng(31)
+    tol = 1 if dt == np.float32 else 16
+
+    def check(name, got, f, x, floor=1.0):
+        want = np.array([float(f(mp.mpf(float(v)))) for v in x])
+        want = np.where(np.abs(want) > np.finfo(dt).max, np.sign(want) * np.inf, want)  # beyond T's range: the rounded result is +-Inf
+        err = ulp_diff(got, want, scale=np.maximum(np.abs(want), floor))
+        assert err.max() <= tol + 0.5, (name, float(err.max()), float(x[np.argmax(err)]))
+
+    x = np.concatenate([rng.uniform(-30, 30, 1200), rng.uniform(0, 2, 300), rng.uniform(50, 1e6, 100), rng.standard_normal(400)]).astype(dt)
+    frac = np.abs(x - np.rint(x))
+    x = x[(x > 0) | (frac > 0.05)]  # near a pole of the negative axis the condition number, not the routine, sets the error
+    xd = knet.KnetArray(x)
+    check("digamma", knet.Array(knet.unary_op("digamma_impl", xd)), lambda v: mp.psi(0, v), x, floor=1e-6 if dt == np.float32 else 1.0)
+    check("trigamma", knet.Array(knet.unary_op("trigamma_impl", xd)), lambda v: mp.psi(1, v), x)
+    # poles: the largest finite value, as the reference's routines return it
+    poles = np.array([0.0, -1.0, -2.0, -17.0], dtype=dt)
+    for name in ("digamma_impl", "trigamma_impl"):
+        assert np.all(knet.Array(knet.unary_op(name, knet.KnetArray(poles))) == np.finfo(dt).max), name
+    # closed forms: psi(1) = -gamma, psi(1/2) = -gamma - 2 ln 2, psi1(1) = pi^2/6, psi1(1/2) = pi^2/2
+    pts = knet.KnetArray(np.array([1.0, 0.5], dtype=dt))
+    assert ulp_diff(knet.Array(knet.unary_op("digamma_impl", pts)), np.array([-np.euler_gamma, -np.euler_gamma - 2 * np.log(2)])).max() <= 2
+    assert ulp_diff(knet.Array(knet.unary_op("trigamma_impl", pts)), np.array([np.pi ** 2 / 6, np.pi ** 2 / 2])).max() <= 2
+    xb = np.concatenate([rng.uniform(-60, 60, 500), rng.uniform(0, 3, 100), rng.uniform(100, 3000, 30)]).astype(dt)
+    xbd = knet.KnetArray(xb)
+    xpos = np.abs(xb) + dt(0.05)
+    xposd = knet.KnetArray(xpos)
+    for d in (2, 3, 7, 20, 64, -2, -3, 0, 1):
+        got = knet.Array(knet.unary_op_with_degree("jn", d, xbd))
+        check("jn%d" % d, got, lambda v: mp.besselj(d, v), xb, floor=1.0 if dt == np.float64 else 1e-3)
+        got = knet.Array(knet.unary_op_with_degree("yn", d, xposd))
+        check("yn%d" % d, got, lambda v: mp.bessely(d, v), xpos, floor=1.0 if dt == np.float64 else 1e-3)
+    # recurrence identity J_{n-1} + J_{n+1} = (2n/x) J_n ties the orders together without any reference routine
+    j = [knet.Array(knet.unary_op_with_degree("jn", d, xposd)).astype(np.float64) for d in (4, 5, 6)]
+    assert np.abs(j[0] + j[2] - (10.0 / xpos) * j[1]).max() <= (1e-5 if dt == np.float32 else 1e-13)
+    edge = knet.KnetArray(np.array([0.0, -1.0, np.inf], dtype=dt))
+    assert np.array_equal(knet.Array(knet.unary_op_with_degree("jn", 3, edge))[[0, 2]], np.array([0, 0], dtype=dt))
+    yn = knet.Array(knet.unary_op_with_degree("yn", 2, edge))
+    assert yn[0] == -np.inf and np.isnan(yn[1]) and yn[2] == 0
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gradient_rows_in_every_broadcast_form(knet, oracle, dt):
+    """The reference generates the scalar and broadcast forms for every row of its binary table, the *back rows included
+    (src/libknet8/cuda01.jl:32, cuda12.jl:40, cuda13.jl:190, cuda16.jl:105, cuda17.jl:70): each must equal the same-shape
+    kernel applied to the operands broadcast on the host."""
+    rng = np.random.default_rng(32)
+    dy = rng.standard_normal((6, 5, 4)).astype(dt)
+    ycol = rng.standard_normal((6, 1, 1)).astype(dt)
+    yrow = rng.standard_normal((1, 5, 1)).astype(dt)
+    full = rng.standard_normal((6, 5, 4)).astype(dt)
+    names = ["reluback", "sigmback", "tanhback", "eluback", "seluback", "invxback", "geluback", "swishback"]
+    for name in names:
+        def same_shape(a, b):
+            a, b = np.broadcast_arrays(a, b)
+            ad, bd, z = knet.KnetArray(a), knet.KnetArray(b), knet.KnetArray(np.zeros(a.shape, dt))
+            knet.knet8("%s_%s_11" % (name, z.suffix), z.length, ad.ptr, bd.ptr, z.ptr)
+            return knet.Array(z)
+        for a, b in ((dy, ycol), (ycol, dy), (dy, yrow), (yrow, full), (ycol, yrow), (dy, full)):
+            got = knet.Array(knet.broadcast_op(name, knet.KnetArray(a), knet.KnetArray(b)))
+            assert bits_equal(got, same_shape(a, b)), (name, a.shape, b.shape)
+        got = knet.Array(knet.broadcast_op(name, 0.75, knet.KnetArray(full)))            # _01: scalar first operand
+        assert bits_equal(got, same_shape(np.full(full.shape, 0.75, dt), full)), name
+        # 7 dims: the _17 form
+        a7 = rng.standard_normal((2, 1, 3, 1, 2, 1, 2)).astype(dt)
+        b7 = rng.standard_normal((1, 3, 1, 2, 1, 2, 1)).astype(dt)
+        got = knet.Array(knet.broadcast_op(name, knet.KnetArray(a7), knet.KnetArray(b7)))
+        assert bits_equal(got, same_shape(a7, b7)), name
+    # the two-operand geluback/swishback rows (xi = x, yi = dy) agree with the three-operand ops21 kernels
+    x = rng.standard_normal(999).astype(dt)
+    g = rng.standard_normal(999).astype(dt)
+    xd, gd = knet.KnetArray(x), knet.KnetArray(g)
+    for name in ("geluback", "swishback"):
+        two = knet.Array(knet.back11_op(name, xd, gd))
+        three = knet.Array(knet.back111_op(name, xd, xd, gd))
+        assert bits_equal(two, three), name
+    knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_pow_and_comparisons(knet, dt):
     rng = np.random.default_rng(22)
     x = rng.integers(-3, 4, size=(33, 17)).astype(dt)
