@@ -179,13 +179,12 @@ def extras(torch, K):
         res["nll_logsoftmax_back_32 (%d,%d)" % (C, N)] = time_kernel(
             K, torch, lambda i: (lambda: K.knet8("nll_logsoftmax_back_32", C, N, ys[i].ptr, labels.ptr, ctypes.c_float(1.0 / N), dxs[i].ptr, loss.ptr)),
             8 * C * N + 4 * N, list(range(nsets)))
-        if C == 32000:
-            # yardsticks: plain elementwise kernels moving the same bytes over the same buffers -- what this chip delivers to
-            # any kernel of this size, launch ramp and drain included
-            res["yardstick reluback_32_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (C * N, C, N)] = time_kernel(
-                K, torch, lambda i: (lambda: K.knet8("reluback_32_11", C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)), 12 * C * N, list(range(nsets)))
-            res["yardstick relu_32 n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (C * N, C, N)] = time_kernel(
-                K, torch, lambda i: (lambda: K.knet8("relu_32", C * N, ys[i].ptr, dxs[i].ptr)), 8 * C * N, list(range(nsets)))
+        # yardsticks: plain elementwise kernels moving the same bytes over the same buffers -- what this chip delivers to
+        # any kernel of this size, launch ramp and drain included
+        res["yardstick reluback_32_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (C * N, C, N)] = time_kernel(
+            K, torch, lambda i: (lambda: K.knet8("reluback_32_11", C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)), 12 * C * N, list(range(nsets)))
+        res["yardstick relu_32 n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (C * N, C, N)] = time_kernel(
+            K, torch, lambda i: (lambda: K.knet8("relu_32", C * N, ys[i].ptr, dxs[i].ptr)), 8 * C * N, list(range(nsets)))
         del ys, dys, dxs
     # config 5 per-layer dropback
     n5 = 4096 * 2048
