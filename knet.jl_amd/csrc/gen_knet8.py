@@ -229,6 +229,7 @@ class Out:
 PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_elementwise.h"
 #include "../knet8_special.h"
+#include "../knet8_random.h"
 #include "../knet8_broadcast.h"
 #include "../knet8_reduce.h"
 #include "../knet8_fused.h"
@@ -358,6 +359,18 @@ def gen_elementwise():
              "template <typename T> struct OpDropback { T q; __device__ __forceinline__ T operator()(T y, T dy) const { return y == T(0) ? T(0) : dy / q; } };\n")
     s.append("template <typename T> struct OpAxpy { T a; __device__ __forceinline__ T operator()(T x, T y) const { const T p = a * x; return y + p; } };\n")
     s.append("template <typename T> struct OpScal { T a; __device__ __forceinline__ T operator()(T x) const { return a * x; } };\n")
+    o.decl.append("/* rand_S / randn_S: y[0..n) = U[0,1) / N(0,1) from the default stream -- what rand!(a::KnetArray) and randn! take from\n"
+                  "   cuRAND (src/knetarrays/random.jl:5-6; dropout! draws its mask buffer this way, src/ops20_gpu/dropout.jl:14).  The\n"
+                  "   *_seeded forms name the stream position explicitly: Philox4x32-10 with key = seed, counters offset, offset+1, ...\n"
+                  "   (4 fp32 or 2 fp64 values per counter), so element i depends on (seed, offset, i) only.  Under hipGraph capture use the\n"
+                  "   seeded forms: the default stream's position is read at capture time and every replay would repeat it. */")
+    for T, S in TYPES:
+        for name, normal in (("rand", "false"), ("randn", "true")):
+            o.entry("%s_%s" % (name, S), "void", [("int", "n"), (T + "*", "y")], None, "src/knetarrays/random.jl:5-6",
+                    body="  if (n <= 0) return;\n  unsigned long long seed, offset;\n  knet8::rng_take(rand_blocks<%s>(n), &seed, &offset);\n"
+                         "  launch_rand<%s, %s>(stream, n, seed, offset, y);\n  knet8::check_launch(\"%s_%s\");" % (T, T, normal, name, S))
+            o.entry("%s_seeded_%s" % (name, S), "void", [("int", "n"), ("unsigned long long", "seed"), ("unsigned long long", "offset"), (T + "*", "y")],
+                    "launch_rand<%s, %s>(stream, n, seed, offset, y)" % (T, normal), "src/knetarrays/random.jl:5-6 with the generator state passed in")
     for T, S in TYPES:
         o.entry("fill_%s" % S, "void", [("int", "n"), (T, "x"), (T + "*", "y")],
                 "launch_ew<%s, 0>(stream, n, (const %s*)nullptr, (const %s*)nullptr, (const %s*)nullptr, y, OpFill<%s>{x})" % (T, T, T, T, T),
@@ -600,6 +613,9 @@ KNET8_API int knet8_version(void);
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
    key 2: small products with 16 to this many 32x32 output tiles and k >= 97 split k inside one workgroup per tile (default 256; 1: never) */
 KNET8_API int knet8_tune(int key, int value);
+/* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
+   src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */
+KNET8_API void knet8_seed(unsigned long long seed);
 /* replaces cublasSgemm_v2 / cublasDgemm_v2 at src/knetarrays/linalg.jl:26-52 (column-major, transa/transb in 'N','T'): hipBLASLt */
 KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc, hipStream_t stream);
 KNET8_API int gemm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc);

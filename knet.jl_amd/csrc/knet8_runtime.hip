@@ -10,6 +10,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <random>
 #include <string>
 #include <tuple>
 #include <unordered_map>
@@ -43,6 +44,24 @@ static bool ok(hipError_t e, const char* what) {
 }
 
 // ---- launch-heuristic knobs ------------------------------------------------------------------------------
+// Default random stream: seed and the next unused generator counter.  Unseeded, the seed comes from the operating system's
+// entropy source at first use, as the reference's generators start from a random seed until seed! is called.
+static std::mutex g_rng_mu;
+static unsigned long long g_rng_seed = 0, g_rng_offset = 0;
+static bool g_rng_seeded = false;
+void rng_take(unsigned long long blocks, unsigned long long* seed, unsigned long long* offset) {
+  std::lock_guard<std::mutex> lock(g_rng_mu);
+  if (!g_rng_seeded) {
+    std::random_device rd;
+    g_rng_seed = ((unsigned long long)rd() << 32) ^ (unsigned long long)rd();
+    g_rng_offset = 0;
+    g_rng_seeded = true;
+  }
+  *seed = g_rng_seed;
+  *offset = g_rng_offset;
+  g_rng_offset += blocks;
+}
+
 static int g_tune[kTuneCount] = {0, 0, 0, 0, 0, 0, 0, 0};
 int tuning(int key) {
   if (key < 0 || key >= kTuneCount) return 0;
@@ -400,6 +419,13 @@ KNET8_API const char* knet8_last_error(void) {
 }
 
 KNET8_API int knet8_version(void) { return 100; }
+
+KNET8_API void knet8_seed(unsigned long long seed) {
+  std::lock_guard<std::mutex> lock(g_rng_mu);
+  g_rng_seed = seed;
+  g_rng_offset = 0;
+  g_rng_seeded = true;
+}
 
 KNET8_API int knet8_tune(int key, int value) {
   if (key < 0 || key >= kTuneCount) return -1;

@@ -1,10 +1,10 @@
 """``dropout(x, p)`` and ``dropback`` (src/ops20/dropout.jl:15-42, src/ops20_gpu/dropout.jl:7-23).
 
-The reference fills ``y`` with uniforms from the device generator (``rand!(y)``) and calls ``dropout_S`` in place;
-CPU and GPU draw from different streams, which is why its own test only compares them statistically
-(test/dropout.jl:8-17).  Here the uniform buffer can be passed explicitly (``uniform=``) so that the device result
-can be compared element by element with the CPU path; without it the buffer is drawn from numpy's PCG64 with the
-given seed and uploaded.
+The reference fills ``y`` with uniforms from the device generator (``rand!(y)``, after ``CUDA.seed!(seed)`` for a
+non-zero ``seed``) and calls ``dropout_S`` in place; CPU and GPU draw from different streams, which is why its own test
+only compares them statistically (test/dropout.jl:8-17).  Here the buffer comes from the library's generator in the same
+way; it can also be passed explicitly (``uniform=``) so that the device result can be compared element by element with
+the CPU path.
 """
 import numpy as np
 
@@ -39,8 +39,10 @@ def dropback(dy, y, x, p):
 @primitive
 def _dropout(x, p, uniform=None, seed=0):
     if uniform is None:
-        rng = np.random.default_rng(seed if seed != 0 else None)
-        uniform = KnetArray(rng.random(x.length, dtype=x.dtype).reshape(x.dims, order="F"))
+        from .random import rand_, seed_
+        if seed != 0:
+            seed_(seed)       # if seed !== 0; CUDA.seed!(seed); end   (src/ops20_gpu/dropout.jl:13)
+        uniform = rand_(x.similar())
     elif not isinstance(uniform, KnetArray):
         uniform = KnetArray(np.asarray(uniform, dtype=x.dtype))
     else:

@@ -299,6 +299,75 @@ def addents(x, ents, y):
     return _shape_like(xf, x.shape)
 
 
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw, SC'11; the Random123 library's ``philox4x32``) in numpy integer arithmetic.
+
+    ``counter``: (n, 4) uint32 words c0..c3, ``key``: (k0, k1).  Returns the (n, 4) uint32 output blocks.  The reference draws
+    from cuRAND (src/knetarrays/random.jl:5-6), whose stream cannot be reproduced here: what this restates is the published
+    generator the device kernels use, pinned by Random123's known-answer vectors (tests/test_oracle_elementwise.py).
+    """
+    c = np.array(counter, dtype=np.uint64).reshape(-1, 4)
+    c0, c1, c2, c3 = (c[:, j].copy() for j in range(4))
+    k0, k1 = np.uint64(key[0]), np.uint64(key[1])
+    m0, m1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
+    w0, w1 = np.uint64(0x9E3779B9), np.uint64(0xBB67AE85)
+    lo32, sh = np.uint64(0xFFFFFFFF), np.uint64(32)
+    for _ in range(10):
+        p0, p1 = m0 * c0, m1 * c2                       # 32x32 -> 64-bit products, exact in uint64
+        c0, c1, c2, c3 = (p1 >> sh) ^ c1 ^ k0, p1 & lo32, (p0 >> sh) ^ c3 ^ k1, p0 & lo32
+        k0, k1 = (k0 + w0) & lo32, (k1 + w1) & lo32
+    return np.stack([c0, c1, c2, c3], axis=1).astype(np.uint32)
+
+
+def _philox_stream(nblocks, seed, offset):
+    ctr = (np.uint64(offset) + np.arange(nblocks, dtype=np.uint64))
+    c = np.zeros((nblocks, 4), dtype=np.uint64)
+    c[:, 0], c[:, 1] = ctr & np.uint64(0xFFFFFFFF), ctr >> np.uint64(32)
+    seed = int(seed)
+    return philox4x32_10(c, (seed & 0xFFFFFFFF, seed >> 32))
+
+
+def rand_uniform(n, seed, offset, dtype):
+    """What ``rand_seeded_S(n, seed, offset, y)`` writes: block ``offset + i // per`` of the stream keyed by ``seed``; fp32 takes
+    the top 24 bits of each of the four words, fp64 27 + 26 bits of a pair of words; both land in [0, 1)."""
+    dtype = np.dtype(dtype)
+    per = 4 if dtype == np.float32 else 2
+    w = _philox_stream((n + per - 1) // per, seed, offset)
+    if dtype == np.float32:
+        u = (w >> np.uint32(8)).astype(np.float32) * np.float32(2.0 ** -24)
+    else:
+        w = w.astype(np.uint64)
+        hi, lo = w[:, 0::2] >> np.uint64(5), w[:, 1::2] >> np.uint64(6)
+        u = (hi.astype(np.float64) * 2.0 ** 26 + lo.astype(np.float64)) * 2.0 ** -53
+    return u.reshape(-1)[:n]
+
+
+def rand_normal(n, seed, offset, dtype):
+    """What ``randn_seeded_S`` writes: Box-Muller on pairs of uniforms of the same blocks, the first moved to (0, 1]
+    (computed in fp64 here: the device's fp32 log/sin/cos may differ in the last places)."""
+    dtype = np.dtype(dtype)
+    per = 4 if dtype == np.float32 else 2
+    w = _philox_stream((n + per - 1) // per, seed, offset).astype(np.uint64)
+    if dtype == np.float32:
+        u1 = ((w[:, 0::2] >> np.uint64(8)) + np.uint64(1)).astype(np.float64) * 2.0 ** -24
+        u2 = (w[:, 1::2] >> np.uint64(8)).astype(np.float64) * 2.0 ** -24
+    else:
+        u = ((w[:, 0::2] >> np.uint64(5)).astype(np.float64) * 2.0 ** 26 + (w[:, 1::2] >> np.uint64(6)).astype(np.float64)) * 2.0 ** -53
+        u1, u2 = 1.0 - u[:, 0:1], u[:, 1:2]
+    r = np.sqrt(-2.0 * np.log(u1))
+    # cos and sin of pi*t, t = 2*u2 in [0, 2): split t = k/2 + f exactly with |f| <= 1/4, so that the rounding of pi*f cannot
+    # be amplified (forming 2*pi*u2 first would lose up to 8 ulp near t = 2)
+    t = 2.0 * u2
+    k = np.rint(2.0 * t)
+    f = t - 0.5 * k
+    cf, sf = np.cos(np.pi * f), np.sin(np.pi * f)
+    q = k.astype(np.int64) % 4
+    c = np.choose(q, [cf, -sf, -cf, sf])
+    sn = np.choose(q, [sf, cf, -sf, -cf])
+    z = np.stack([r * c, r * sn], axis=2)   # (blocks, pairs, 2)
+    return z.reshape(-1)[:n].astype(dtype)
+
+
 def dropout(x, p, u):
     """``dropout!``: ``u`` is the uniform buffer the reference draws with ``rand!``."""
     x = np.asarray(x)

@@ -209,3 +209,79 @@ def test_dropout_closed_form(oracle):
     assert oracle.dropout(np.float32([3.0]), 0.5, np.float32([0.5]))[0] == 0
     # expectation preserved
     assert abs(oracle.dropout(np.ones(200000, np.float32), 0.3, rng.random(200000, dtype=np.float32)).mean() - 1) < 0.01
+
+
+def test_philox_known_answers_and_uniform_mapping(oracle):
+    """The generator behind rand!/randn! is Philox4x32-10; the reference's own stream (cuRAND) cannot be reproduced, so the pin is
+    the published algorithm: the known-answer vectors of the Random123 library (kat_vectors: philox4x32 10) and the properties
+    of the word -> float mapping."""
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0), (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        assert [int(v) for v in oracle.philox4x32_10([ctr], key)[0]] == list(want)
+    # a brute-force scalar restatement with Python integers agrees with the vectorised one on arbitrary counters and keys
+    def scalar(c, k):
+        c, k = list(c), list(k)
+        for _ in range(10):
+            p0, p1 = 0xD2511F53 * c[0], 0xCD9E8D57 * c[2]
+            c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & 0xFFFFFFFF, (p0 >> 32) ^ c[3] ^ k[1], p0 & 0xFFFFFFFF]
+            k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
+        return c
+    rng = np.random.default_rng(5)
+    cs = rng.integers(0, 2 ** 32, size=(50, 4), dtype=np.uint64)
+    key = (int(rng.integers(0, 2 ** 32)), int(rng.integers(0, 2 ** 32)))
+    got = oracle.philox4x32_10(cs, key)
+    for i in range(50):
+        assert [int(v) for v in got[i]] == scalar([int(v) for v in cs[i]], key)
+    # stream layout: element i comes from block offset + i // per, whatever the length of the call
+    for dt, per in ((np.float32, 4), (np.float64, 2)):
+        a = oracle.rand_uniform(1001, 12345, 7, dt)
+        assert a.dtype == dt and a.shape == (1001,)
+        assert np.array_equal(a[:40], oracle.rand_uniform(40, 12345, 7, dt))
+        assert np.array_equal(a[per * 5:per * 5 + 8], oracle.rand_uniform(8, 12345, 12, dt))
+        assert a.min() >= 0 and a.max() < 1
+    # seed 0, offset 0, fp32: the top 24 bits of the first known-answer block
+    assert np.array_equal(oracle.rand_uniform(4, 0, 0, np.float32), (np.array(kat[0][2], dtype=np.uint32) >> 8).astype(np.float32) * np.float32(2.0 ** -24))
+    # extremes of the mapping: all-ones words stay below 1, zero words give 0
+    assert (0xffffffff >> 8) * 2.0 ** -24 < 1 and ((0xffffffff >> 5) * 2.0 ** 26 + (0xffffffff >> 6)) * 2.0 ** -53 < 1
+
+
+def test_random_streams_have_the_right_moments(oracle):
+    n = 400000
+    for dt in (np.float32, np.float64):
+        u = oracle.rand_uniform(n, 99, 0, dt).astype(np.float64)
+        assert abs(u.mean() - 0.5) < 4 * np.sqrt(1 / 12 / n) and abs(u.var() - 1 / 12) < 1e-3
+        counts = np.histogram(u, bins=64, range=(0, 1))[0]
+        chi2 = ((counts - n / 64) ** 2 / (n / 64)).sum()
+        assert chi2 < 63 + 5 * np.sqrt(2 * 63)          # chi-square with 63 degrees of freedom, five sigma
+        assert abs(np.corrcoef(u[:-1], u[1:])[0, 1]) < 5 / np.sqrt(n)
+        z = oracle.rand_normal(n, 99, 0, dt).astype(np.float64)
+        assert np.all(np.isfinite(z))
+        assert abs(z.mean()) < 4 / np.sqrt(n) and abs(z.var() - 1) < 0.01
+        assert abs((z ** 3).mean()) < 0.03 and abs((z ** 4).mean() - 3) < 0.06
+        assert abs(np.corrcoef(z[0::2], z[1::2])[0, 1]) < 5 / np.sqrt(n / 2)   # the cos and sin halves of a pair
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_normal_variates_are_the_box_muller_transform_of_the_uniform_blocks(oracle, dt):
+    import mpmath as mp
+    mp.mp.prec = 120
+    n = 800
+    z = oracle.rand_normal(n, 11, 5, dt).astype(np.float64)
+    per = 4 if dt == np.float32 else 2
+    words = oracle._philox_stream(n // per, 11, 5)
+    want = []
+    for w in words:
+        w = [int(v) for v in w]
+        if dt == np.float32:
+            pairs = [(mp.mpf((w[0] >> 8) + 1) / 2 ** 24, mp.mpf(w[1] >> 8) / 2 ** 24), (mp.mpf((w[2] >> 8) + 1) / 2 ** 24, mp.mpf(w[3] >> 8) / 2 ** 24)]
+        else:
+            u = [mp.mpf((w[0] >> 5) * 2 ** 26 + (w[1] >> 6)) / 2 ** 53, mp.mpf((w[2] >> 5) * 2 ** 26 + (w[3] >> 6)) / 2 ** 53]
+            pairs = [(1 - u[0], u[1])]
+        for u1, u2 in pairs:
+            r = mp.sqrt(-2 * mp.log(u1))
+            want += [float(r * mp.cos(2 * mp.pi * u2)), float(r * mp.sin(2 * mp.pi * u2))]
+    want = np.array(want)
+    err = np.abs(z - want) / np.spacing(np.maximum(np.abs(want), 1.0).astype(dt)).astype(np.float64)
+    assert err.max() <= 2.5
