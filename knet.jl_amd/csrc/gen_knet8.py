@@ -371,6 +371,10 @@ def gen_elementwise():
                          "  launch_rand<%s, %s>(stream, n, seed, offset, y);\n  knet8::check_launch(\"%s_%s\");" % (T, T, normal, name, S))
             o.entry("%s_seeded_%s" % (name, S), "void", [("int", "n"), ("unsigned long long", "seed"), ("unsigned long long", "offset"), (T + "*", "y")],
                     "launch_rand<%s, %s>(stream, n, seed, offset, y)" % (T, normal), "src/knetarrays/random.jl:5-6 with the generator state passed in")
+            o.entry("%s_state_%s" % (name, S), "void", [("int", "n"), ("unsigned long long*", "state"), (T + "*", "y")],
+                    "launch_rand_state<%s, %s>(stream, n, state, y)" % (T, normal),
+                    "src/knetarrays/random.jl:5-6 with the generator state {seed, next counter} in device memory: read by the launch and\n"
+                    "   moved forward by a second one-lane launch, so a captured graph draws fresh numbers on every replay")
     for T, S in TYPES:
         o.entry("fill_%s" % S, "void", [("int", "n"), (T, "x"), (T + "*", "y")],
                 "launch_ew<%s, 0>(stream, n, (const %s*)nullptr, (const %s*)nullptr, (const %s*)nullptr, y, OpFill<%s>{x})" % (T, T, T, T, T),

@@ -98,6 +98,34 @@ __global__ __launch_bounds__(256) void rand_kernel(long n, unsigned long long se
   }
 }
 
+// Generator position kept in device memory: state[0] = seed, state[1] = next unused counter.  A launch that reads its position
+// from there and a one-lane launch that moves it forward can be captured into a hipGraph: every replay draws fresh numbers,
+// which kernel arguments frozen at capture time cannot give.
+template <typename T, bool NORMAL>
+__global__ __launch_bounds__(256) void rand_state_kernel(long n, const unsigned long long* __restrict__ state, T* __restrict__ y, bool vec) {
+  constexpr int N = RandConv<T>::kPerBlock;
+  typedef typename Vec16<T>::type V;
+  const long blk = (long)blockIdx.x * 256 + threadIdx.x;
+  const long i0 = blk * N;
+  if (i0 >= n) return;
+  const Philox4 b = philox4x32_10(state[1] + (unsigned long long)blk, state[0]);
+  T o[N];
+  if (NORMAL) RandConv<T>::normal(b, o); else RandConv<T>::uniform(b, o);
+  if (vec && i0 + N <= n) {
+    V v;
+#pragma unroll
+    for (int j = 0; j < N; j++) v[j] = o[j];
+    st_stream(reinterpret_cast<V*>(y + i0), v);
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; j++)
+      if (i0 + j < n) y[i0 + j] = o[j];
+  }
+}
+static __global__ void rand_state_advance_kernel(unsigned long long* state, unsigned long long blocks) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) state[1] += blocks;
+}
+
 // Counters a call of n elements consumes.
 template <typename T> inline unsigned long long rand_blocks(long n) {
   constexpr int N = RandConv<T>::kPerBlock;
@@ -111,6 +139,17 @@ inline void launch_rand(hipStream_t stream, long n, unsigned long long seed, uns
   const unsigned long long grid = (blocks + 255) / 256;
   if (grid > 0x7fffffffull) { record_error("rand: too many elements"); return; }
   hipLaunchKernelGGL((rand_kernel<T, NORMAL>), dim3((unsigned)grid), dim3(256), 0, stream, n, seed, offset, y, aligned16(y));
+}
+
+template <typename T, bool NORMAL>
+inline void launch_rand_state(hipStream_t stream, long n, unsigned long long* state, T* y) {
+  if (n <= 0) return;
+  if (state == nullptr) { record_error("rand_state: null state"); return; }
+  const unsigned long long blocks = rand_blocks<T>(n);
+  const unsigned long long grid = (blocks + 255) / 256;
+  if (grid > 0x7fffffffull) { record_error("rand: too many elements"); return; }
+  hipLaunchKernelGGL((rand_state_kernel<T, NORMAL>), dim3((unsigned)grid), dim3(256), 0, stream, n, state, y, aligned16(y));
+  hipLaunchKernelGGL(rand_state_advance_kernel, dim3(1), dim3(64), 0, stream, state, blocks);
 }
 
 }  // namespace knet8

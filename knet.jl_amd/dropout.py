@@ -37,12 +37,15 @@ def dropback(dy, y, x, p):
 
 
 @primitive
-def _dropout(x, p, uniform=None, seed=0):
+def _dropout(x, p, uniform=None, seed=0, rng=None):
     if uniform is None:
         from .random import rand_, seed_
-        if seed != 0:
-            seed_(seed)       # if seed !== 0; CUDA.seed!(seed); end   (src/ops20_gpu/dropout.jl:13)
-        uniform = rand_(x.similar())
+        if rng is not None:
+            uniform = rand_(x.similar(), state=rng)   # position on the device: safe to capture into a graph
+        else:
+            if seed != 0:
+                seed_(seed)   # if seed !== 0; CUDA.seed!(seed); end   (src/ops20_gpu/dropout.jl:13)
+            uniform = rand_(x.similar())
     elif not isinstance(uniform, KnetArray):
         uniform = KnetArray(np.asarray(uniform, dtype=x.dtype))
     else:
@@ -51,15 +54,16 @@ def _dropout(x, p, uniform=None, seed=0):
     return y, (lambda dy: (dropback(dy, y, x, p), None))
 
 
-def dropout(x, p, seed=0, drop=None, uniform=None):
-    """``dropout(x, p; seed, drop)``: identity unless recording (or ``drop=True``), as in the reference."""
+def dropout(x, p, seed=0, drop=None, uniform=None, rng=None):
+    """``dropout(x, p; seed, drop)``: identity unless recording (or ``drop=True``), as in the reference.  ``uniform`` passes the
+    mask buffer explicitly; ``rng`` (an ``RngState``) draws it from a generator position kept on the device."""
     from .autograd import value
     if drop is None:
         drop = recording()
     if not drop:
         return x
     if 0 < p < 1:
-        return _dropout(x, p, uniform=uniform, seed=seed)
+        return _dropout(x, p, uniform=uniform, seed=seed, rng=rng)
     if p == 0:
         return x
     if p == 1:

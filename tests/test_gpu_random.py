@@ -97,3 +97,46 @@ def test_dropout_draws_its_own_mask_as_the_reference_tests_it(knet, oracle):
     want = np.where(oracle.dropout(x, 0.25, u7) != 0, np.float32(1) / np.float32(0.75), np.float32(0))
     assert bits_equal(g, want.astype(np.float32))
     knet.libknet8().check()
+
+
+def test_generator_state_on_the_device_advances_across_graph_replays(knet, oracle):
+    """A captured step with dropout must draw a fresh mask on every replay: the position {seed, next counter} lives in device
+    memory, is read by the generating launch and moved forward by a second launch, both inside the graph."""
+    lib = knet.libknet8()
+    old_stream = lib.stream
+    try:
+        rng = np.random.default_rng(3)
+        x = rng.standard_normal((257, 33)).astype(np.float32)    # 8481 values: 2121 blocks, the last one partial
+        xd = knet.KnetArray(x)
+        state = knet.RngState(seed=77)
+        # eager: two draws continue the stream
+        a = knet.Array(knet.rand_(knet.KnetArray(dtype=np.float32, dims=(10,)), state=state))
+        b = knet.Array(knet.rand_(knet.KnetArray(dtype=np.float64, dims=(3,)), state=state))
+        assert bits_equal(a, oracle.rand_uniform(10, 77, 0, np.float32)) and bits_equal(b, oracle.rand_uniform(3, 77, 3, np.float64))
+        assert state.get() == (77, 5)
+        state.set(77, 0)
+        blocks = (x.size + 3) // 4
+
+        def step():
+            y = knet.dropout(xd, 0.5, drop=True, rng=state)
+            return [y, knet.sum(y, dims=1)]
+        g = knet.capture(step)                       # one eager warm-up run + the capture: the stream stands at 1 * blocks
+        assert state.get() == (77, blocks)
+        for r in range(4):
+            g.replay()
+            knet.synchronize()
+            y = knet.Array(g.outputs[0])
+            u = oracle.rand_uniform(x.size, 77, (1 + r) * blocks, np.float32).reshape(x.shape, order="F")
+            assert bits_equal(y, oracle.dropout(x, 0.5, u)), r
+            assert np.allclose(knet.Array(g.outputs[1]), y.sum(axis=0, keepdims=True), rtol=1e-5, atol=1e-5)
+            # eager draws from the same state between replays take their place in the stream too
+            e = knet.Array(knet.rand_(knet.KnetArray(dtype=np.float32, dims=(4,)), state=state))
+            assert bits_equal(e, oracle.rand_uniform(4, 77, (2 + r) * blocks, np.float32))
+            state.set(77, (2 + r) * blocks)           # put the position back for the arithmetic of the next round
+        del g
+        knet.knet8("rand_state_32", 4, 0, xd.ptr)     # a null state is recorded as an error, nothing is launched
+        with pytest.raises(RuntimeError):
+            lib.check()
+        lib.check()
+    finally:
+        lib.stream = old_stream
