@@ -22,6 +22,6 @@ from .loss import nll, findindices, accuracy, getindex, ungetindex, bce, logisti
 from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat)
 from .dropout import dropout, dropback, dropout_, dropback_
 from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
-from .linalg import dense, matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose
+from .linalg import dense, matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
 
 libknet8()  # fail loudly at import time if the HIP library is missing

@@ -236,6 +236,7 @@ PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_softmax.h"
 #include "../knet8_index.h"
 #include "../knet8_transpose.h"
+#include "../knet8_permute.h"
 using namespace knet8;
 
 """
@@ -518,6 +519,12 @@ def gen_softmax():
         o.entry("permute213_%s" % S, "void", [("int", "m"), ("int", "n"), ("int", "batch"), (T + "*", "x"), (T + "*", "y")],
                 "launch_transpose<%s>(stream, m, n, x, y, batch)" % T,
                 "permutedims(x, (2,1,3)) of an (m, n, batch) array (CUDA.jl's permutedims in the reference, src/knetarrays/reshape.jl:18)")
+    o.decl.append("/* permutedims_S: y = permutedims(x, perm) for an array of `ndims` (1 to 8) dimensions.  `dims` (sizes of x) and `perm`\n"
+                  "   (1-based, as in Julia) are HOST arrays read during the call; x and y are device arrays of prod(dims) elements.\n"
+                  "   Replaces permutedims!(CuArray(y), CuArray(x), perm) of CUDA.jl at src/knetarrays/reshape.jl:18-29. */")
+    for T, S in TYPES:
+        o.entry("permutedims_%s" % S, "void", [("int", "ndims"), ("const int*", "dims"), ("const int*", "perm"), (T + "*", "x"), (T + "*", "y")],
+                "launch_permutedims<%s>(stream, ndims, dims, perm, x, y)" % T, "src/knetarrays/reshape.jl:18-29")
     o.decl.append("\n/* ---- gather / scatter on 1-based int32 linear indices -- src/libknet8/cuda1.jl:342-362 ---- */")
     for T, S in TYPES:
         o.entry("getents_%s" % S, "void", [("int", "n"), ("int*", "ents"), (T + "*", "x"), (T + "*", "y")],

@@ -125,3 +125,35 @@ def transpose(x):
     if x.ndims > 2:
         raise ValueError("transpose needs a vector or a matrix")
     return _transpose(x), (lambda dy: (_transpose(dy),))
+
+
+def _permutedims(x, perm):
+    perm = [int(p) for p in perm]
+    nd = x.ndims
+    if len(perm) != nd or sorted(perm) != list(range(1, nd + 1)):
+        raise ValueError("ArgumentError: no valid permutation of dimensions")   # src/knetarrays/reshape.jl:24
+    if nd > 8:
+        raise ValueError("permutedims: at most 8 dimensions")
+    y = x.similar(tuple(x.dims[p - 1] for p in perm))
+    if y.length:
+        import ctypes
+        dims_h = (ctypes.c_int * nd)(*x.dims)
+        perm_h = (ctypes.c_int * nd)(*perm)
+        knet8("permutedims_%s" % x.suffix, nd, ctypes.cast(dims_h, ctypes.c_void_p), ctypes.cast(perm_h, ctypes.c_void_p), x.ptr, y.ptr)
+    return y
+
+
+@primitive
+def permutedims(x, perm=None):
+    """``permutedims(x, perm)`` with 1-based ``perm`` (src/knetarrays/reshape.jl:21-29) -> ``permutedims_S``; for a matrix or vector
+    without ``perm`` the transpose (``:31-33``).  The gradient permutes the incoming gradient back (``invperm``)."""
+    if perm is None:
+        if x.ndims > 2:
+            raise ValueError("permutedims needs perm for more than 2 dimensions")
+        return _transpose(x), (lambda dy: (_transpose(dy).reshape(x.dims),))
+    perm = [int(p) for p in perm]
+    y = _permutedims(x, perm)
+    inv = [0] * len(perm)
+    for i, p in enumerate(perm):
+        inv[p - 1] = i + 1
+    return y, (lambda dy: (_permutedims(dy, inv), None))
