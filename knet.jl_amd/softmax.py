@@ -3,8 +3,9 @@
 Mirrors src/ops20_gpu/softmax.jl:10-59.  There ``dims=:`` or ``dims=1`` reshape to ``(1,1,m,n)`` and call
 cuDNN (``_cudnnSoftmaxForward`` LOG / ACCURATE, backward ``_cudnnSoftmaxBackward``); here the same cases
 call ``logsoftmax_S / softmax_S`` and ``logsoftmaxback_S / softmaxback_S`` of libknet8.  2-d ``dims=2`` goes
-through a transpose as in the reference (``:19-20``); other ``dims`` use the generic formulation
-(src/ops20/softmax.jl:42-74) built from reductions and broadcasts.
+through a transpose as in the reference (``:19-20``), batched over trailing dims; any other ``dims`` go through one N-d
+permutation that brings the reduced dimensions to the front (the reference uses the broadcast/reduction chain of
+src/ops20/softmax.jl:42-74 there).
 """
 from .autograd import primitive
 from .karray import KnetArray
@@ -109,23 +110,28 @@ def _make(kernel, backkernel):
                 knet8("%s_strided_%s" % (backkernel, y.suffix), inner, d, outer, y.ptr, dy.ptr, dx.ptr)
                 return (dx,)
             return y, back
-        # dims that are not adjacent (e.g. (1,3) of a 3-d array, test/loss.jl:46): the generic formulation of
-        # src/ops20/softmax.jl:42-63 from reductions and broadcasts
-        from .activation import unary_op
-        from .binary import broadcast_op as bc
+        # dims that are not adjacent (e.g. (1,3) of a 3-d array, test/loss.jl:46): bring the reduced dims to the front with one
+        # N-d permutation, run the column kernels, permute back (the reference falls back to the broadcast/reduction chain of
+        # src/ops20/softmax.jl:42-63 here: six or more passes over the array instead of three)
+        from .linalg import _permutedims
         d = sorted(set(int(i) for i in dims))
-        x1 = bc("sub", x, R.reduce_op("maximum", x, d))
-        e = unary_op("exp", x1)
-        ssum = R.reduce_op("sum", e, d)
-        if kernel == "logsoftmax":
-            y = bc("sub", x1, unary_op("log", ssum))
-            return y, (lambda dy: (bc("sub", dy, bc("mul", unary_op("exp", y), R.reduce_op("sum", dy, d))),))
-        y = bc("div", e, ssum)
+        if any(i < 1 or i > x.ndims for i in d):
+            raise ValueError("softmax: dims out of range: %r" % (dims,))
+        perm = d + [i for i in range(1, x.ndims + 1) if i not in d]
+        inv = [0] * len(perm)
+        for i, p in enumerate(perm):
+            inv[p - 1] = i + 1
+        m = 1
+        for i in d:
+            m *= x.size(i)
+        n = x.length // m
+        yt = _fwd(kernel, _permutedims(x, perm), m, n)
+        y = _permutedims(yt, inv)
 
-        def back_generic(dy):
-            yd = bc("mul", y, dy)
-            return (bc("sub", yd, bc("mul", y, R.reduce_op("sum", yd, d))),)
-        return y, back_generic
+        def back_p(dy):
+            dxt = _bwd(backkernel, yt, _permutedims(dy, perm), m, n)
+            return (_permutedims(dxt.reshape(yt.dims), inv),)
+        return y, back_p
 
     f.__name__ = kernel
     return f
