@@ -160,13 +160,29 @@ def logsumexp(x, dims=None):
 
     Built on the column kernels: logsumexp = x - logsoftmax(x) at any position of the reduced slice, and
     exp.(x .- y) is softmax(x)."""
-    mn = _columns(x, dims)
-    if mn is None:
-        raise NotImplementedError("logsumexp over dims=%r" % (dims,))
-    m, n = mn
-    y = _fwd("logsoftmax", x, m, n)
     from .binary import broadcast_op
-    diff = broadcast_op("sub", x, y)  # every row of a column holds the same value: take the maximum to pick one
+    from .linalg import _permutedims
+    mn = _columns(x, dims)
+    perm = inv = None
+    xp = x
+    if mn is None:
+        # reduced dims that are not the leading ones: one permutation brings them to the front (kept dims keep their order, so
+        # the vector of results reshapes straight into the output)
+        d = sorted(set([dims] if isinstance(dims, int) else [int(i) for i in dims]))
+        if any(i < 1 or i > x.ndims for i in d):
+            raise ValueError("logsumexp: dims out of range: %r" % (dims,))
+        perm = d + [i for i in range(1, x.ndims + 1) if i not in d]
+        inv = [0] * len(perm)
+        for i, q in enumerate(perm):
+            inv[q - 1] = i + 1
+        xp = _permutedims(x, perm)
+        m = 1
+        for i in d:
+            m *= x.size(i)
+        mn = (m, x.length // m)
+    m, n = mn
+    y = _fwd("logsoftmax", xp, m, n)
+    diff = broadcast_op("sub", xp, y)  # every row of a column holds the same value: take the maximum to pick one
     out = R.reduce_op("maximum", diff.reshape(m, n), 1)
     if dims is None:
         res = out.to_numpy().ravel()[0]
@@ -175,9 +191,11 @@ def logsumexp(x, dims=None):
         res = out.reshape(tuple(1 if (i + 1) in d else x.dims[i] for i in range(x.ndims)))
 
     def back(dy):
-        sm = _fwd("softmax", x, m, n)
+        sm = _fwd("softmax", xp, m, n)
         if isinstance(dy, KnetArray):
             g = broadcast_op("mul", sm.reshape(m, n), dy.reshape(1, n)) if n > 1 else broadcast_op("mul", float(dy.to_numpy().ravel()[0]), sm)
-            return (g.reshape(x.dims),)
-        return (broadcast_op("mul", dy, sm),)
+            g = g.reshape(xp.dims)
+        else:
+            g = broadcast_op("mul", dy, sm)
+        return (_permutedims(g, inv) if inv is not None else g.reshape(x.dims),)
     return res, back

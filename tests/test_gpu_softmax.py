@@ -226,6 +226,27 @@ def test_logsumexp_value_and_gradient(knet, oracle):
         assert close(knet.Array(knet.grad(J, p)), wantg, 2e-5), (shape, dims)
 
 
+def test_logsumexp_over_any_dims(knet):
+    """Reduced dims that are not the leading ones (src/ops20/softmax.jl:65-74 accepts any dims): against the formula in fp64."""
+    rng = np.random.default_rng(39)
+    for shape, dims in [((5, 7), 2), ((3, 4, 5), 2), ((3, 4, 5), 3), ((3, 4, 5), [1, 3]), ((6, 5, 4, 3), [2, 4]), ((40, 300), 2)]:
+        x = (rng.standard_normal(shape) * 2).astype(np.float32)
+        ax = tuple(i - 1 for i in ([dims] if isinstance(dims, int) else dims))
+        x64 = x.astype(np.float64)
+        mx = x64.max(axis=ax, keepdims=True)
+        want = np.log(np.exp(x64 - mx).sum(axis=ax, keepdims=True)) + mx
+        got = knet.Array(knet.logsumexp(knet.KnetArray(x), dims=dims))
+        assert got.shape == want.shape and np.allclose(got, want, rtol=1e-5, atol=1e-5), (shape, dims)
+        dy = rng.standard_normal(want.shape).astype(np.float32)
+        p = knet.Param(knet.KnetArray(x))
+        J = knet.diff(lambda: knet.sum(knet.mul(knet.logsumexp(p, dims=dims), knet.KnetArray(dy))))
+        wantg = dy * np.exp(x64 - want)
+        assert close(knet.Array(knet.grad(J, p)), wantg, 2e-5), (shape, dims)
+    with pytest.raises(ValueError):
+        knet.logsumexp(knet.KnetArray(np.zeros((3, 4), np.float32)), dims=3)
+    knet.libknet8().check()
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_streaming_kernel_on_short_columns_and_masked_logits(knet, oracle, dt):
     """The two-pass streaming kernel (normally only for columns beyond the register capacity) is forced on short columns through
