@@ -71,9 +71,18 @@ def _nll_fused(scores, labels, dims=1, count=None):
     ``labels`` may be a host integer array (checked and uploaded, loss returned as a host scalar, as the reference's nll does) or
     an Int32 ``KnetArray`` already on the device together with ``count`` = number of non-zero labels; in that case nothing
     synchronises with the host and the loss comes back as a 1-element ``KnetArray`` (what a captured graph needs)."""
-    if dims != 1 or scores.ndims != 2:
-        raise NotImplementedError("fused nll needs a (classes, instances) matrix and dims=1")
-    m, n = scores.dims
+    transposed = False
+    orig = scores
+    if dims == 1:          # classes down the first dimension, every other dimension counts instances (findindices, loss.jl:120-127)
+        m = scores.size(1)
+        n = scores.length // m if m else 0
+    elif dims == 2 and scores.ndims == 2:   # instances down the first dimension: through the transpose, as logsoftmax(dims=2) goes
+        from .linalg import _transpose
+        n, m = scores.dims
+        scores = _transpose(scores)
+        transposed = True
+    else:
+        raise ValueError("fused nll supports dims=1, or dims=2 for a matrix")
     T = scores.dtype.type
     on_device = isinstance(labels, KnetArray)
     if on_device:
@@ -100,6 +109,12 @@ def _nll_fused(scores, labels, dims=1, count=None):
     else:
         total = R.reduce_op("sum", lossv)
         loss = T(total) / T(count)
+
+    if transposed:
+        from .linalg import _transpose
+        dx = _transpose(dx.reshape(m, n))
+    else:
+        dx = dx.reshape(orig.dims)
 
     def back(dy):
         from .linalg import scal

@@ -136,6 +136,25 @@ def test_nll_known_answer_and_dims2(knet, oracle):
     assert knet.accuracy(knet.KnetArray(scores), [1, 2]) == 1.0 and knet.accuracy(knet.KnetArray(scores), [2, 2]) == 0.5
     with pytest.raises(ValueError):
         knet.nll(knet.KnetArray(scores), [1, 2, 3])
+    # the fused kernel on the same layouts: instances along the first dimension (dims=2, through a transpose), and an N-d score
+    # array with the classes first (findindices flattens the other dimensions, src/ops20/loss.jl:120-127)
+    rng = np.random.default_rng(40)
+    sc = (rng.standard_normal((37, 11)) * 2).astype(np.float32)
+    lab = rng.integers(0, 12, size=37)
+    p = knet.Param(knet.KnetArray(sc))
+    J = knet.diff(lambda: knet.nll(p, lab, dims=2, fused=True))
+    assert abs(float(J.value) - float(oracle.nll(sc, lab, dims=2))) <= 1e-5 * abs(float(oracle.nll(sc, lab, dims=2)))
+    assert close(knet.Array(knet.grad(J, p)), oracle.nll_back(sc, lab, dims=2), 1e-5)
+    sc3 = (rng.standard_normal((9, 5, 7)) * 2).astype(np.float32)
+    lab3 = rng.integers(0, 10, size=(5, 7))
+    p = knet.Param(knet.KnetArray(sc3))
+    J = knet.diff(lambda: knet.nll(p, lab3, fused=True))
+    flat, lf = sc3.reshape(9, 35, order="F"), lab3.reshape(-1, order="F")
+    assert abs(float(J.value) - float(oracle.nll(flat, lf))) <= 1e-5 * abs(float(oracle.nll(flat, lf)))
+    g = knet.Array(knet.grad(J, p))
+    assert g.shape == sc3.shape and close(g.reshape(9, 35, order="F"), oracle.nll_back(flat, lf), 1e-5)
+    with pytest.raises(ValueError):
+        knet.nll(knet.KnetArray(sc3), lab3, dims=2, fused=True)
 
 
 def test_config4_full_size(knet, oracle):
