@@ -40,8 +40,10 @@ inline bool perm_plan(int nd, const int* dims, const int* perm, PermPlan& p, lon
     if (dims[i] < 0) { why = "permutedims: negative dimension"; return false; }
   }
   total = 1;
-  for (int i = 0; i < nd; i++) total *= dims[i];
-  if (total >= (1L << 31)) { why = "permutedims: more than 2^31-1 elements"; return false; }
+  for (int i = 0; i < nd; i++) {
+    total *= dims[i];
+    if (total >= (1L << 31)) { why = "permutedims: more than 2^31-1 elements"; return false; }   // checked as it grows: no overflow
+  }
   long sxl[kPermMaxDims], syl[kPermMaxDims], ys = 1, xs = 1;
   for (int k = 0; k < nd; k++) { sxl[k] = xs; xs *= dims[k]; }
   for (int i = 0; i < nd; i++) { syl[perm[i] - 1] = ys; ys *= dims[perm[i] - 1]; }
