@@ -486,11 +486,187 @@ __global__ __launch_bounds__(256) void softmax_strided_kernel(long inner, long d
     out[base + k * inner] = Algo::out(a[base + k * inner], Algo::kInputs == 2 ? b[base + k * inner] : T(0), mx, fin);
 }
 
+// The same for large arrays, in two launches.  A workgroup owns a panel: TI = 64*NV neighbouring `inner` positions (a wave reads
+// 64*NV*sizeof(T) contiguous bytes per row) times a chunk of d, its four waves taking every fourth row.
+//   reduce: every lane folds its rows into a running (max, sum of exp) pair per position (or a plain sum for the gradients),
+//           the waves are merged in LDS and the panel's pairs go to scratch: partial[outer][chunk][max|sum][inner];
+//   apply:  a workgroup merges the pairs of all chunks of its positions, then walks its panel again and writes the result.
+// Each input is read twice (the second time mostly from the memory-side cache), the output written once; the permutation
+// route (permute, column kernel, permute back) moves every array three times as often.
+constexpr int kPanelWaves = 4, kPanelU = 4, kPanelMaxChunks = 64;
+
+template <typename T, int NV>
+__device__ __forceinline__ void panel_load(const T* p, T (&v)[NV]) {
+  if (NV > 1) {
+    typedef typename Vec16<T>::type V;
+    const V t = *reinterpret_cast<const V*>(p);   // kept cacheable: the apply pass reads the same lines again
+#pragma unroll
+    for (int e = 0; e < NV; e++) v[e] = t[e];
+  } else {
+    v[0] = *p;
+  }
+}
+
+template <typename T, typename Algo, int NV>
+__global__ __launch_bounds__(kPanelWaves * kWave) void softmax_panel_reduce_kernel(long inner, long d, long itiles, long nchunks, long dchunk, long ipad,
+                                                                                   const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ partial) {
+  constexpr int TI = kWave * NV, NW = kPanelWaves, U = kPanelU;
+  constexpr bool kTwo = Algo::kInputs == 2;
+  __shared__ T lds_m[NW][TI], lds_s[NW][TI];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  long blk = blockIdx.x;
+  const long it = blk % itiles; blk /= itiles;
+  const long c = blk % nchunks;
+  const long o = blk / nchunks;
+  const long a0 = it * TI + (long)lane * NV;
+  const bool live = a0 < inner;             // vector path: inner % NV == 0, a vector is inside or outside as a whole
+  const long base = o * d * inner + a0;
+  const long k0 = c * dchunk;
+  long k1 = k0 + dchunk;
+  if (k1 > d) k1 = d;
+  const T ninf = T(-INFINITY);
+  T m[NV], sum[NV];
+#pragma unroll
+  for (int e = 0; e < NV; e++) { m[e] = Algo::kNeedMax ? ninf : T(0); sum[e] = T(0); }
+  if (live) {
+    for (long k = k0 + wave; k < k1; k += NW * U) {
+      T va[U][NV], vb[U][NV];
+#pragma unroll
+      for (int q = 0; q < U; q++) {
+        const long kk = k + q * NW;
+        if (kk < k1) {
+          panel_load<T, NV>(a + base + kk * inner, va[q]);
+          if (kTwo) panel_load<T, NV>(b + base + kk * inner, vb[q]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < NV; e++) { va[q][e] = Algo::kNeedMax ? ninf : T(0); vb[q][e] = T(0); }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        if (Algo::kNeedMax) {
+          T bm = m[e];
+#pragma unroll
+          for (int q = 0; q < U; q++) bm = va[q][e] > bm ? va[q][e] : bm;
+          if (bm > m[e]) { sum[e] = sum[e] * dev_exp(m[e] - bm); m[e] = bm; }
+#pragma unroll
+          for (int q = 0; q < U; q++) sum[e] = sum[e] + (va[q][e] == ninf ? T(0) : dev_exp(va[q][e] - m[e]));
+        } else {
+#pragma unroll
+          for (int q = 0; q < U; q++) sum[e] = sum[e] + Algo::term(va[q][e], kTwo ? vb[q][e] : T(0), T(0));
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < NV; e++) { lds_m[wave][lane * NV + e] = m[e]; lds_s[wave][lane * NV + e] = sum[e]; }
+  __syncthreads();
+  if (threadIdx.x < TI) {
+    T mm = lds_m[0][threadIdx.x], ss = lds_s[0][threadIdx.x];
+#pragma unroll
+    for (int w = 1; w < NW; w++) {
+      if (Algo::kNeedMax) maxsum_merge(mm, ss, lds_m[w][threadIdx.x], lds_s[w][threadIdx.x]);
+      else ss = ss + lds_s[w][threadIdx.x];
+    }
+    T* row = partial + ((o * nchunks + c) * 2) * ipad + it * TI + threadIdx.x;
+    row[0] = mm;
+    row[ipad] = ss;
+  }
+}
+
+template <typename T, typename Algo, int NV>
+__global__ __launch_bounds__(kPanelWaves * kWave) void softmax_panel_apply_kernel(long inner, long d, long itiles, long nchunks, long dchunk, long ipad,
+                                                                                  const T* __restrict__ a, const T* __restrict__ b, const T* __restrict__ partial,
+                                                                                  T* __restrict__ out) {
+  constexpr int TI = kWave * NV, NW = kPanelWaves, U = kPanelU;
+  constexpr bool kTwo = Algo::kInputs == 2;
+  typedef typename Vec16<T>::type V;
+  __shared__ T lds_m[TI], lds_f[TI];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  long blk = blockIdx.x;
+  const long it = blk % itiles; blk /= itiles;
+  const long c = blk % nchunks;
+  const long o = blk / nchunks;
+  if (threadIdx.x < TI) {
+    const T* row = partial + (o * nchunks * 2) * ipad + it * TI + threadIdx.x;
+    T mm = row[0], ss = row[ipad];
+    for (long cc = 1; cc < nchunks; cc++) {
+      const T m2 = row[cc * 2 * ipad], s2 = row[(cc * 2 + 1) * ipad];
+      if (Algo::kNeedMax) maxsum_merge(mm, ss, m2, s2);
+      else ss = ss + s2;
+    }
+    lds_m[threadIdx.x] = mm;
+    lds_f[threadIdx.x] = Algo::finish(ss);
+  }
+  __syncthreads();
+  const long a0 = it * TI + (long)lane * NV;
+  if (a0 >= inner) return;
+  T mx[NV], fin[NV];
+#pragma unroll
+  for (int e = 0; e < NV; e++) { mx[e] = lds_m[lane * NV + e]; fin[e] = lds_f[lane * NV + e]; }
+  const long base = o * d * inner + a0;
+  const long k0 = c * dchunk;
+  long k1 = k0 + dchunk;
+  if (k1 > d) k1 = d;
+  for (long k = k0 + wave; k < k1; k += NW * U) {
+    T va[U][NV], vb[U][NV];
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long kk = k + q * NW;
+      if (kk < k1) {
+        panel_load<T, NV>(a + base + kk * inner, va[q]);
+        if (kTwo) panel_load<T, NV>(b + base + kk * inner, vb[q]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < U; q++) {
+      const long kk = k + q * NW;
+      if (kk < k1) {
+        if (NV > 1) {
+          V vo;
+#pragma unroll
+          for (int e = 0; e < NV; e++) vo[e] = Algo::out(va[q][e], kTwo ? vb[q][e] : T(0), mx[e], fin[e]);
+          st_stream(reinterpret_cast<V*>(out + base + kk * inner), vo);
+        } else {
+          __builtin_nontemporal_store(Algo::out(va[q][0], kTwo ? vb[q][0] : T(0), mx[0], fin[0]), out + base + kk * inner);
+        }
+      }
+    }
+  }
+}
+
+constexpr long kStridedSmall = 1 << 14;   // elements; below this one lane-per-slice launch beats two panel launches
+
 template <typename T, typename Algo>
 inline void launch_softmax_strided(hipStream_t stream, long inner, long d, long outer, const T* a, const T* b, T* out) {
   if (inner <= 0 || d <= 0 || outer <= 0) return;
   const long total = inner * outer;
-  hipLaunchKernelGGL((softmax_strided_kernel<T, Algo>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, inner, d, outer, a, b, out);
+  if (total * d <= kStridedSmall) {
+    hipLaunchKernelGGL((softmax_strided_kernel<T, Algo>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, inner, d, outer, a, b, out);
+    return;
+  }
+  constexpr int N = Vec16<T>::N;
+  const bool vec = inner % N == 0 && aligned16(a) && aligned16(out) && (Algo::kInputs < 2 || aligned16(b));
+  const long ti = (long)kWave * (vec ? N : 1);
+  const long itiles = (inner + ti - 1) / ti, ipad = itiles * ti;
+  long nchunks = (4L * tuning(kTuneNumCUs) + itiles * outer - 1) / (itiles * outer);   // about four workgroups per CU
+  const long maxchunks = d / (kPanelWaves * kPanelU) > 0 ? d / (kPanelWaves * kPanelU) : 1;
+  if (nchunks > maxchunks) nchunks = maxchunks;
+  if (nchunks > kPanelMaxChunks) nchunks = kPanelMaxChunks;   // every workgroup of the apply pass merges all chunks of its positions
+  if (nchunks < 1) nchunks = 1;
+  const long dchunk = (d + nchunks - 1) / nchunks;
+  nchunks = (d + dchunk - 1) / dchunk;
+  const long blocks = itiles * nchunks * outer;
+  if (blocks > 0x7fffffffL) { record_error("softmax over a strided dimension: too many panels"); return; }
+  Workspace ws = workspace_for(stream, sizeof(T) * (size_t)(outer * nchunks * 2 * ipad), 0);
+  if (ws.partial == nullptr) { record_error("softmax over a strided dimension: no scratch memory"); return; }
+  T* partial = static_cast<T*>(ws.partial);
+#define KNET8_PANEL(NV) do { \
+    hipLaunchKernelGGL((softmax_panel_reduce_kernel<T, Algo, NV>), dim3((unsigned)blocks), dim3(kPanelWaves * kWave), 0, stream, inner, d, itiles, nchunks, dchunk, ipad, a, b, partial); \
+    hipLaunchKernelGGL((softmax_panel_apply_kernel<T, Algo, NV>), dim3((unsigned)blocks), dim3(kPanelWaves * kWave), 0, stream, inner, d, itiles, nchunks, dchunk, ipad, a, b, partial, out); \
+  } while (0)
+  if (vec) KNET8_PANEL(N); else KNET8_PANEL(1);
+#undef KNET8_PANEL
 }
 
 template <typename T, typename Algo, int TEAM, int E>

@@ -54,7 +54,9 @@ def _bwd(kernel, y, dy, m, n):
     return dx
 
 
-_STRIDED_MAX = 1 << 14  # elements; above this the lane-per-slice kernel has too few lanes or too long walks
+_STRIDED_MAX = 1 << 14     # elements; above this the library's strided entry points switch from one lane per slice to panels
+_PANEL_MIN_INNER = 32      # panels put lanes along `inner`: below this most of a wave would idle and the permutation route wins
+_PANEL_MIN_SLICES = 2048   # inner*outer: with fewer slices the panels cannot fill the chip without cutting d into too many chunks
 
 
 def _permute213(x, m, n, batch):
@@ -87,10 +89,11 @@ def _make(kernel, backkernel):
             _, d, outer = v3
             y = _fwd(kernel, x, d, outer)
             return y, (lambda dy: (_bwd(backkernel, y, dy, d, outer),))
-        if v3 is not None and x.length > _STRIDED_MAX:
-            # A run of adjacent non-leading dims of a large array: permute (inner, d, outer) -> (d, inner, outer), run the column kernels
-            # on contiguous columns of length d, permute back -- the reference's route for 2-d dims=2 (src/ops20_gpu/softmax.jl:19-20),
-            # batched over the trailing dims.  The transposed result is kept for the backward pass, which needs exactly that.
+        if v3 is not None and (v3[0] < _PANEL_MIN_INNER or v3[0] * v3[2] < _PANEL_MIN_SLICES) and x.length > _STRIDED_MAX:
+            # A short contiguous run in front of the reduced dims (lanes along it would mostly idle), or few long slices: permute (inner, d, outer) ->
+            # (d, inner, outer), run the column kernels on contiguous columns of length d, permute back -- the reference's route
+            # for 2-d dims=2 (src/ops20_gpu/softmax.jl:19-20), batched over the trailing dims.  The transposed result is kept for
+            # the backward pass, which needs exactly that.
             inner, d, outer = v3
             xt = _permute213(x, inner, d, outer)
             yt = _fwd(kernel, xt, d, inner * outer)
@@ -100,7 +103,9 @@ def _make(kernel, backkernel):
                 dxt = _bwd(backkernel, yt, _permute213(dy, inner, d, outer), d, inner * outer)
                 return (_permute213(dxt, d, inner, outer).reshape(x.dims),)
             return y, back_t
-        if v3 is not None:  # small arrays: one strided kernel (a lane per slice) instead of three launches
+        if v3 is not None:
+            # in place, lanes along the contiguous `inner` axis: one lane-per-slice launch for small arrays, panel kernels
+            # (reduce + apply) for large ones -- no transposes
             inner, d, outer = v3
             y = x.similar()
             knet8("%s_strided_%s" % (kernel, x.suffix), inner, d, outer, x.ptr, y.ptr)

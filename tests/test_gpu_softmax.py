@@ -245,6 +245,56 @@ def test_logsumexp_value_and_gradient(knet, oracle):
         assert close(knet.Array(knet.grad(J, p)), wantg, 2e-5), (shape, dims)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_panel_kernels_for_softmax_along_a_strided_dimension(knet, oracle, dt):
+    """`*_strided_S(inner, d, outer, ...)` above 16 K elements: two launches (panel reduce, panel apply), lanes along `inner`.
+    Shapes cover vector and scalar lanes, ragged inner tiles, one and many chunks of d, several outer slabs, d not a multiple of
+    the unroll, and -inf entries (masked logits) including a slice that is -inf throughout."""
+    rng = np.random.default_rng(43)
+    tol = 1e-5 if dt == np.float32 else 1e-12
+    for inner, d, outer in ((256, 100, 3), (512, 3200, 1), (4096, 37, 1), (250, 129, 2), (33, 1000, 5), (1000, 17, 4), (64, 5000, 1), (260, 16, 20)):
+        x = (rng.standard_normal((inner, d, outer)) * 2).astype(dt)
+        if inner == 250:
+            x[rng.random(x.shape) < 0.2] = -np.inf
+            x[7, :, 1] = -np.inf              # a slice with no finite entry: NaN in, NaN out, as the formula gives on the CPU
+        xd = knet.KnetArray(x)
+        for name in ("logsoftmax", "softmax"):
+            y = xd.similar()
+            knet.knet8("%s_strided_%s" % (name, xd.suffix), inner, d, outer, xd.ptr, y.ptr)
+            got = knet.Array(y)
+            with np.errstate(all="ignore"):
+                want = getattr(oracle, name)(x, dims=2)
+            ok = np.isfinite(want)
+            assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got == -np.inf, want == -np.inf), (name, inner, d, outer)
+            assert np.allclose(got[ok], want[ok], rtol=tol * 10, atol=tol), (name, inner, d, outer)
+        xf = np.where(np.isfinite(x), x, dt(-30)).astype(dt)
+        yl, ys = oracle.logsoftmax(xf, dims=2), oracle.softmax(xf, dims=2)
+        dy = rng.standard_normal(x.shape).astype(dt)
+        for name, yv in (("logsoftmaxback", yl), ("softmaxback", ys)):
+            yd, dyd = knet.KnetArray(yv.astype(dt)), knet.KnetArray(dy)
+            dx = yd.similar()
+            knet.knet8("%s_strided_%s" % (name, yd.suffix), inner, d, outer, yd.ptr, dyd.ptr, dx.ptr)
+            want = getattr(oracle, name)(yv.astype(dt), dy, dims=2)
+            assert close(knet.Array(dx), want, 2e-5 if dt == np.float32 else 1e-11), (name, inner, d, outer)
+    # a view that does not start on a 16-byte boundary: scalar lanes
+    base = (rng.standard_normal(256 * 100 * 2 + 1) * 2).astype(dt)
+    big = knet.KnetArray(base)
+    v = big.view1d(1, 256 * 100 * 2)
+    y = v.similar()
+    knet.knet8("logsoftmax_strided_%s" % v.suffix, 256, 100, 2, v.ptr, y.ptr)
+    want = oracle.logsoftmax(base[1:].reshape((256, 100, 2), order="F"), dims=2)
+    assert np.allclose(knet.Array(y).reshape((256, 100, 2), order="F"), want, rtol=tol * 10, atol=tol)
+    # through the host mirror and the tape: dims=2 of a matrix, dims=(2,3) of a 4-d array
+    for shape, dims in (((300, 257), 2), ((40, 30, 20, 3), (2, 3))):
+        x = (rng.standard_normal(shape) * 2).astype(dt)
+        c = rng.standard_normal(shape).astype(dt)
+        p, cd = knet.Param(knet.KnetArray(x)), knet.KnetArray(c)
+        J = knet.diff(lambda: knet.sum(knet.mul(knet.logsoftmax(p, dims=dims), cd)))
+        yv = oracle.logsoftmax(x, dims=dims)
+        assert close(knet.Array(knet.grad(J, p)), oracle.logsoftmaxback(yv, c, dims=dims), 5e-5 if dt == np.float32 else 1e-11), shape
+    knet.libknet8().check()
+
+
 def test_logsumexp_over_any_dims(knet):
     """Reduced dims that are not the leading ones (src/ops20/softmax.jl:65-74 accepts any dims): against the formula in fp64."""
     rng = np.random.default_rng(39)

@@ -97,12 +97,17 @@ def test_softmax_and_activation_dispatch(knet, rec):
     assert calls[-1][:3] == ("softmax_32", 200, 30)
     knet.logsoftmax(arr((7,)), dims=1)
     assert calls[-1][:3] == ("logsoftmax_32", 7, 1)
+    knet.logsoftmax(x, dims=2)                             # non-leading dim: the strided entry point (inner, d, outer), whatever the size
+    assert calls[-1][:4] == ("logsoftmax_strided_32", 32000, 512, 1)
     n0 = len(calls)
-    knet.logsoftmax(x, dims=2)                             # non-leading dim of a large array: permute, column kernel, permute back
-    assert [c[:4] for c in calls[n0:]] == [("permute213_32", 32000, 512, 1), ("logsoftmax_32", 512, 32000, calls[n0 + 1][3]),
-                                           ("permute213_32", 512, 32000, 1)]
-    knet.logsoftmax(arr((30, 20)), dims=2)                 # small: one strided kernel (inner, d, outer)
+    knet.logsoftmax(arr((512, 32000)), dims=2)             # few, long slices: permute, column kernel, permute back
+    assert [c[0] for c in calls[n0:]] == ["permute213_32", "logsoftmax_32", "permute213_32"]
+    knet.logsoftmax(arr((30, 20)), dims=2)
     assert calls[-1][:4] == ("logsoftmax_strided_32", 30, 20, 1)
+    n0 = len(calls)
+    knet.logsoftmax(arr((8, 1000, 4096)), dims=2)          # a short contiguous run in front of a large array: permute, column kernel, permute back
+    assert [c[:4] for c in calls[n0:]] == [("permute213_32", 8, 1000, 4096), ("logsoftmax_32", 1000, 8 * 4096, calls[n0 + 1][3]),
+                                           ("permute213_32", 1000, 8, 4096)]
     knet.logsoftmax(arr((1, 500, 60)), dims=2)             # leading dims of size 1: contiguous columns after all
     assert calls[-1][:3] == ("logsoftmax_32", 500, 60)
     knet.logsoftmaxback(x, x, dims=1)
