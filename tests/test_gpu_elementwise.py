@@ -418,6 +418,25 @@ def test_pow_and_comparisons(knet, dt):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt,n", [(np.float32, 1 << 28), (np.float64, 1 << 27)])
+def test_config2_full_size_bit_exact(knet, oracle, dt, n):
+    """Benchmark config 2 at its real size: the five activation gradients on 2^28 fp32 / 2^27 fp64 elements, y from the forward of
+    x ~ N(0,1), dy ~ N(0,1), every bit compared with the CPU restatement."""
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal(n, dtype=dt)
+    dy = rng.standard_normal(n, dtype=dt)
+    dyd = knet.KnetArray(dy)
+    for name, fwd in BACK11:
+        y = oracle.unary(fwd, x)
+        yd = knet.KnetArray(y)
+        got = knet.Array(getattr(knet, name)(dyd, yd))
+        want = oracle.back11(name, dy, y)
+        assert got.view(np.uint32 if dt == np.float32 else np.uint64).tobytes() == want.view(np.uint32 if dt == np.float32 else np.uint64).tobytes(), name
+        del yd, got, want, y
+    knet.libknet8().fn["knet8_trim"]()
+    knet.libknet8().check()
+
+
 def test_largest_length_the_abi_can_express(knet):
     """n = 2^31 - 1 elements (the `int n` of the entry points at its maximum): 8 GiB per fp32 array.  reluback on a +1/-1 pattern and
     the whole-array sum over it; sizes and offsets inside the kernels must not wrap."""
