@@ -57,6 +57,76 @@ def test_every_symbol_of_the_reference_library_is_exported(built_lib):
     assert not [n for n in names if not hasattr(lib, n)]
 
 
+def _split_top(text):
+    """Split at top-level commas (parentheses, braces and brackets nest; string literals are skipped)."""
+    parts, depth, cur, q = [], 0, "", False
+    for ch in text:
+        if ch == '"':
+            q = not q
+        if not q:
+            if ch in "([{":
+                depth += 1
+            elif ch in ")]}":
+                depth -= 1
+            elif ch == "," and depth == 0:
+                parts.append(cur.strip())
+                cur = ""
+                continue
+        cur += ch
+    if cur.strip():
+        parts.append(cur.strip())
+    return parts
+
+
+def test_julia_binding_calls_match_the_header():
+    """Every `@knet8(name, (argtypes...), args...)` and `ccall((:name, libknet8), ...)` in knet.jl_amd/julia/*.jl names a symbol
+    include/knet8.h declares, with as many argument types as the C declaration has parameters (the files are not executed here)."""
+    import glob
+    import re
+    lk = _load("lk_for_test3", "knet.jl_amd/libknet8.py")
+    decls = lk.parse_header()
+    acts = ("relu", "sigm", "tanh", "elu", "selu")
+
+    def expand(tmpl):
+        names = [tmpl]
+        for pat, vals in ((r"\$\(?S\)?", ("32", "64")), (r"\$\(f\)", acts)):
+            names = [re.sub(pat, v, n, count=0) for n in names for v in vals] if re.search(pat, names[0]) else names
+        return names
+    checked = 0
+    for path in sorted(glob.glob(os.path.join(ROOT, "knet.jl_amd", "julia", "*.jl"))):
+        text = "\n".join(l for l in open(path).read().splitlines() if not l.lstrip().startswith("#"))
+        # variables holding symbol templates:  fwd, bwd = "bias$(f)_$S", "$(f)back_biasgrad_$S"   /   g = "gemm_$(S)_stream"
+        names = {}
+        for m in re.finditer(r"^\s*([\w, ]+?)\s*=\s*(\"[^\n]*\")\s*$", text, flags=re.M):
+            vs, ss = [v.strip() for v in m.group(1).split(",")], re.findall(r'"([^"]*)"', m.group(2))
+            if len(vs) == len(ss):
+                names.update(zip(vs, ss))
+        for m in re.finditer(r"\(:(\w+),\s*(?:LibKnet8\.)?libknet8\)", text):
+            assert m.group(1) in decls, (os.path.basename(path), m.group(1))
+            checked += 1
+        for m in re.finditer(r"@knet8r?\(", text):
+            depth, i = 1, m.end()
+            while depth:
+                depth += {"(": 1, ")": -1}.get(text[i], 0)
+                i += 1
+            args = _split_top(text[m.end():i - 1])
+            sym = args[0]
+            is_r = text[m.start():m.end()].startswith("@knet8r")
+            types = args[2 if is_r else 1]
+            if sym.startswith('$("'):
+                tmpl = re.match(r'\$\("([^"]*)"\)', sym).group(1)
+            elif sym.startswith("$"):
+                tmpl = names[sym[1:]]
+            else:
+                tmpl = sym
+            ntypes = len(_split_top(types.strip()[1:-1]))
+            for name in expand(tmpl):
+                assert name in decls, (os.path.basename(path), name)
+                assert len(decls[name][1]) == ntypes, (os.path.basename(path), name, decls[name][1], types)
+                checked += 1
+    assert checked >= 40
+
+
 def test_no_undefined_device_runtime_surprises(built_lib):
     # the product must not link the oracle or anything outside HIP / hipBLASLt / the C++ runtime
     out = subprocess.check_output(["readelf", "-d", built_lib], text=True)
