@@ -145,6 +145,46 @@ def time_kernel(K, torch, make_launch, nbytes, footprints, reps=20):
     return out
 
 
+def neighbours(torch, K):
+    """Kernels either side of the gradient path (random numbers for dropout masks, permutations, softmax along a strided
+    dimension): cold figures on rotating buffers, same method as the config-3/4 table."""
+    res = {}
+    f32 = np.float32
+
+    def arr(n, seed):
+        a = K.KnetArray(dtype=f32, dims=(n,))
+        K.randn_(a, seed=seed)
+        return a
+    n28 = 1 << 28
+    out = K.KnetArray(dtype=f32, dims=(n28,))    # 1 GiB: four times the memory-side cache, one buffer is cold enough
+    res["rand_32 n=2^28 (write only)"] = time_kernel(
+        K, torch, lambda i: (lambda: K.knet8("rand_seeded_32", n28, 1, 0, out.ptr)), 4 * n28, [0], reps=6)
+    del out
+    for dims, perm in (((4096, 8192), (2, 1)), ((56, 56, 256, 64), (3, 1, 2, 4)), ((32000, 512), (2, 1))):
+        n = int(np.prod(dims))
+        nsets = max(2, int(1.3e9 / (8 * n)) + 1)
+        xs = [arr(n, 300 + i) for i in range(nsets)]
+        ys = [x.similar() for x in xs]
+        nd = len(dims)
+        dh, ph = (ctypes.c_int * nd)(*dims), (ctypes.c_int * nd)(*perm)
+        res["permutedims_32 %s perm %s" % (dims, perm)] = time_kernel(
+            K, torch, lambda i: (lambda: K.knet8("permutedims_32", nd, ctypes.cast(dh, ctypes.c_void_p), ctypes.cast(ph, ctypes.c_void_p), xs[i].ptr, ys[i].ptr)),
+            8 * n, list(range(nsets)))
+        del xs, ys
+    for inner, d, outer in ((32000, 512, 1), (256, 1000, 64)):
+        n = inner * d * outer
+        nsets = max(2, int(1.3e9 / (12 * n)) + 1)
+        xs = [arr(n, 400 + i) for i in range(nsets)]
+        ys = [x.similar() for x in xs]
+        res["logsoftmax_strided_32 (%d,%d,%d) over the middle dimension (algorithmic 8 B/element)" % (inner, d, outer)] = time_kernel(
+            K, torch, lambda i: (lambda: K.knet8("logsoftmax_strided_32", inner, d, outer, xs[i].ptr, ys[i].ptr)), 8 * n, list(range(nsets)))
+        res["logsoftmaxback_strided_32 (%d,%d,%d) (algorithmic 12 B/element)" % (inner, d, outer)] = time_kernel(
+            K, torch, lambda i: (lambda: K.knet8("logsoftmaxback_strided_32", inner, d, outer, xs[i].ptr, ys[i].ptr, ys[i].ptr)), 12 * n, list(range(nsets)))
+        del xs, ys
+    K.libknet8().check()
+    return res
+
+
 def extras(torch, K):
     res = {}
     f32 = torch.float32
@@ -476,6 +516,9 @@ def main():
         ex = extras(torch, K)
         line["kernels_config3_4_5"] = {k: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for k, v in ex.items()}
         torch.cuda.empty_cache()
+        K.libknet8().fn["knet8_trim"]()
+        nb = neighbours(torch, K)
+        line["kernels_next_to_the_path"] = {k: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for k, v in nb.items()}
         K.libknet8().fn["knet8_trim"]()
         line["mlp"] = {
             "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager through the tape, step-by-step nll as in the reference)":
