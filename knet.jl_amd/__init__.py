@@ -16,7 +16,7 @@ from .reduction import sum, prod, maximum, minimum, sumabs, sumabs2, maxabs, min
 from .binary import add, sub, mul, div, fill, zero, unbroadcast, broadcast_op
 from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softmaxback
 from .cat import cat, hcat, vcat
-from .statistics import mean, var, std, norm, isequal, isapprox
+from .statistics import mean, var, std, varm, stdm, norm, isequal, isapprox
 from .random import seed_, rand_, randn_, RngState
 from .loss import nll, findindices, accuracy, getindex, ungetindex, bce, logistic
 from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat)

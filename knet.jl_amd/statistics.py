@@ -41,8 +41,14 @@ def _sqrt(v):
     return y, (lambda dy: (dy / (2 * y),))
 
 
-def mean(x, dims=None):
-    """``b = sum(a; dims); b .* T(length(b)/length(a))`` (statistics.jl:4)."""
+def mean(x, dims=None, f=None):
+    """``b = sum(a; dims); b .* T(length(b)/length(a))`` (statistics.jl:4); with ``f`` in ("abs", "abs2") the reference's
+    ``mean(f, a) = sum(f, a) / length(a)`` (statistics.jl:5, through the ``sumabs`` / ``sumabs2`` reductions)."""
+    if f is not None:
+        if f not in ("abs", "abs2"):
+            raise ValueError("mean(f, x): f must be 'abs' or 'abs2'")
+        total = (R.sumabs if f == "abs" else R.sumabs2)(x)
+        return _divn(total, _len(x))
     b = R.sum(x, dims=dims)
     return _scale(b, _len(b) / _len(x))
 
@@ -58,6 +64,16 @@ def var(x, dims=None, corrected=True, mean=None):
 def std(x, dims=None, corrected=True, mean=None):
     """``sqrt.(var(x; ...))`` (statistics.jl:6)."""
     return _sqrt(var(x, dims=dims, corrected=corrected, mean=mean))
+
+
+def varm(x, m, dims=None, corrected=True):
+    """``varm(x, m; corrected, dims)`` (statistics.jl:9)."""
+    return var(x, dims=dims, corrected=corrected, mean=m)
+
+
+def stdm(x, m, dims=None, corrected=True):
+    """``stdm(x, m; corrected, dims)`` (statistics.jl:7)."""
+    return std(x, dims=dims, corrected=corrected, mean=m)
 
 
 def norm(x, p=2):

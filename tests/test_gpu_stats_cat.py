@@ -92,3 +92,57 @@ def test_mean_var_std_norm_and_comparisons(knet, dt):
     sd = x2.std(axis=0, ddof=1, keepdims=True)
     assert np.allclose(knet.Array(knet.grad(J, w)), (x2 - x2.mean(axis=0, keepdims=True)) / ((x2.shape[0] - 1) * sd), rtol=1e-4, atol=1e-5)
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_statistics_as_the_reference_tests_them(knet, dt):
+    """test/statistics.jl:12-51 on a (3,4) array: every call against numpy, every gradient against central differences in fp64
+    of the same formula (the reference uses @gcheck)."""
+    rng = np.random.default_rng(44)
+    a = rng.standard_normal((3, 4)).astype(dt)
+    k = knet.KnetArray(a)
+    a64 = a.astype(np.float64)
+    rt = 1e-5 if dt == np.float32 else 1e-12
+
+    def val(v):
+        return knet.Array(v) if isinstance(v, knet.KnetArray) else np.float64(v)
+    cases = [
+        (lambda x: knet.mean(x), lambda x: x.mean()),
+        (lambda x: knet.mean(x, dims=1), lambda x: x.mean(axis=0, keepdims=True)),
+        (lambda x: knet.mean(x, dims=2), lambda x: x.mean(axis=1, keepdims=True)),
+        (lambda x: knet.mean(x, f="abs"), lambda x: np.abs(x).mean()),
+        (lambda x: knet.mean(x, f="abs2"), lambda x: (x * x).mean()),
+        (lambda x: knet.std(x), lambda x: x.std(ddof=1)),
+        (lambda x: knet.std(x, dims=1), lambda x: x.std(axis=0, ddof=1, keepdims=True)),
+        (lambda x: knet.std(x, dims=2), lambda x: x.std(axis=1, ddof=1, keepdims=True)),
+        (lambda x: knet.stdm(x, knet.mean(x)), lambda x: x.std(ddof=1)),
+        (lambda x: knet.stdm(x, knet.mean(x, dims=1), dims=1), lambda x: x.std(axis=0, ddof=1, keepdims=True)),
+        (lambda x: knet.stdm(x, knet.mean(x, dims=2), dims=2), lambda x: x.std(axis=1, ddof=1, keepdims=True)),
+        (lambda x: knet.var(x), lambda x: x.var(ddof=1)),
+        (lambda x: knet.var(x, dims=1), lambda x: x.var(axis=0, ddof=1, keepdims=True)),
+        (lambda x: knet.var(x, dims=2), lambda x: x.var(axis=1, ddof=1, keepdims=True)),
+        (lambda x: knet.varm(x, knet.mean(x)), lambda x: x.var(ddof=1)),
+        (lambda x: knet.varm(x, knet.mean(x, dims=1), dims=1), lambda x: x.var(axis=0, ddof=1, keepdims=True)),
+        (lambda x: knet.varm(x, knet.mean(x, dims=2), dims=2), lambda x: x.var(axis=1, ddof=1, keepdims=True)),
+    ]
+    for n, (f, ref) in enumerate(cases):
+        got = val(f(k))
+        want = ref(a64)
+        assert np.shape(got) == np.shape(want) and np.allclose(got, want, rtol=rt * 10, atol=rt), n
+        # gradient of sum(f(x)) wrt x
+        p = knet.Param(k)
+
+        def loss():
+            v = f(p)
+            return knet.sum(v) if isinstance(knet.value(v), knet.KnetArray) else v
+        J = knet.diff(loss)
+        g = knet.Array(knet.grad(J, p))
+        fd = np.zeros_like(a64)
+        h = 1e-6
+        for idx in np.ndindex(a64.shape):
+            up, dn = a64.copy(), a64.copy()
+            up[idx] += h
+            dn[idx] -= h
+            fd[idx] = (np.sum(ref(up)) - np.sum(ref(dn))) / (2 * h)
+        assert np.allclose(g, fd, rtol=2e-3 if dt == np.float32 else 1e-6, atol=2e-4 if dt == np.float32 else 1e-7), (n, g, fd)
+    knet.libknet8().check()
