@@ -18,8 +18,9 @@ from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softm
 from .cat import cat, hcat, vcat
 from .statistics import mean, var, std, varm, stdm, norm, isequal, isapprox
 from .random import seed_, rand_, randn_, RngState
-from .loss import nll, findindices, accuracy, getindex, ungetindex, bce, logistic
-from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat)
+from .loss import nll, findindices, accuracy, ungetindex, bce, logistic
+from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat,
+                       getindex, setindex_)
 from .dropout import dropout, dropback, dropout_, dropback_
 from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
 from .linalg import dense, matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims

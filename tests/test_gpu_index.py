@@ -182,3 +182,142 @@ def test_icat_and_concat(knet, dt):
     got = knet.Array(knet.concat([knet.KnetArray(a) if a.size else knet.KnetArray(np.zeros(1, dt)).view1d(0, 0) for a in arrs]))
     assert bits_equal(got, np.concatenate(arrs))
     knet.libknet8().check()
+
+
+def _np_index(I, shape):
+    """The numpy (0-based) equivalent of a 1-based index tuple of the mirror, for arrays stored in Julia (column-major) order."""
+    out = []
+    for i in I:
+        if i is None:
+            out.append(slice(None))
+        elif isinstance(i, (int, np.integer)):
+            out.append(int(i) - 1)
+        elif isinstance(i, tuple) and len(i) == 2:
+            out.append(slice(i[0] - 1, i[1]))
+        elif isinstance(i, tuple):
+            a, s, b = i
+            out.append(np.arange(a, b + (1 if s > 0 else -1), s) - 1)
+        else:
+            arr = np.asarray(i)
+            out.append(arr if arr.dtype == np.bool_ else arr - 1)
+    return tuple(out)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_every_index_form_of_the_reference_test(knet, dt):
+    """test/karray.jl:24-66: Colon, Int, UnitRange, StepRange, Vector{Int}, repeated indices, Array{Int}, masks, in one and two
+    positions; a[i...] == k[i...], k[i...] .= 0 and back, and the gradient of getindex."""
+    rng = np.random.default_rng(61)
+    a = rng.random((3, 4)).astype(dt)
+    flat = lambda x: x.reshape(-1, order="F")
+    mask_all = rng.random((3, 4)) > 0.4
+    forms = [
+        (None,), (None, None),
+        (3,), (2, 3),
+        ((3, 5),), ((1, 2), (3, 4)),
+        (2, None), (None, 2),
+        ((1, 2), None), (None, (1, 2)),
+        ((1, 2), 2), (2, (1, 2)),
+        ((1, 2, 3),),
+        ((1, 2, 3), None), (None, (1, 2, 3)),
+        ([1, 3],), ([2, 2],),
+        ([1, 3], None), (None, [1, 3]),
+        ([2, 2], None), (None, [2, 2]),
+        (mask_all,),
+        (np.array([[1, 3], [2, 4]]),),
+        (None, np.array([True, False, True, True])), (np.array([True, False, True]), None),
+    ]
+    for I in forms:
+        k = knet.KnetArray(a)
+        got = knet.getindex(k, *I)
+        if len(I) == 1:      # linear indexing walks the array in column-major order
+            lin = _np_index(I, a.shape)[0]
+            fa = flat(a)
+            if isinstance(lin, np.ndarray) and lin.dtype == np.bool_:
+                want = fa[flat(lin)]
+            elif isinstance(lin, np.ndarray):
+                want = fa[flat(lin)].reshape(lin.shape, order="F")
+            else:
+                want = fa[lin]
+        else:
+            want = a[_np_index(I, a.shape)]
+        if isinstance(got, knet.KnetArray):
+            g = knet.Array(got)
+            assert g.shape == np.shape(want) and bits_equal(g, np.asarray(want)), I
+        else:
+            assert dt(got) == want, I
+        # k[i...] .= 0, then back to the old values (array assignment), compared with the same assignments in numpy
+        ref = a.copy(order="F")
+        knet.setindex_(k, 0, *I)
+        if len(I) == 1:
+            fr = flat(ref).copy()
+            lin = _np_index(I, a.shape)[0]
+            fr[flat(lin) if isinstance(lin, np.ndarray) else lin] = 0
+            ref = fr.reshape(a.shape, order="F")
+        else:
+            ref[_np_index(I, a.shape)] = 0
+        assert bits_equal(knet.Array(k), ref), I
+        if isinstance(got, knet.KnetArray):
+            # repeated indices write the same value twice: the result is the original array again
+            knet.setindex_(k, knet.KnetArray(np.asarray(want)), *I)
+        else:
+            knet.setindex_(k, float(want), *I)
+        assert bits_equal(knet.Array(k), a), I
+        # gradient of sum(w .* a[i...]) wrt a: w scattered (and accumulated on repeats) at the selection
+        p = knet.Param(knet.KnetArray(a))
+        if isinstance(got, knet.KnetArray):
+            w = rng.integers(1, 5, size=np.shape(want)).astype(dt)
+            J = knet.diff(lambda: knet.sum(knet.mul(knet.getindex(p, *I), knet.KnetArray(w))))
+        else:
+            w = np.asarray(1, dtype=dt)
+            J = knet.diff(lambda: knet.getindex(p, *I))
+        g = knet.Array(knet.grad(J, p))
+        wantg = np.zeros(a.shape, dt, order="F")
+        if len(I) == 1:
+            fg = np.zeros(a.size, dt)
+            lin = _np_index(I, a.shape)[0]
+            np.add.at(fg, flat(lin) if isinstance(lin, np.ndarray) else lin, flat(np.asarray(w)) if np.ndim(w) else w)
+            wantg = fg.reshape(a.shape, order="F")
+        else:
+            np.add.at(wantg, _np_index(I, a.shape), w)
+        assert bits_equal(g, wantg), I
+    knet.libknet8().check()
+
+
+def test_index_dispatch_on_higher_dims_masks_on_the_device_and_errors(knet):
+    rng = np.random.default_rng(62)
+    a = rng.random((3, 4, 5)).astype(np.float32)
+    k = knet.KnetArray(a)
+    # A[:,:,I] (src/knetarrays/getindex.jl:748-770)
+    assert bits_equal(knet.Array(knet.getindex(k, None, None, 2)), a[:, :, 1])
+    assert bits_equal(knet.Array(knet.getindex(k, None, None, (2, 4))), a[:, :, 1:4])
+    assert bits_equal(knet.Array(knet.getindex(k, None, None, None)), a)
+    assert bits_equal(knet.Array(knet.getindex(k, None, None, [5, 1, 1])), a[:, :, [4, 0, 0]])
+    knet.setindex_(k, 7, None, None, (2, 3))
+    ref = a.copy()
+    ref[:, :, 1:3] = 7
+    assert bits_equal(knet.Array(k), ref)
+    assert knet.getindex(k, 2, 3, 4) == ref[1, 2, 3]
+    # x[:, m] with an index matrix (getindex.jl:780): embedding lookup of a batch of sequences
+    emb = rng.random((6, 10)).astype(np.float32)
+    m = rng.integers(1, 11, size=(4, 3))
+    got = knet.Array(knet.getindex(knet.KnetArray(emb), None, m))
+    assert got.shape == (6, 4, 3) and bits_equal(got, emb[:, m - 1])
+    # a mask computed on the device: k .> 0.5 is a KnetArray of 0/1 values (getindex.jl:584-590)
+    x = rng.random((5, 7)).astype(np.float32)
+    xd = knet.KnetArray(x)
+    maskd = knet.broadcast_op("gt", xd, 0.5)
+    assert bits_equal(knet.Array(knet.getindex(xd, maskd)), x.reshape(-1, order="F")[(x > 0.5).reshape(-1, order="F")])
+    knet.setindex_(xd, 0, maskd)
+    assert bits_equal(knet.Array(xd), np.where(x > 0.5, np.float32(0), x))
+    # errors
+    for bad in ((0,), (13,), ((0, 2),), ((2, 13),), (4, 1), (None, 5), ([0, 1],), (None, [1, 5]), (np.array([True, False]),)):
+        with pytest.raises(IndexError):
+            knet.getindex(knet.KnetArray(rng.random((3, 4)).astype(np.float32)), *bad)
+    with pytest.raises(TypeError):
+        knet.getindex(knet.KnetArray(a), [1, 2], [1, 2])
+    with pytest.raises(TypeError):
+        knet.getindex(knet.KnetArray(a), 1.5)
+    with pytest.raises(ValueError):
+        knet.setindex_(knet.KnetArray(a[:, :, 0].copy()), knet.KnetArray(np.zeros(5, np.float32)), None, [1, 2])
+    knet.libknet8().check()
