@@ -26,3 +26,27 @@ from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, u
 from .linalg import dense, matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
 
 libknet8()  # fail loudly at import time if the HIP library is missing
+
+
+# ---- operator sugar: a + b, a - b, a * b (elementwise, Julia's .*), a / b, -a, a @ b (matrix product, Julia's *) on KnetArray,
+# Param and tape nodes; each is the primitive of the same name, so expressions written with operators are differentiable.
+def _attach_operators():
+    from . import autograd as _ag
+
+    def _neg(a):
+        return mul(a, -1)
+    ops = {
+        "__add__": lambda a, b: add(a, b), "__radd__": lambda a, b: add(b, a),
+        "__sub__": lambda a, b: sub(a, b), "__rsub__": lambda a, b: sub(b, a),
+        "__mul__": lambda a, b: mul(a, b), "__rmul__": lambda a, b: mul(b, a),
+        "__truediv__": lambda a, b: div(a, b), "__rtruediv__": lambda a, b: div(b, a),
+        "__matmul__": lambda a, b: matmul(a, b), "__rmatmul__": lambda a, b: matmul(b, a),
+        "__neg__": _neg,
+    }
+    for cls in (KnetArray, _ag.Node, Param):
+        for name, fn in ops.items():
+            setattr(cls, name, fn)
+
+
+from .binary import div  # noqa: E402
+_attach_operators()

@@ -162,8 +162,18 @@ def mul(x, y):
                                                                                 unbroadcast(y, broadcast_op("mul", dy, x)) if need[1] else None))
 
 
+@primitive
 def div(x, y):
-    return broadcast_op("div", x, y)
+    """``x ./ y``; gradients ``unbroadcast(x, dy./y)`` and ``unbroadcast(y, -dy.*x./(y.*y))`` (AutoGrad's rule for ``/``)."""
+    def back(dy, need=(True, True)):
+        gx = gy = None
+        if need[0]:
+            gx = unbroadcast(x, broadcast_op("div", dy, y))
+        if need[1]:
+            yy = broadcast_op("mul", y, y) if isinstance(y, KnetArray) else y * y
+            gy = unbroadcast(y, _neg(broadcast_op("div", broadcast_op("mul", dy, x), yy)))
+        return gx, gy
+    return broadcast_op("div", x, y), selective(back)
 
 
 def fill(x, v):

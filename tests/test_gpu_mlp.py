@@ -165,3 +165,39 @@ def test_matmul_and_transpose_gradients_as_the_reference_checks_them(knet):
         J = knet.diff(lambda: knet.sum(knet.mul(knet.transpose(pa), knet.KnetArray(wt))))
         assert np.array_equal(knet.Array(knet.grad(J, pa)), wt.T)
     knet.libknet8().check()
+
+
+def test_operator_sugar_and_division_gradient(knet):
+    """a + b, a - b, a * b, a / b, -a, a @ b on KnetArray / Param / tape nodes are the primitives of the same name; `/` has the
+    quotient-rule gradients (checked by central differences in fp64), also through broadcasting."""
+    rng = np.random.default_rng(71)
+    a = rng.standard_normal((5, 7))
+    b = rng.standard_normal((5, 7)) + 3.0
+    c = rng.standard_normal((5, 1)) + 3.0
+    w = rng.standard_normal((4, 5))
+    ka, kb, kc, kw = (knet.KnetArray(v) for v in (a, b, c, w))
+    assert np.allclose(knet.Array(ka + kb), a + b) and np.allclose(knet.Array(ka - kb), a - b)
+    assert np.allclose(knet.Array(ka * kb), a * b) and np.allclose(knet.Array(ka / kb), a / b)
+    assert np.allclose(knet.Array(-ka), -a) and np.allclose(knet.Array(kw @ ka), w @ a)
+    assert np.allclose(knet.Array(2.0 * ka + 1.0), 2 * a + 1) and np.allclose(knet.Array(1.0 - ka), 1 - a)
+    assert np.allclose(knet.Array(ka / 4.0), a / 4) and np.allclose(knet.Array(3.0 / kb), 3 / b)
+    assert np.allclose(knet.Array(ka / kc), a / c)
+    pa, pb, pc, pw = (knet.Param(knet.KnetArray(v)) for v in (a, b, c, w))
+
+    def f_np(a_, b_, c_, w_):
+        return float(np.sum((w_ @ (a_ / b_ + 2.0 * a_ / c_)) * (w_ @ (-a_ + 1.0 / b_))))
+
+    J = knet.diff(lambda: knet.sum((pw @ (pa / pb + 2.0 * pa / pc)) * (pw @ (-pa + 1.0 / pb))))
+    assert abs(float(J.value) - f_np(a, b, c, w)) <= 1e-10 * abs(f_np(a, b, c, w))
+    for p, k, arrs in ((pa, 0, a), (pb, 1, b), (pc, 2, c), (pw, 3, w)):
+        g = knet.Array(knet.grad(J, p))
+        fd = np.zeros_like(arrs)
+        h = 1e-6
+        for idx in np.ndindex(arrs.shape):
+            args = [a.copy(), b.copy(), c.copy(), w.copy()]
+            args[k][idx] += h
+            up = f_np(*args)
+            args[k][idx] -= 2 * h
+            fd[idx] = (up - f_np(*args)) / (2 * h)
+        assert np.allclose(g, fd, rtol=1e-5, atol=1e-6), k
+    knet.libknet8().check()
