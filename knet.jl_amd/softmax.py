@@ -66,12 +66,6 @@ def _permute213(x, m, n, batch):
     return y
 
 
-def permutedims(x):
-    """2-d transpose (the reference uses CUDA.jl's permutedims, src/knetarrays/reshape.jl:18)."""
-    from .linalg import transpose
-    return transpose(x)
-
-
 def _make(kernel, backkernel):
     @primitive
     def f(x, dims=None):
