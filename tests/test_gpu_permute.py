@@ -45,6 +45,7 @@ def test_every_kernel_shape_class(knet):
              ((129, 131), (1, 0)),             # plain transpose, ragged 64x64 tiles
              ((3, 1000), (1, 0)), ((1000, 3), (1, 0)), ((16, 777), (1, 0)), ((777, 10), (1, 0)),   # skinny tiles
              ((70, 6, 75), (2, 1, 0)), ((70, 6, 75), (2, 0, 1)), ((70, 6, 75), (1, 2, 0)),
+             ((7, 3, 100), (2, 0, 1)), ((3, 7, 200), (2, 0, 1)), ((100, 3, 7), (1, 2, 0)), ((200, 7, 3), (2, 0, 1)),   # every skinny tile shape with a batch stride
              ((8, 9, 10, 11), (3, 0, 1, 2)),   # dims 0-2 merge into one: a 2-d transpose of (720, 11)
              ((8, 9, 10, 11), (2, 3, 0, 1)),   # pairs merge: (72, 110) transposed
              ((56, 56, 32, 4), (2, 0, 1, 3)),  # channels first <-> channels last
