@@ -65,6 +65,36 @@ def test_zero_and_negative_sizes_are_no_ops(knet):
     knet.libknet8().check()
 
 
+def test_every_entry_point_is_a_no_op_on_empty_arrays(knet):
+    """All kernel entry points of the header, called with every size argument 0 (what an empty KnetArray passes): nothing is
+    launched, nothing is recorded as an error, nothing is written."""
+    lib = knet.libknet8()
+    a = knet.KnetArray(np.full(64, 3.0, np.float64))
+    count = 0
+    for name, (ret, args) in sorted(lib.decls.items()):
+        if name.endswith("_stream") or name.startswith(("knet8_", "gemm_", "permutedims")):
+            continue      # runtime calls; gemm takes transpose characters; permutedims rejects ndims = 0 by design
+        vals = []
+        for t in args:
+            if t == "int":
+                vals.append(0)
+            elif t == "float":
+                vals.append(ctypes.c_float(1.0))
+            elif t == "double":
+                vals.append(ctypes.c_double(1.0))
+            elif t == "unsigned long long":
+                vals.append(0)
+            else:
+                vals.append(a.ptr)
+        lib.fn[name](*vals)
+        msg = lib.fn["knet8_last_error"]()
+        assert not msg, (name, msg)
+        count += 1
+    assert count > 600
+    knet.synchronize()
+    assert np.all(knet.Array(a) == 3.0)
+
+
 def test_broadcast_forms_keep_operand_order(knet):
     rng = np.random.default_rng(53)
     fn = knet.libknet8().fn
