@@ -4,6 +4,12 @@ TEST INFRASTRUCTURE: only the tests, the smoke check and the benchmark's CPU
 baseline may import this module.  Arrays are numpy arrays carrying Julia shapes;
 memory order is column-major (``order='F'``) exactly as Knet's ``Array`` path.
 Dimension numbers (``dims``) and labels are 1-based as in the reference.
+
+Besides the C functions (pins listed in ``knet_cpu.c``) this module restates in numpy the counter-based generator behind
+``rand!/randn!`` (``philox4x32_10``, ``rand_uniform``, ``rand_normal``): pinned by the Random123 known-answer vectors, a
+brute-force integer restatement and an mpmath evaluation of the Box-Muller transform (tests/test_oracle_elementwise.py).
+PARITY UNPINNED there: the actual numbers of the reference's streams, which come from cuRAND (device) and Julia's generator
+(CPU) and cannot be reproduced here; the reference's own test compares the two only statistically (test/dropout.jl:8-17).
 """
 import ctypes
 import os
