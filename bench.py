@@ -527,7 +527,7 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
             "config1 same graph with dense layers (product, bias and relu in one launch)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
-            "config1 same step from a compiled C99 host through the C ABI (eager, 8 launches, fused layer kernels)": c_host_steps(K),
+            "config1 same step from a compiled C99 host through the C ABI (eager, 5 launches: fused layer kernels forward and backward)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),

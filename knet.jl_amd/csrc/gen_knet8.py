@@ -233,6 +233,7 @@ PRELUDE = BANNER + """#include "../knet8_runtime.h"
 #include "../knet8_broadcast.h"
 #include "../knet8_reduce.h"
 #include "../knet8_fused.h"
+#include "../knet8_dense.h"
 #include "../knet8_softmax.h"
 #include "../knet8_index.h"
 #include "../knet8_transpose.h"
@@ -440,6 +441,18 @@ def gen_elementwise():
                     [("int", "m"), ("int", "n"), (T + "*", "dy"), (T + "*", "y"), (T + "*", "dz"), (T + "*", "db")],
                     "launch_actback_biasgrad<%s>(stream, m, n, dy, y, dz, db, Op11_%sback<%s>())" % (T, act, T),
                     "%sback_S_11 + sum_S_21, src/ops20_gpu/activation.jl:30-37, src/knetarrays/reduction.jl:21-77" % act)
+    o.decl.append("/* dense_back_S: the backward pass of one small dense layer y = f(W*x + b) in one launch.  W is m x k, x is k x n, y and dy\n"
+                  "   are m x n (column-major, no padding); act 0: dz = dy, act 1: dz = y > 0 ? dy : 0 (relu).  Writes dW = dz*x' (m x k),\n"
+                  "   db = sum(dz; dims=2) (m) and dx = W'*dz (k x n); any of the three may be NULL (db needs dW).  Returns 0 when done, 1 when\n"
+                  "   the layer is too large for the small-matrix kernels -- nothing is launched then and the caller uses Fback_biasgrad_S\n"
+                  "   and gemm_S instead --, -1 on bad arguments.  No libknet8 counterpart: replaces reluback + sum(dz;dims=2) + two gemm!\n"
+                  "   calls (src/ops20_gpu/activation.jl:30-37, src/knetarrays/reduction.jl:21-77, src/knetarrays/linalg.jl:11-18). */")
+    for T, S in TYPES:
+        o.entry("dense_back_%s" % S, "int",
+                [("int", "act"), ("int", "m"), ("int", "n"), ("int", "k"), (T + "*", "W"), (T + "*", "x"), (T + "*", "y"), (T + "*", "dy"),
+                 (T + "*", "dW"), (T + "*", "db"), (T + "*", "dx")], None,
+                "reluback_S_11 + sum_S_21 + gemm! x 2, src/knetarrays/linalg.jl:11-18",
+                body="  const int rc = launch_dense_back<%s>(stream, act, m, n, k, W, x, y, dy, dW, db, dx);\n  knet8::check_launch(\"dense_back_%s\");\n  return rc;" % (T, S))
     for T, S in TYPES:
         o.entry("biasreludrop_%s" % S, "void", [("int", "m"), ("int", "n"), (T, "p"), (T + "*", "z"), (T + "*", "b"), (T + "*", "y")],
                 "launch_bias_act<%s, true>(stream, m, n, z, b, y, BiasReluDrop<%s>{p, %s(1) - p})" % (T, T, T),

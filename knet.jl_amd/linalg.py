@@ -73,6 +73,18 @@ def dense(w, x, b, act=None):
         raise RuntimeError("gemm_bias_act failed")
 
     def back(dy, need=(True, True, True)):
+        # small layers: activation gradient, bias gradient and both products in one launch (dense_back_S); it declines (1) large ones
+        if need[0] or not need[2]:
+            dW = w.similar((m, k)) if need[0] else None
+            dx = x2.similar() if need[1] else None
+            db = b.similar() if (need[2] and need[0]) else None
+            rc = lib.call("dense_back_%s" % w.suffix, 1 if act == "relu" else 0, m, n, k, w.ptr, x2.ptr, y.ptr, dy.ptr,
+                          dW.ptr if dW is not None else None, db.ptr if db is not None else None, dx.ptr if dx is not None else None)
+            if rc == 0:
+                return (dW.reshape(w.dims) if dW is not None else None, dx.reshape(x.dims) if dx is not None else None, db)
+            if rc < 0:
+                lib.check()
+                raise RuntimeError("dense_back failed")
         if act == "relu":
             dz, db = y.similar(), b.similar()
             knet8("reluback_biasgrad_%s" % w.suffix, m, n, dy.ptr, y.ptr, dz.ptr, db.ptr)

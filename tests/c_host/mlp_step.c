@@ -26,7 +26,7 @@ static void up(void *d, const void *h, size_t bytes) {
 }
 
 struct net {
-  float *W1, *b1, *W2, *b2, *x, *y1, *s, *dx, *lossv, *db2, *dW2, *dy1, *dz1, *db1, *dW1;
+  float *W1, *b1, *W2, *b2, *x, *y1, *s, *dx, *lossv, *db2, *dW2, *dy1, *db1, *dW1;
   int *labels;
 };
 
@@ -36,12 +36,12 @@ static void step(struct net *n, hipStream_t st) {
   gemm_bias_act_32_stream('N', 'N', D2, NB, D1, 1.0f, n->W2, D2, n->y1, D1, n->b2, 0, n->s, D2, st);
   /* loss and its gradient wrt the scores in one pass */
   nll_logsoftmax_back_32_stream(D2, NB, n->s, n->labels, 1.0f / NB, n->dx, n->lossv, st);
-  /* backward */
-  sum_32_21_stream(D2 * NB, n->dx, 1, D2, n->db2, st);                                              /* db2 = sum(dx; dims=2) */
-  gemm_32_stream('N', 'T', D2, D1, NB, 1.0f, n->dx, D2, n->y1, D1, 0.0f, n->dW2, D2, st);             /* dW2 = dx * y1'      */
-  gemm_32_stream('T', 'N', D1, NB, D2, 1.0f, n->W2, D2, n->dx, D2, 0.0f, n->dy1, D1, st);             /* dy1 = W2' * dx      */
-  reluback_biasgrad_32_stream(D1, NB, n->dy1, n->y1, n->dz1, n->db1, st);                             /* dz1, db1            */
-  gemm_32_stream('N', 'T', D1, D0, NB, 1.0f, n->dz1, D1, n->x, D0, 0.0f, n->dW1, D1, st);             /* dW1 = dz1 * x'      */
+  /* backward: one launch per layer (dense_back_32 returns 1 for layers too large for its kernel; these are not) */
+  if (dense_back_32_stream(0, D2, NB, D1, n->W2, n->y1, n->s, n->dx, n->dW2, n->db2, n->dy1, st) != 0 ||   /* dW2 = dx*y1', db2, dy1 = W2'*dx */
+      dense_back_32_stream(1, D1, NB, D0, n->W1, n->x, n->y1, n->dy1, n->dW1, n->db1, NULL, st) != 0) {    /* dz1 = relu'(y1).*dy1: dW1, db1  */
+    fprintf(stderr, "dense_back declined or failed\n");
+    exit(4);
+  }
 }
 
 int main(int argc, char **argv) {
@@ -58,7 +58,7 @@ int main(int argc, char **argv) {
   struct net n;
   n.W1 = dev(nW1); n.b1 = dev(D1); n.W2 = dev(nW2); n.b2 = dev(D2); n.x = dev(nx);
   n.y1 = dev(D1 * NB); n.s = dev(D2 * NB); n.dx = dev(D2 * NB); n.lossv = dev(NB);
-  n.db2 = dev(D2); n.dW2 = dev(nW2); n.dy1 = dev(D1 * NB); n.dz1 = dev(D1 * NB); n.db1 = dev(D1); n.dW1 = dev(nW1);
+  n.db2 = dev(D2); n.dW2 = dev(nW2); n.dy1 = dev(D1 * NB); n.db1 = dev(D1); n.dW1 = dev(nW1);
   n.labels = (int *)knet8_malloc(NB * sizeof(int));
   const float *p = h;
   up(n.W1, p, nW1 * 4); p += nW1;

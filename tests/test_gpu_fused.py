@@ -204,3 +204,45 @@ def test_dense_primitive_in_the_mlp_matches_oracle(knet, oracle):
     J = knet.diff(lambda: knet.nll(knet.dense(params[2], knet.dense(params[0], px, params[1], act="relu"), params[3]), labels, fused=True))
     assert knet.grad(J, px).dims == (28, 28, 1, 100)
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_dense_back_one_launch_per_layer(knet, dt):
+    """dense_back_S: dz = f'(y) .* dy on the fly, dW = dz*x', db = sum(dz;dims=2), dx = W'*dz in one launch, against numpy in fp64;
+    ragged tile edges, every combination of wanted outputs, both activations; large layers are declined (1), nothing written."""
+    rng = np.random.default_rng(45)
+    lib = knet.libknet8()
+    tol = 2e-5 if dt == np.float32 else 1e-12
+    for m, n, k in ((64, 100, 784), (10, 100, 64), (33, 65, 31), (1, 1, 1), (32, 32, 32), (100, 7, 300)):
+        W = rng.standard_normal((m, k)).astype(dt)
+        x = rng.standard_normal((k, n)).astype(dt)
+        y = rng.standard_normal((m, n)).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        Wd, xd, yd, dyd = (knet.KnetArray(v) for v in (W, x, y, dy))
+        for act in (0, 1):
+            dz = np.where(y > 0, dy, 0).astype(np.float64) if act == 1 else dy.astype(np.float64)
+            want = (dz @ x.astype(np.float64).T, dz.sum(axis=1), W.astype(np.float64).T @ dz)
+            for wantW, wantb, wantx in ((True, True, True), (True, True, False), (True, False, True), (False, False, True), (True, False, False)):
+                dW = knet.KnetArray(np.full((m, k), 7, dt)) if wantW else None
+                db = knet.KnetArray(np.full((m,), 7, dt)) if wantb else None
+                dx = knet.KnetArray(np.full((k, n), 7, dt)) if wantx else None
+                rc = lib.call("dense_back_%s" % Wd.suffix, act, m, n, k, Wd.ptr, xd.ptr, yd.ptr, dyd.ptr,
+                              dW.ptr if dW else None, db.ptr if db else None, dx.ptr if dx else None)
+                assert rc == 0
+                for got, w in ((dW, want[0]), (db, want[1]), (dx, want[2])):
+                    if got is not None:
+                        g = knet.Array(got)
+                        assert np.abs(g - w.reshape(g.shape)).max() <= tol * max(np.abs(w).max(), 1.0) * 4, (m, n, k, act)
+    # too large for the small kernels: declined, outputs untouched
+    m, n, k = 2048, 2048, 2048
+    big = knet.KnetArray(np.zeros((m, n), dt))
+    out = knet.KnetArray(np.full((m, n), 7, dt))
+    assert lib.call("dense_back_%s" % big.suffix, 0, m, n, k, big.ptr, big.ptr, big.ptr, big.ptr, out.ptr, None, None) == 1
+    assert np.all(knet.Array(out) == 7)
+    # db without dW: declined
+    small = knet.KnetArray(np.zeros((4, 4), dt))
+    assert lib.call("dense_back_%s" % small.suffix, 0, 4, 4, 4, small.ptr, small.ptr, small.ptr, small.ptr, None, small.ptr, None) == 1
+    assert lib.call("dense_back_%s" % small.suffix, 2, 4, 4, 4, small.ptr, small.ptr, small.ptr, small.ptr, small.ptr, None, None) == -1
+    with pytest.raises(RuntimeError):
+        lib.check()
+    lib.check()
