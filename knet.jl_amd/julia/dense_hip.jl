@@ -62,3 +62,19 @@ for (T, S) in ((Float32, 32), (Float64, 64))
         return y
     end
 end
+
+# The layer's whole backward pass in one call for small layers: dz = f'(y) .* dy on the fly, dw = dz*x', db = sum(dz;dims=2),
+# dx = w'*dz (dense_back_S).  Returns false when the library declines (a layer too large for its small-matrix kernels): the caller
+# then uses Fback_biasgrad_S and gemm! as before.
+for (T, S) in ((Float32, 32), (Float64, 64))
+    @eval function dense_back!(dw::KnetArray{$T,2}, db::KnetArray{$T}, dx::Union{KnetArray{$T,2},Nothing},
+                               w::KnetArray{$T,2}, x::KnetArray{$T,2}, y::KnetArray{$T,2}, dy::KnetArray{$T,2}; act::Integer=1)
+        m, k = size(w); n = size(x, 2)
+        @assert size(x, 1) == k && size(y) == (m, n) && size(dy) == (m, n) && size(dw) == (m, k) && length(db) == m
+        rc = ccall(($("dense_back_$(S)_stream"), LibKnet8.libknet8), Cint,
+                   (Cint, Cint, Cint, Cint, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{Cvoid}),
+                   act, m, n, k, w, x, y, dy, dw, db, dx === nothing ? C_NULL : dx, LibKnet8.knet8_stream())
+        rc < 0 && LibKnet8.knet8_check()
+        return rc == 0
+    end
+end
