@@ -69,9 +69,9 @@ __global__ __launch_bounds__(256) void dense_back_kernel(int act, int m, int n, 
         else       { As[lo][h] = ga[s][r]; Bs[lo][h] = gb[s][r]; }
       }
       __syncthreads();
-      if (sums && t < TS) {
-#pragma unroll 8
-        for (int kk = 0; kk < TS; kk++) rowsum = rowsum + As[kk][t];   // zero beyond n: adds nothing
+      if (sums) {   // all 256 lanes: lane (i = t % 32, part = t / 32) adds the four kk of its part; parts meet at the end
+#pragma unroll
+        for (int q = 0; q < TS / 8; q++) rowsum = rowsum + As[hi * (TS / 8) + q][lo];   // zero beyond n: adds nothing
       }
 #pragma unroll
       for (int kk = 0; kk < TS; kk++) {
@@ -89,7 +89,17 @@ __global__ __launch_bounds__(256) void dense_back_kernel(int act, int m, int n, 
       const int i = i0 + tx + 16 * a, j = j0 + ty + 16 * b;
       if (i < M && j < N) C[i + (long)j * M] = acc[a][b];
     }
-  if (sums && t < TS && i0 + t < m) db[i0 + t] = rowsum;
+  if (sums) {     // the eight parts of each row, in part order
+    T* part = &Bs[0][0];
+    part[hi * TS + lo] = rowsum;     // every lane is past its last read of Bs (barrier at the end of the loop)
+    __syncthreads();
+    if (t < TS && i0 + t < m) {
+      T r = T(0);
+#pragma unroll
+      for (int q = 0; q < 8; q++) r = r + part[q * TS + t];
+      db[i0 + t] = r;
+    }
+  }
 }
 
 // 0: done.  1: not applicable (a product too large for the small kernels, or db wanted without dW): nothing was launched and the

@@ -105,80 +105,86 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T 
 // arithmetic: three dependent memory round trips after the last product.  Here one wave owns the whole 32x32 tile for a slice
 // of k (4x4 outputs per lane) and the KS waves of a workgroup take KS slices; their partial tiles meet in LDS.  Every wave runs
 // the same number of k steps (loads beyond its slice or beyond k read zeros), so the workgroup barriers line up.
-template <typename T, bool TA, bool TB, int KS>
+// TS is the edge of a wave's output tile: 32 (4x4 outputs per lane) or 16 (2x2 per lane).  The small tile is for products with
+// so few 32x32 tiles and so long a k that even sixteen waves per tile leave most of the chip idle and each wave with a long serial
+// walk: four times the workgroups, a quarter of the arithmetic per wave.
+template <typename T, bool TA, bool TB, int KS, int TS = kGsTile>
 __global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda,
                                                               const T* __restrict__ B, int ldb, T beta, T* C, int ldc, const T* bias, int act, int kslice) {
-  __shared__ T As[KS][kGsTile][kGsTile + 1];  // As[w][kk][i] = op(A)(i0+i, k0+kk) of wave w's current step
-  __shared__ T Bs[KS][kGsTile][kGsTile + 1];
-  const int tiles_m = (m + kGsTile - 1) / kGsTile;
+  constexpr int KT = kGsTile;            // k elements per step
+  constexpr int Q = TS / 8;              // outputs per lane along each axis (lanes form an 8x8 grid)
+  constexpr int R = TS * KT / kWave;     // operand elements a lane stages per step
+  __shared__ T As[KS][KT][TS + 1];  // As[w][kk][i] = op(A)(i0+i, k0+kk) of wave w's current step
+  __shared__ T Bs[KS][KT][TS + 1];
+  const int tiles_m = (m + TS - 1) / TS;
   const int tile = blockIdx.x;
-  const int i0 = (tile % tiles_m) * kGsTile, j0 = (tile / tiles_m) * kGsTile;
+  const int i0 = (tile % tiles_m) * TS, j0 = (tile / tiles_m) * TS;
   const int w = threadIdx.x / kWave, l = threadIdx.x & (kWave - 1);
-  const int tx = l & 7, ty = l >> 3;  // outputs (tx + 8a, ty + 8b), a, b = 0..3
-  const int lo = l & 31, hi = l >> 5;  // loader coordinates: `lo` along the operand's contiguous axis
+  const int tx = l & 7, ty = l >> 3;  // outputs (tx + 8a, ty + 8b), a, b = 0..Q-1
+  // loader coordinates: `lo` runs along the operand's contiguous axis (TS long for the tile edge, KT long for k), `hi` across it
+  const int lo_t = l & (TS - 1), hi_t = l / TS;           // contiguous along the tile edge: kk = hi_t + (64/TS) r
+  const int lo_k = l & (KT - 1), hi_k = l / KT;           // contiguous along k: edge index = hi_k + (64/KT) r
   const int kbeg = w * kslice;
   int kend = kbeg + kslice;
   if (kend > k) kend = k;
-  T acc[4][4];
+  T acc[Q][Q];
 #pragma unroll
-  for (int a = 0; a < 4; a++)
+  for (int a = 0; a < Q; a++)
 #pragma unroll
-    for (int b = 0; b < 4; b++) acc[a][b] = T(0);
-  T ga[16], gb[16];
+    for (int b = 0; b < Q; b++) acc[a][b] = T(0);
+  T ga[R], gb[R];
   auto fetch = [&](int k0) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int h = hi + 2 * r;
-      if (!TA) { const int i = i0 + lo, kk = k0 + h; ga[r] = (i < m && kk < kend) ? A[i + (long)kk * lda] : T(0); }
-      else     { const int kk = k0 + lo, i = i0 + h; ga[r] = (i < m && kk < kend) ? A[kk + (long)i * lda] : T(0); }
-      if (!TB) { const int kk = k0 + lo, j = j0 + h; gb[r] = (j < n && kk < kend) ? B[kk + (long)j * ldb] : T(0); }
-      else     { const int j = j0 + lo, kk = k0 + h; gb[r] = (j < n && kk < kend) ? B[j + (long)kk * ldb] : T(0); }
+    for (int r = 0; r < R; r++) {
+      if (!TA) { const int i = i0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; ga[r] = (i < m && kk < kend) ? A[i + (long)kk * lda] : T(0); }
+      else     { const int kk = k0 + lo_k, i = i0 + hi_k + (kWave / KT) * r; ga[r] = (i < m && kk < kend) ? A[kk + (long)i * lda] : T(0); }
+      if (!TB) { const int kk = k0 + lo_k, j = j0 + hi_k + (kWave / KT) * r; gb[r] = (j < n && kk < kend) ? B[kk + (long)j * ldb] : T(0); }
+      else     { const int j = j0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; gb[r] = (j < n && kk < kend) ? B[j + (long)kk * ldb] : T(0); }
     }
   };
   fetch(kbeg);
-  for (int k0 = kbeg; k0 < kbeg + kslice; k0 += kGsTile) {
+  for (int k0 = kbeg; k0 < kbeg + kslice; k0 += KT) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int h = hi + 2 * r;
-      if (!TA) As[w][h][lo] = ga[r]; else As[w][lo][h] = ga[r];
-      if (!TB) Bs[w][lo][h] = gb[r]; else Bs[w][h][lo] = gb[r];
+    for (int r = 0; r < R; r++) {
+      if (!TA) As[w][hi_t + (kWave / TS) * r][lo_t] = ga[r]; else As[w][lo_k][hi_k + (kWave / KT) * r] = ga[r];
+      if (!TB) Bs[w][lo_k][hi_k + (kWave / KT) * r] = gb[r]; else Bs[w][hi_t + (kWave / TS) * r][lo_t] = gb[r];
     }
     __syncthreads();
-    if (k0 + kGsTile < kbeg + kslice) fetch(k0 + kGsTile);
+    if (k0 + KT < kbeg + kslice) fetch(k0 + KT);
 #pragma unroll 8
-    for (int kk = 0; kk < kGsTile; kk++) {
-      T av[4], bv[4];
+    for (int kk = 0; kk < KT; kk++) {
+      T av[Q], bv[Q];
 #pragma unroll
-      for (int a = 0; a < 4; a++) av[a] = As[w][kk][tx + 8 * a];
+      for (int a = 0; a < Q; a++) av[a] = As[w][kk][tx + 8 * a];
 #pragma unroll
-      for (int b = 0; b < 4; b++) bv[b] = Bs[w][kk][ty + 8 * b];
+      for (int b = 0; b < Q; b++) bv[b] = Bs[w][kk][ty + 8 * b];
 #pragma unroll
-      for (int a = 0; a < 4; a++)
+      for (int a = 0; a < Q; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) acc[a][b] = kfma(av[a], bv[b], acc[a][b]);
+        for (int b = 0; b < Q; b++) acc[a][b] = kfma(av[a], bv[b], acc[a][b]);
     }
     __syncthreads();
   }
   if (KS > 1) {
-    // partial tiles into LDS (each wave reuses its own staging area: 32*33 >= 1024 elements), summed in wave order
+    // partial tiles into LDS (each wave reuses its own staging area: KT*(TS+1) >= TS*TS elements), summed in wave order
     T* mine = &As[w][0][0];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < Q; a++)
 #pragma unroll
-      for (int b = 0; b < 4; b++) mine[(ty + 8 * b) * kGsTile + tx + 8 * a] = acc[a][b];
+      for (int b = 0; b < Q; b++) mine[(ty + 8 * b) * TS + tx + 8 * a] = acc[a][b];
     __syncthreads();
-    for (int o = threadIdx.x; o < kGsTile * kGsTile; o += KS * kWave) {
+    for (int o = threadIdx.x; o < TS * TS; o += KS * kWave) {
       T sum = T(0);
 #pragma unroll
       for (int q = 0; q < KS; q++) sum += (&As[q][0][0])[o];
-      const int i = i0 + (o & (kGsTile - 1)), j = j0 + o / kGsTile;
+      const int i = i0 + (o & (TS - 1)), j = j0 + o / TS;
       if (i < m && j < n) gemm_store(C + i + (long)j * ldc, sum, alpha, beta, bias, i, act);
     }
   } else {
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < Q; a++)
 #pragma unroll
-      for (int b = 0; b < 4; b++) {
+      for (int b = 0; b < Q; b++) {
         const int i = i0 + tx + 8 * a, j = j0 + ty + 8 * b;
         if (i < m && j < n) gemm_store(C + i + (long)j * ldc, acc[a][b], alpha, beta, bias, i, act);
       }
@@ -193,6 +199,22 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
                               T beta, T* C, int ldc, const T* bias = nullptr, int act = 0) {
   const long tiles = (long)((m + kGsTile - 1) / kGsTile) * ((n + kGsTile - 1) / kGsTile);
   const long ksteps = (k + kGsTile - 1) / kGsTile;
+  if (ksteps >= 8 && tiles < 16 && tuning(kTuneGemmWaveTiles) != 1) {
+    // Few tiles, long k (the first layer of the MNIST MLP, 64x100x784): the cross-workgroup split below pays three dependent
+    // memory round trips for its combine, sixteen waves on a 32x32 tile are bound by one CU's LDS.  16x16 tiles, sixteen k slices
+    // per workgroup, partial tiles combined in LDS.
+    constexpr int kKs = sizeof(T) == 4 ? 16 : 8;
+    const int kslice = (int)((ksteps + kKs - 1) / kKs) * kGsTile;
+    const long tiles16 = (long)((m + 15) / 16) * ((n + 15) / 16);
+    const dim3 grid16((unsigned)tiles16);
+#define KNET8_GW16(TA, TB) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, kKs, 16>), grid16, dim3(kKs * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
+    if (!ta && !tb) KNET8_GW16(false, false);
+    else if (ta && !tb) KNET8_GW16(true, false);
+    else if (!ta && tb) KNET8_GW16(false, true);
+    else KNET8_GW16(true, true);
+#undef KNET8_GW16
+    return;
+  }
   if (ksteps >= 4 && tiles >= 16 && tiles <= tuning(kTuneGemmWaveTiles)) {
     // Enough tiles to occupy a fair share of the CUs and a k long enough that walking it serially would dominate: one wave per k
     // slice inside the workgroup, no cross-workgroup combine.  Measured (us per call, back-to-back launches, this kernel vs the

@@ -164,8 +164,10 @@ def test_allocator_pool(knet):
 def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
     rng = np.random.default_rng(54)
     rtol = 1e-5 if dt == np.float32 else 1e-13
-    # the small-product kernels: cross-workgroup k split (few tiles), k slices inside a workgroup (16+ tiles, k >= 97), plain tiles
-    for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000), (130, 131, 129), (512, 300, 256), (256, 300, 96), (100, 500, 97)]:
+    # the small-product kernels: 16x16 tiles with k slices inside a workgroup (few tiles, k >= 225), cross-workgroup k split (few tiles,
+    # shorter k), k slices inside a workgroup on 32x32 tiles (16+ tiles, k >= 97), plain tiles
+    for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000), (130, 131, 129), (512, 300, 256), (256, 300, 96), (100, 500, 97),
+                      (10, 100, 500), (33, 17, 300), (1, 1, 1000), (17, 95, 225), (64, 100, 200)]:
         A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
         want = oracle.gemm(A, B)
         Ad, Bd, Atd, Btd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.ascontiguousarray(A.T)), knet.KnetArray(np.ascontiguousarray(B.T))
