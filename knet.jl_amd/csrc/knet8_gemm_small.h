@@ -199,20 +199,26 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
                               T beta, T* C, int ldc, const T* bias = nullptr, int act = 0) {
   const long tiles = (long)((m + kGsTile - 1) / kGsTile) * ((n + kGsTile - 1) / kGsTile);
   const long ksteps = (k + kGsTile - 1) / kGsTile;
-  if (ksteps >= 8 && tiles < 16 && tuning(kTuneGemmWaveTiles) != 1) {
-    // Few tiles, long k (the first layer of the MNIST MLP, 64x100x784): the cross-workgroup split below pays three dependent
-    // memory round trips for its combine, sixteen waves on a 32x32 tile are bound by one CU's LDS.  16x16 tiles, sixteen k slices
-    // per workgroup, partial tiles combined in LDS.
-    constexpr int kKs = sizeof(T) == 4 ? 16 : 8;
-    const int kslice = (int)((ksteps + kKs - 1) / kKs) * kGsTile;
-    const long tiles16 = (long)((m + 15) / 16) * ((n + 15) / 16);
+  const long tiles16 = (long)((m + 15) / 16) * ((n + 15) / 16);
+  if (tiles16 * ksteps <= 4096 && tuning(kTuneGemmWaveTiles) != 1) {
+    // The smaller products (up to about 7e7 flop): 16x16 tiles, one wave per tile and k slice, as many slices per workgroup as there
+    // are 32-deep steps (up to 16), partial tiles combined in LDS -- every load of the product is in flight at once and no combine
+    // leaves the workgroup.  Measured (us per call, back-to-back launches; this path vs the 32x32-tile paths below):
+    // 64x100x784 7.6/12.1, 10x100x64 3.8/5.3, 64x784x100 NT 4.1/6.1, 128^3 3.9/6.1, 256^3 4.2/6.4, 300^3 7.5/9.6, 256x300x512 TN 7.7/10.1,
+    // 1000x10x1000 7.8/15.5, 64x4096x100 5.2/6.7; from about 1e8 flop (512x512x190: 7.8/6.9) the larger tiles win.
+    int ks = 1;
+    while (ks < 16 && ks < ksteps) ks *= 2;
+    const int kslice = (int)((ksteps + ks - 1) / ks) * kGsTile;
     const dim3 grid16((unsigned)tiles16);
-#define KNET8_GW16(TA, TB) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, kKs, 16>), grid16, dim3(kKs * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
+#define KNET8_GW16K(TA, TB, KSX) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KSX, 16>), grid16, dim3(KSX * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
+#define KNET8_GW16(TA, TB) do { if (ks == 1) KNET8_GW16K(TA, TB, 1); else if (ks == 2) KNET8_GW16K(TA, TB, 2); else if (ks == 4) KNET8_GW16K(TA, TB, 4); \
+                                else if (ks == 8) KNET8_GW16K(TA, TB, 8); else KNET8_GW16K(TA, TB, 16); } while (0)
     if (!ta && !tb) KNET8_GW16(false, false);
     else if (ta && !tb) KNET8_GW16(true, false);
     else if (!ta && tb) KNET8_GW16(false, true);
     else KNET8_GW16(true, true);
 #undef KNET8_GW16
+#undef KNET8_GW16K
     return;
   }
   if (ksteps >= 4 && tiles >= 16 && tiles <= tuning(kTuneGemmWaveTiles)) {
