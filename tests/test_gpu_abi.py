@@ -164,10 +164,12 @@ def test_allocator_pool(knet):
 def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
     rng = np.random.default_rng(54)
     rtol = 1e-5 if dt == np.float32 else 1e-13
-    # the small-product kernels: 16x16 tiles with k slices inside a workgroup (few tiles, k >= 225), cross-workgroup k split (few tiles,
-    # shorter k), k slices inside a workgroup on 32x32 tiles (16+ tiles, k >= 97), plain tiles
+    # the small-product kernels: 16x16 tiles with k slices inside a workgroup (up to about 7e7 flop), above that 32x32 tiles with k
+    # slices inside a workgroup (16+ tiles) or the cross-workgroup k split (fewer tiles)
     for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000), (130, 131, 129), (512, 300, 256), (256, 300, 96), (100, 500, 97),
-                      (10, 100, 500), (33, 17, 300), (1, 1, 1000), (17, 95, 225), (64, 100, 200)]:
+                      (10, 100, 500), (33, 17, 300), (1, 1, 1000), (17, 95, 225), (64, 100, 200),
+                      (64, 64, 10000), (40, 33, 9000),      # few tiles, very long k: the cross-workgroup k split with its ticket
+                      (512, 512, 190), (700, 300, 200)]:    # near the upper end of the small-product range: 32x32 wave tiles
         A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
         want = oracle.gemm(A, B)
         Ad, Bd, Atd, Btd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.ascontiguousarray(A.T)), knet.KnetArray(np.ascontiguousarray(B.T))
