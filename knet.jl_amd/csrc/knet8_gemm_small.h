@@ -1,10 +1,15 @@
 // Small-matrix GEMM C = alpha*op(A)*op(B) + beta*C (column-major), for products far too small to fill the
-// machine -- the 64x100x784-class products of the MNIST MLP, where the vendor library needs 15-25 us per call and
-// a whole captured training step is otherwise ~80 us.  Large products go to hipBLASLt (knet8_runtime.hip).
-//
-// 32x32 output tile per 256-lane workgroup (2x2 outputs per lane), k walked in steps of 32 through LDS; when the
-// tiles alone would leave most CUs idle the k range is split over P workgroups per tile whose partial tiles are
-// combined, in fixed order, by the last one to finish (same write-through + ticket scheme as the reductions).
+// machine -- the 64x100x784-class products of the MNIST MLP, where the vendor library needs 15-25 us per call.  Large products
+// go to hipBLASLt (knet8_runtime.hip).  At this size a product's time is one launch (3.2 us for an empty kernel), one memory round
+// trip and a few 32-deep tile steps: what matters is how many steps run one after the other and whether partial results have to
+// leave the workgroup.  Three kernels, chosen in launch_gemm_small:
+//   * gemm_wave_kernel<.., KS, 16>: 16x16 output tile per workgroup, one wave per k slice (KS = 1..16 slices), partial tiles summed
+//     in LDS -- everything up to about 7e7 flop;
+//   * gemm_wave_kernel<.., KS, 32>: the same with 32x32 tiles (4x4 outputs per lane) for the upper end of the range, when there are
+//     at least 16 such tiles;
+//   * gemm_small_kernel: 32x32 tile per 256-lane workgroup, k split over P workgroups per tile whose partial tiles are combined, in
+//     fixed order, by the last one to finish (write-through + ticket, as in the reductions) -- few tiles with a very long k.
+// All three add the bias and apply relu in their output stage when asked (gemm_bias_act_S): same bits as separate launches.
 #pragma once
 #include "knet8_device.h"
 #include "knet8_runtime.h"
