@@ -197,7 +197,12 @@ __global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int
 }
 
 // True if this product should use the small kernel.
-inline bool gemm_is_small(int m, int n, int k) { return 2.0 * m * n * (double)k <= 1.0e8 && (long)m * n <= 262144; }
+// hipBLASLt has a floor of about 12 us per call on this chip; the kernels here stay below it up to about 1e8 flop in general and
+// 2.7e8 flop when k <= 512 (512^3: 10.4 vs 12.0 us; 256x256x2048: 28 vs 12.6 us -- long k runs serially inside a wave).
+inline bool gemm_is_small(int m, int n, int k) {
+  const double flop = 2.0 * m * n * (double)k, limit = 1.0e6 * tuning(kTuneGemmSmallMflop);
+  return (flop <= limit || (flop <= 2.7 * limit && k <= 512)) && (long)m * n <= 262144;
+}
 
 template <typename T>
 inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb,
