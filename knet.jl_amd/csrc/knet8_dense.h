@@ -7,7 +7,7 @@
 // workgroups of one grid split into two jobs: 16x16 tiles of dW = dz*x' (the tiles of the first block column also add up the rows
 // of dz they walk: db) and 16x16 tiles of dx = W'*dz.  dz is never written.  Sums run in a fixed order: deterministic results;
 // against the separate launches they differ only in the order of summation.
-// Only for products the small-matrix GEMM would take (gemm_is_small); larger layers keep the separate launches.
+// Only for layers of up to about 6e7 flop per product; larger ones keep the separate launches (the entry point returns 1).
 #pragma once
 #include "knet8_device.h"
 #include "knet8_gemm_small.h"
@@ -122,7 +122,9 @@ inline int launch_dense_back(hipStream_t stream, int act, int m, int n, int k, c
     record_error("dense_back: missing operand");
     return -1;
   }
-  if (!gemm_is_small(m, k, n) || !gemm_is_small(k, n, m) || (db != nullptr && dW == nullptr)) return 1;
+  // both products have 2*m*n*k flop; measured against reluback_biasgrad + two gemm launches (us): 64x100x784 5.6/14.5, 256^3 8.4/14.5,
+  // 300^3 12.5/21.6, 512x128x512 16.4/16.2, 512^3 32.5/27.4 -- one launch wins up to about 6e7 flop
+  if (2.0 * m * n * (double)k > 6.0e7 || (long)m * k > 262144 || (long)k * n > 262144 || (db != nullptr && dW == nullptr)) return 1;
   const int tw_m = (m + kDbTile - 1) / kDbTile, tw_n = (k + kDbTile - 1) / kDbTile;
   const int tx_m = (k + kDbTile - 1) / kDbTile, tx_n = (n + kDbTile - 1) / kDbTile;
   const int tiles_w = dW ? tw_m * tw_n : 0, tiles_x = dx ? tx_m * tx_n : 0;
