@@ -1,7 +1,7 @@
 /* A compiled host driving the C ABI directly, the way Knet's Julia code does through ccall: one forward + backward step of the
  * MLP of examples/mnist-mlp/mlp.jl:25-35 (784-64-10, batch 100), every device operation an entry point of knet8.h.
  *
- *   mlp_step IN OUT [steps]
+ *   mlp_step IN OUT [steps]        (IN may be "@random")
  *
  * IN holds, as raw little-endian data in this order: float W1[64*784], b1[64], W2[10*64], b2[10], x[784*100] (all column-major),
  * int32 labels[100] (1-based).  OUT receives float loss, dW1[64*784], db1[64], dW2[10*64], db2[10].  With `steps` the step is then
@@ -51,9 +51,16 @@ int main(int argc, char **argv) {
   const size_t nin = nW1 + D1 + nW2 + D2 + nx;
   float *h = (float *)malloc(nin * sizeof(float));
   int hl[NB];
-  FILE *f = fopen(argv[1], "rb");
-  if (!f || fread(h, sizeof(float), nin, f) != nin || fread(hl, sizeof(int), NB, f) != NB) { fprintf(stderr, "cannot read %s\n", argv[1]); return 2; }
-  fclose(f);
+  FILE *f = NULL;
+  if (argv[1][0] == '@') { /* "@random": inputs from a fixed linear congruential sequence, for profiling runs without an input file */
+    unsigned long long sd = 88172645463325252ULL;
+    for (size_t i = 0; i < nin; i++) { sd = sd * 6364136223846793005ULL + 1442695040888963407ULL; h[i] = ((float)(sd >> 40) / 16777216.0f - 0.5f) * 0.1f; }
+    for (int i = 0; i < NB; i++) { sd = sd * 6364136223846793005ULL + 1442695040888963407ULL; hl[i] = 1 + (int)((sd >> 33) % D2); }
+  } else {
+    f = fopen(argv[1], "rb");
+    if (!f || fread(h, sizeof(float), nin, f) != nin || fread(hl, sizeof(int), NB, f) != NB) { fprintf(stderr, "cannot read %s\n", argv[1]); return 2; }
+    fclose(f);
+  }
   if (knet8_device_count() < 1) { fprintf(stderr, "no device\n"); return 3; }
   struct net n;
   n.W1 = dev(nW1); n.b1 = dev(D1); n.W2 = dev(nW2); n.b2 = dev(D2); n.x = dev(nx);
