@@ -23,7 +23,7 @@ from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_,
                        getindex, setindex_)
 from .dropout import dropout, dropback, dropout_, dropback_
 from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, update_, gclip_
-from .linalg import dense, matmul, mat, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
+from .linalg import dense, matmul, mat, bmm, bmm_, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
 
 libknet8()  # fail loudly at import time if the HIP library is missing
 

@@ -646,6 +646,12 @@ KNET8_API int gemm_32_stream(char transa, char transb, int m, int n, int k, floa
 KNET8_API int gemm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float beta, float* C, int ldc);
 KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc, hipStream_t stream);
 KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta, double* C, int ldc);
+/* replaces cublasSgemmStridedBatched / cublasDgemmStridedBatched at src/ops20_gpu/bmm.jl:46-50 (bmm!): product b of the batch uses
+   A + b*strideA, B + b*strideB, C + b*strideC (strides in elements); hipBLASLt strided batch */
+KNET8_API int bmm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, long long strideA, float* B, int ldb, long long strideB, float beta, float* C, int ldc, long long strideC, int batch, hipStream_t stream);
+KNET8_API int bmm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, long long strideA, float* B, int ldb, long long strideB, float beta, float* C, int ldc, long long strideC, int batch);
+KNET8_API int bmm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, long long strideA, double* B, int ldb, long long strideB, double beta, double* C, int ldc, long long strideC, int batch, hipStream_t stream);
+KNET8_API int bmm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, long long strideA, double* B, int ldb, long long strideB, double beta, double* C, int ldc, long long strideC, int batch);
 /* dense layer in one call: C = act(alpha*op(A)*op(B) + bias[i]) with bias of length m and act 0 (none) or 1 (relu).  No counterpart in
    the reference, which runs gemm!, the bias broadcast (src/knetarrays/binary.jl:61-95) and relu (src/ops20_gpu/activation.jl:17-29) as
    three launches; same bits as that chain.  Small products fold bias and relu into the product kernel's output stage. */

@@ -440,10 +440,16 @@ KNET8_API int knet8_tune(int key, int value) {
 // ---- GEMM through hipBLASLt ----------------------------------------------------------------------------------
 namespace knet8 {
 
+struct GemmBatch {   // strided batch: product b uses A + b*sa, B + b*sb, C + b*sc (elements)
+  int count = 1;
+  long long sa = 0, sb = 0, sc = 0;
+};
 struct GemmKey {
-  int dev, dtype, ta, tb, m, n, k, lda, ldb, ldc;
+  int dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch;
+  long long sa, sb, sc;
   bool operator<(const GemmKey& o) const {
-    return std::tie(dev, dtype, ta, tb, m, n, k, lda, ldb, ldc) < std::tie(o.dev, o.dtype, o.ta, o.tb, o.m, o.n, o.k, o.lda, o.ldb, o.ldc);
+    return std::tie(dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch, sa, sb, sc) <
+           std::tie(o.dev, o.dtype, o.ta, o.tb, o.m, o.n, o.k, o.lda, o.ldb, o.ldc, o.batch, o.sa, o.sb, o.sc);
   }
 };
 struct GemmPlan {
@@ -474,11 +480,12 @@ struct EpiRelu { template <typename T> __device__ __forceinline__ T operator()(T
 
 template <typename T>
 static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
-                hipStream_t stream, const T* bias = nullptr, int act = 0) {
-  if (m <= 0 || n <= 0) return 0;
+                hipStream_t stream, const T* bias = nullptr, int act = 0, GemmBatch batch = GemmBatch()) {
+  if (m <= 0 || n <= 0 || batch.count <= 0) return 0;
   const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
   const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
-  if (gemm_is_small(m, n, k)) {
+  if (batch.count > 1 && (bias || act)) { record_error("gemm: the bias/activation form takes no batch"); return -1; }
+  if (batch.count == 1 && gemm_is_small(m, n, k)) {
     launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act);
     check_launch("gemm (small)");
     return 0;
@@ -506,7 +513,7 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   if (!h && !lt_ok(hipblasLtCreate(&h), "create")) return -1;
   void*& ws = g_gemm_ws[std::make_pair(dev, stream)];
   if (!ws && !ok(hipMalloc(&ws, kGemmWorkspace), "hipMalloc(gemm workspace)")) return -1;
-  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc};
+  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, batch.sa, batch.sb, batch.sc};
   GemmPlan& p = g_plans[key];
   if (!p.valid) {
     const hipblasOperation_t opa = ta ? HIPBLAS_OP_T : HIPBLAS_OP_N, opb = tb ? HIPBLAS_OP_T : HIPBLAS_OP_N;
@@ -516,6 +523,15 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
     if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.la, dt, ta ? k : m, ta ? m : k, lda), "layout A")) return -1;
     if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lb, dt, tb ? n : k, tb ? k : n, ldb), "layout B")) return -1;
     if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lc, dt, m, n, ldc), "layout C")) return -1;
+    if (batch.count > 1) {
+      const int32_t bc = batch.count;
+      const int64_t st[3] = {batch.sa, batch.sb, batch.sc};
+      hipblasLtMatrixLayout_t lay[3] = {p.la, p.lb, p.lc};
+      for (int q = 0; q < 3; q++) {
+        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &bc, sizeof(bc)), "batch count")) return -1;
+        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &st[q], sizeof(st[q])), "batch stride")) return -1;
+      }
+    }
     hipblasLtMatmulPreference_t pref = nullptr;
     if (!lt_ok(hipblasLtMatmulPreferenceCreate(&pref), "pref create")) return -1;
     size_t wsbytes = kGemmWorkspace;
@@ -565,6 +581,24 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   return lt_ok(hipblasLtMatmul(h, p.desc, &alpha, A, p.la, B, p.lb, &beta, C, p.lc, C, p.lc, &p.algo, ws, kGemmWorkspace, stream), "matmul") ? 0 : -1;
 }
 
+
+// Strided batch of products C_b = alpha*op(A_b)*op(B_b) + beta*C_b, b = 0..batch-1, operand b at base + b*stride (elements).
+template <typename T>
+static int bmm_entry(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, long long sa, const T* B, int ldb, long long sb, T beta,
+                     T* C, int ldc, long long sc, int batch, hipStream_t stream) {
+  if (batch < 0 || sa < 0 || sb < 0 || sc < 0) { record_error("bmm: negative batch count or stride"); return -1; }
+  if (batch <= 1 || k <= 0) {   // nothing to batch, or empty products (C = beta*C): the plain entry handles both
+    for (int b = 0; b < batch; b++) {
+      const int rc = gemm<T>(transa, transb, m, n, k, alpha, A + b * sa, lda, B + b * sb, ldb, beta, C + b * sc, ldc, stream);
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
+  GemmBatch gb;
+  gb.count = batch; gb.sa = sa; gb.sb = sb; gb.sc = sc;
+  return gemm<T>(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, 0, gb);
+}
+
 }  // namespace knet8
 
 extern "C" {
@@ -583,6 +617,23 @@ KNET8_API int gemm_64_stream(char transa, char transb, int m, int n, int k, doub
 KNET8_API int gemm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double beta,
                       double* C, int ldc) {
   return gemm_64_stream(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, 0);
+}
+
+KNET8_API int bmm_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, long long strideA, float* B, int ldb,
+                            long long strideB, float beta, float* C, int ldc, long long strideC, int batch, hipStream_t stream) {
+  return knet8::bmm_entry<float>(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, stream);
+}
+KNET8_API int bmm_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, long long strideA, float* B, int ldb, long long strideB,
+                     float beta, float* C, int ldc, long long strideC, int batch) {
+  return bmm_32_stream(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, 0);
+}
+KNET8_API int bmm_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, long long strideA, double* B, int ldb,
+                            long long strideB, double beta, double* C, int ldc, long long strideC, int batch, hipStream_t stream) {
+  return knet8::bmm_entry<double>(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, stream);
+}
+KNET8_API int bmm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, long long strideA, double* B, int ldb, long long strideB,
+                     double beta, double* C, int ldc, long long strideC, int batch) {
+  return bmm_64_stream(transa, transb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, 0);
 }
 
 static int check_epilogue(int act) {

@@ -17,7 +17,7 @@ LIB_PATH = os.environ.get("KNET8_LIBRARY", os.path.join(_PKG, "lib", "libknet8.s
 HEADER_PATH = os.path.join(_ROOT, "include", "knet8.h")
 
 _CTYPES = {
-    "void": None, "int": ctypes.c_int, "unsigned long long": ctypes.c_ulonglong, "float": ctypes.c_float, "double": ctypes.c_double, "char": ctypes.c_char,
+    "void": None, "int": ctypes.c_int, "unsigned long long": ctypes.c_ulonglong, "long long": ctypes.c_longlong, "float": ctypes.c_float, "double": ctypes.c_double, "char": ctypes.c_char,
     "size_t": ctypes.c_size_t, "hipStream_t": ctypes.c_void_p, "float*": ctypes.c_void_p, "double*": ctypes.c_void_p,
     "int*": ctypes.c_void_p, "const int*": ctypes.c_void_p, "void*": ctypes.c_void_p, "const void*": ctypes.c_void_p, "size_t*": ctypes.c_void_p, "unsigned long long*": ctypes.c_void_p,
     "const char*": ctypes.c_char_p, "float**": ctypes.c_void_p, "double**": ctypes.c_void_p,

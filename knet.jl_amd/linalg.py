@@ -95,6 +95,62 @@ def dense(w, x, b, act=None):
     return y, selective(back)
 
 
+def bmm_(transA, transB, alpha, A, B, beta, C):
+    """``bmm!(transA, transB, alpha, A, B, beta, C)`` on 3-d arrays (src/ops20_gpu/bmm.jl:16-53): one strided-batch launch
+    (``bmm_S``, cublasXgemmStridedBatched in the reference), the same shape checks and DimensionMismatch errors."""
+    if A.ndims != 3 or B.ndims != 3 or C.ndims != 3:
+        raise ValueError("DimensionMismatch: %r" % ((A.dims, B.dims, C.dims),))
+    if transA not in ("N", "T", "C") or transB not in ("N", "T", "C"):
+        raise ValueError("Unknown cublas op %r" % ((transA, transB),))
+    (ma, ka, bsa), (kb, nb, bsb) = A.dims, B.dims
+    m, k = (ma, ka) if transA == "N" else (ka, ma)
+    n, kk = (nb, kb) if transB == "N" else (kb, nb)
+    if bsa != bsb or k != kk or C.dims != (m, n, bsa):
+        raise ValueError("DimensionMismatch: %r" % ((A.dims, B.dims, C.dims),))
+    if A.dtype != B.dtype or A.dtype != C.dtype:
+        raise TypeError("MethodError: element types differ")
+    c = A.ctype
+    lib = libknet8()
+    rc = lib.call("bmm_%s" % A.suffix, transA.encode(), transB.encode(), m, n, k, c(alpha), A.ptr, max(ma, 1), ma * ka, B.ptr, max(kb, 1), kb * nb,
+                  c(beta), C.ptr, max(m, 1), m * n, bsa)
+    if rc != 0:
+        lib.check()
+        raise RuntimeError("bmm failed")
+    return C
+
+
+def _bmm(A, B, transA=False, transB=False):
+    sa, sb = A.dims, B.dims
+    if len(sa) < 2 or len(sb) < 2:
+        raise ValueError("DimensionMismatch: %r" % ((sa, sb),))
+    m, k = (sa[1], sa[0]) if transA else (sa[0], sa[1])
+    kb, n = (sb[1], sb[0]) if transB else (sb[0], sb[1])
+    if kb != k or sa[2:] != sb[2:]:
+        raise AssertionError("bmm: kb == k && sa[3:end] == sb[3:end]: %r" % ((sa, sb),))
+    nb = 1
+    for d in sa[2:]:
+        nb *= d
+    a3, b3 = A.reshape(sa[0], sa[1], nb), B.reshape(sb[0], sb[1], nb)
+    C = bmm_("T" if transA else "N", "T" if transB else "N", 1, a3, b3, 0, A.similar((m, n, nb)))
+    return C.reshape(*((m, n) + tuple(sb[2:])))
+
+
+@primitive
+def bmm(A, B, transA=False, transB=False):
+    """``bmm(A, B; transA=false, transB=false)``: batch of matrix products over the trailing dimensions: (m,k,b...) x (k,n,b...) ->
+    (m,n,b...) (src/ops20/bmm.jl:7-25); gradients as the reference's ``@primitive1`` line states them (``:76``)."""
+    y = _bmm(A, B, transA, transB)
+
+    def back(dy, need=(True, True)):
+        dA = dB = None
+        if need[0]:
+            dA = _bmm(B, dy, transA=transB, transB=True) if transA else _bmm(dy, B, transA=False, transB=not transB)
+        if need[1]:
+            dB = _bmm(dy, A, transA=True, transB=transA) if transB else _bmm(A, dy, transA=not transA, transB=False)
+        return dA, dB
+    return y, selective(back)
+
+
 @primitive
 def mat(x, dims=None):
     """``mat(x; dims=ndims(x)-1)``: reshape to a matrix whose rows are the first ``dims`` dimensions (src/ops20/conv.jl:222; the MLP example

@@ -72,8 +72,8 @@ def test_every_entry_point_is_a_no_op_on_empty_arrays(knet):
     a = knet.KnetArray(np.full(64, 3.0, np.float64))
     count = 0
     for name, (ret, args) in sorted(lib.decls.items()):
-        if name.endswith("_stream") or name.startswith(("knet8_", "gemm_", "permutedims")):
-            continue      # runtime calls; gemm takes transpose characters; permutedims rejects ndims = 0 by design
+        if name.endswith("_stream") or name.startswith(("knet8_", "gemm_", "bmm_", "permutedims")):
+            continue      # runtime calls; gemm and bmm take transpose characters; permutedims rejects ndims = 0 by design
         vals = []
         for t in args:
             if t == "int":
