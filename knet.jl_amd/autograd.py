@@ -27,6 +27,7 @@ class Param:
 
     def __init__(self, value):
         self.value = value
+        self.opt = None   # the optimizer `minimize` attaches (src/train20/train.jl:23-25); set beforehand to override it
 
     def __repr__(self):
         return "P(%r)" % (self.value,)
@@ -108,8 +109,8 @@ def addto(a, b):
 class Result:
     """What ``@diff`` returns: the value plus the gradients of every Param that took part."""
 
-    def __init__(self, value, grads):
-        self.value, self.grads = value, grads
+    def __init__(self, value, grads, params=()):
+        self.value, self.grads, self.params = value, grads, tuple(params)   # params: in order of first use (AutoGrad's params(J))
 
 
 def diff(f):
@@ -150,7 +151,7 @@ def diff(f):
             node.back = None
             if node is not out:
                 node.value = None
-    return Result(v, {pid: n.outgrad for pid, n in tape.leaves.items()})
+    return Result(v, {pid: n.outgrad for pid, n in tape.leaves.items()}, [n.param for n in tape.leaves.values()])
 
 
 def grad(result, param):

@@ -52,7 +52,7 @@ def _vector_dim(small, big):
 def broadcast_op(name, x, y):
     """``x .op y`` for KnetArray/number operands."""
     if not isinstance(x, KnetArray) and not isinstance(y, KnetArray):
-        raise TypeError("broadcast_op needs at least one KnetArray")
+        return _scalar_scalar(name, x, y)
     if not isinstance(x, KnetArray):
         return _scalar_array(name, x, y, True)
     if not isinstance(y, KnetArray):
@@ -73,6 +73,17 @@ def broadcast_op(name, x, y):
         knet8("%s_%s_12" % (name, x.suffix), z.length, x.ptr, vx[0], vx[1], y.ptr, 1, y.length, z.ptr)
         return z
     return _broadcast_nd(name, x, y)
+
+
+def _scalar_scalar(name, x, y):
+    """Two host numbers (a loss value divided by a count, say): plain host arithmetic in the type numpy promotes to, so that an
+    fp32 scalar stays fp32 against a Python number, as a Float32 does against an Int in the reference."""
+    import operator
+    if name not in ("add", "sub", "mul", "div"):
+        raise TypeError("MethodError: %s of two numbers is not provided" % name)
+    if not isinstance(x, (int, float, np.number)) or not isinstance(y, (int, float, np.number)):
+        raise TypeError("MethodError: no method matching %s(::%s, ::%s)" % (name, type(x).__name__, type(y).__name__))
+    return {"add": operator.add, "sub": operator.sub, "mul": operator.mul, "div": operator.truediv}[name](x, y)
 
 
 def _broadcast_nd(name, x, y):
@@ -128,7 +139,7 @@ def _squeeze(dims):
 def unbroadcast(x, dx):
     """Gradient of a broadcast operand: ``x`` is the operand as passed, ``dx`` the gradient of the result."""
     if not isinstance(x, KnetArray):
-        return ksum(dx)  # x is a Number: sum(dx)
+        return ksum(dx) if isinstance(dx, KnetArray) else dx  # x is a Number: sum(dx)
     if not isinstance(dx, KnetArray):
         return dx
     nd = max(x.ndims, dx.ndims)

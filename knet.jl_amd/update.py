@@ -74,8 +74,19 @@ def gclip_(g, gclip):
     return g
 
 
-def update_(w, g, p):
-    """``update!(w, g, p)``: one in-place step of optimizer ``p`` on the weight array ``w`` with gradient ``g``."""
+def update_(w, g, p=None, lr=0.1, gclip=0):
+    """``update!(w, g, p)``: one in-place step of optimizer ``p`` on the weight array ``w`` with gradient ``g``.
+    ``update!(x::Param, g)`` uses the parameter's own optimizer ``x.opt``; without any optimizer the step is SGD with
+    ``lr`` and ``gclip`` (src/train20/update.jl:470-476); a gradient of ``None`` (the parameter took no part) changes nothing."""
+    from .autograd import Param
+    if isinstance(w, Param):
+        if p is None:
+            p = w.opt
+        w = w.value
+    if g is None:
+        return w
+    if p is None:
+        p = SGD(lr, gclip)
     if not isinstance(w, KnetArray) or not isinstance(g, KnetArray):
         raise TypeError("MethodError: update! needs KnetArray weights and gradients")
     if w.length != g.length or w.dtype != g.dtype:
