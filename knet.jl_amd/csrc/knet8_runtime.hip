@@ -457,7 +457,8 @@ struct GemmPlan {
   hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
-  bool valid = false;
+  bool valid = false;   // descriptors and an algorithm exist
+  bool timed = false;   // the algorithm was chosen by timing the candidates (not possible while the stream is being captured)
 };
 static std::mutex g_gemm_mutex;
 static std::map<int, hipblasLtHandle_t> g_lt;
@@ -515,7 +516,10 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   if (!ws && !ok(hipMalloc(&ws, kGemmWorkspace), "hipMalloc(gemm workspace)")) return -1;
   const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, batch.sa, batch.sb, batch.sc};
   GemmPlan& p = g_plans[key];
-  if (!p.valid) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (stream) (void)hipStreamIsCapturing(stream, &cap);
+  const bool capturing = cap != hipStreamCaptureStatusNone;
+  if (!p.desc) {
     const hipblasOperation_t opa = ta ? HIPBLAS_OP_T : HIPBLAS_OP_N, opb = tb ? HIPBLAS_OP_T : HIPBLAS_OP_N;
     if (!lt_ok(hipblasLtMatmulDescCreate(&p.desc, ct, dt), "desc create")) return -1;
     if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &opa, sizeof(opa)), "set transa")) return -1;
@@ -532,6 +536,11 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
         if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &st[q], sizeof(st[q])), "batch stride")) return -1;
       }
     }
+  }
+  // Choose the algorithm: at the first call, and again at the first call that is allowed to time the candidates if the earlier
+  // choice had to be made without (a stream under capture cannot be synchronised; a call with beta != 0 would accumulate into C).
+  const bool can_time = !capturing && beta == T(0);
+  if (!p.valid || (!p.timed && can_time)) {
     hipblasLtMatmulPreference_t pref = nullptr;
     if (!lt_ok(hipblasLtMatmulPreferenceCreate(&pref), "pref create")) return -1;
     size_t wsbytes = kGemmWorkspace;
@@ -548,11 +557,10 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
       return -1;
     }
     int best = 0;
-    if (found > 1) {
-      // Timing runs write C with beta = 0 semantics of the caller's own call, so C's final content is produced by the
-      // real call below; when beta != 0 the candidates are not run (they would accumulate into C repeatedly).
+    if (found > 1 && can_time) {
+      // The timing runs write C exactly as the caller's own call does (beta = 0); the real call below produces its final content.
       hipEvent_t e0 = nullptr, e1 = nullptr;
-      if (beta == T(0) && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+      if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
         float best_ms = 1e30f;
         for (int c = 0; c < found; c++) {
           if (res[c].workspaceSize > kGemmWorkspace) continue;
@@ -577,6 +585,7 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
     p.algo = res[best].algo;
     p.workspace = res[best].workspaceSize;
     p.valid = true;
+    p.timed = can_time;
   }
   return lt_ok(hipblasLtMatmul(h, p.desc, &alpha, A, p.la, B, p.lb, &beta, C, p.lc, C, p.lc, &p.algo, ws, kGemmWorkspace, stream), "matmul") ? 0 : -1;
 }

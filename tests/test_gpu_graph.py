@@ -109,3 +109,39 @@ def test_captured_step_with_fused_layers_dropout_and_split_reductions(knet, orac
         lib.check()
     finally:
         lib.stream = old_stream
+
+
+def test_a_product_first_seen_under_capture_is_planned_without_timing(knet):
+    """A vendor-library product whose shape the library meets for the first time while the stream is being captured: the
+    candidates cannot be timed there (that needs a synchronisation), so the first heuristic answer is recorded; the first eager
+    call afterwards times them.  Replays and the eager call all give the product."""
+    rng = np.random.default_rng(82)
+    lib = knet.libknet8()
+    m, n, k = 530, 540, 523                                   # 3e8 flop: beyond the library's own kernels, and a shape no other test uses
+    a, b = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((k, n)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    ka, kb, kc = knet.KnetArray(a), knet.KnetArray(b), knet.KnetArray(np.zeros((m, n), np.float32))
+    # the vendor library itself is initialised by an eager product of another shape, as any caller's warm-up run does
+    knet.gemm("N", "N", 1, knet.KnetArray(np.ones((600, 610), np.float32)), knet.KnetArray(np.ones((610, 620), np.float32)), 0,
+              knet.KnetArray(np.zeros((600, 620), np.float32)))
+    knet.synchronize()
+    stream = lib.fn["knet8_stream_create"]()
+    try:
+        assert lib.fn["knet8_graph_begin"](stream) == 0
+        rc = lib.fn["gemm_32_stream"](b"N", b"N", m, n, k, 1.0, ka.ptr, m, kb.ptr, k, 0.0, kc.ptr, m, stream)
+        handle = lib.fn["knet8_graph_end"](stream)
+        assert rc == 0 and handle
+        lib.check()
+        for r in range(2):
+            knet.fill(kc, 0)
+            knet.synchronize()
+            assert lib.fn["knet8_graph_launch"](handle, stream) == 0
+            lib.fn["knet8_synchronize"](stream)
+            assert rel(knet.Array(kc), want) <= 1e-5, r
+        lib.fn["knet8_graph_destroy"](handle)
+        kd = knet.gemm("N", "N", 1, ka, kb, 0, knet.KnetArray(np.zeros((m, n), np.float32)))      # eager: the candidates are timed now
+        knet.synchronize()
+        assert rel(knet.Array(kd), want) <= 1e-5
+        lib.check()
+    finally:
+        lib.fn["knet8_stream_destroy"](stream)
