@@ -635,7 +635,6 @@ KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
-   key 2: small products with 16 to this many 32x32 output tiles and k >= 97 split k inside one workgroup per tile (default 256; 1: never);
    key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 100) and at most 262144 outputs take the library's own kernels, larger ones hipBLASLt */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,

@@ -15,20 +15,19 @@
 
 namespace knet8 {
 
-// Tile and workgroup shape: 16x16 outputs per tile, four waves per workgroup, wave w taking the w-th slice of the inner dimension
-// (2x2 outputs per lane); the four partial tiles meet in LDS.  The inner dimension of either product is a batch size or a layer
-// width: with at most 128 of it every wave runs a single 32-deep step, all its loads in flight at once.
+// Tile and workgroup shape: 16x16 outputs per tile on the matrix cores (v_mfma_*_16x16x4, operands straight from global memory as in
+// gemm_mfma_kernel), four waves per workgroup, wave w taking the w-th slice of the inner dimension; the four partial tiles meet in
+// LDS.  The inner dimension of either product is a batch size or a layer width: with at most 256 of it a wave has at most four
+// 16-deep steps, all its loads in flight at once.
 constexpr int kDbTile = 16, kDbWaves = 4;
 
 template <typename T>
 __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, int m, int n, int k, const T* __restrict__ W, const T* __restrict__ x,
                                                                       const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dW,
                                                                       T* __restrict__ db, T* __restrict__ dx, int tiles_w, int tiles_w_m, int tiles_x_m,
-                                                                      int kslice_w, int kslice_x) {
-  constexpr int TS = kDbTile, KT = kGsTile, KS = kDbWaves;
-  constexpr int R = TS * KT / kWave;   // operand elements a lane stages per step (8)
-  __shared__ T As[KS][KT][TS + 1];     // As[w][kk][i] = A(i0+i, k0+kk) of wave w's current step
-  __shared__ T Bs[KS][KT][TS + 1];     // Bs[w][kk][j] = B(k0+kk, j0+j)
+                                                                      int kslice_w, int kslice_x, bool vecw, bool vecz) {
+  constexpr int TS = kDbTile, KS = kDbWaves;
+  __shared__ T part[KS][TS * TS];      // part[w][j*16 + i]
   __shared__ T rs[KS][4][TS];          // row-sum parts
   const bool job_w = (int)blockIdx.x < tiles_w;
   // C (M x N) = A (M x K) * B (K x N):  job_w: dW (m x k) = dz (m x n) * x' (n x k);  else dx (k x n) = W' (k x m) * dz (m x n)
@@ -38,76 +37,77 @@ __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, i
   const int kslice = job_w ? kslice_w : kslice_x;
   const int i0 = (tile % tm) * TS, j0 = (tile / tm) * TS;
   const int w = threadIdx.x / kWave, l = threadIdx.x & (kWave - 1);
-  const int tx = l & 7, ty = l >> 3;                      // outputs (tx + 8a, ty + 8b), a, b = 0..1
-  const int lo_t = l & (TS - 1), hi_t = l / TS;           // operand contiguous along the tile edge: kk = hi_t + 4r
-  const int lo_k = l & (KT - 1), hi_k = l / KT;           // operand contiguous along the inner dimension: edge index = hi_k + 2r
+  const int r16 = l & 15, kq = l >> 4;   // lane supplies A(i0 + r16, kk) and B(kk, j0 + r16) for kk = 4*kq .. 4*kq + 3 of each 16-deep step
   const int kbeg = w * kslice;
   int kend = kbeg + kslice;
   if (kend > K) kend = K;
-  auto dz_at = [&](int i, int j) -> T {   // dz(i, j), i < m, j < n
-    const T g = dy[i + (long)j * m];
-    if (act == 1) return y[i + (long)j * m] > T(0) ? g : T(0);
-    return g;
-  };
-  T acc[2][2] = {{T(0), T(0)}, {T(0), T(0)}};
+  const int i = i0 + r16, j = j0 + r16;
+  const bool iok = i < M, jok = j < N;
+  const bool relu = act == 1;
+  typename Mfma16<T>::Acc acc = {T(0), T(0), T(0), T(0)};
   T rowsum = T(0);
   const bool sums = job_w && j0 == 0 && db != nullptr;
-  T ga[R], gb[R];
-  auto fetch = [&](int k0) {
+  if (job_w) {
+    // A(i, kk) = dz(i, kk) and B(kk, j) = x(j, kk): both contiguous along the tile edge
+    const T* gp = dy + (iok ? i : 0);
+    const T* yp = relu ? y + (iok ? i : 0) : nullptr;
+    const T* xp = x + (jok ? j : 0);
+#pragma unroll 2
+    for (int kc = kbeg; kc < kend; kc += 16) {
+      T a[4], b[4];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      if (job_w) {
-        { const int i = i0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; ga[r] = (i < m && kk < kend) ? dz_at(i, kk) : T(0); }          // dz(i, kk): contiguous along i
-        { const int j = j0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; gb[r] = (j < k && kk < kend) ? x[j + (long)kk * k] : T(0); }     // x'(kk, j) = x(j, kk): along j
-      } else {
-        { const int kk = k0 + lo_k, i = i0 + hi_k + (kWave / KT) * r; ga[r] = (i < k && kk < kend) ? W[kk + (long)i * m] : T(0); }     // W'(i, kk) = W(kk, i): along kk
-        { const int kk = k0 + lo_k, j = j0 + hi_k + (kWave / KT) * r; gb[r] = (j < n && kk < kend) ? dz_at(kk, j) : T(0); }            // dz(kk, j): along kk
+      for (int c = 0; c < 4; c++) {
+        const int kk = kc + 4 * kq + c;
+        const bool kok = kk < kend;
+        T g = (iok && kok) ? gp[(long)kk * m] : T(0);
+        if (relu && iok && kok) g = yp[(long)kk * m] > T(0) ? g : T(0);
+        a[c] = g;
+        b[c] = (jok && kok) ? xp[(long)kk * k] : T(0);
       }
-    }
-  };
-  fetch(kbeg);
-  for (int k0 = kbeg; k0 < kbeg + kslice; k0 += KT) {     // every wave runs the same number of steps: the barriers line up
+      if (sums) rowsum = rowsum + ((a[0] + a[1]) + (a[2] + a[3]));   // zero beyond n: adds nothing
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      if (job_w) { As[w][hi_t + (kWave / TS) * r][lo_t] = ga[r]; Bs[w][hi_t + (kWave / TS) * r][lo_t] = gb[r]; }
-      else       { As[w][lo_k][hi_k + (kWave / KT) * r] = ga[r]; Bs[w][lo_k][hi_k + (kWave / KT) * r] = gb[r]; }
+      for (int c = 0; c < 4; c++) acc = Mfma16<T>::run(a[c], b[c], acc);
     }
-    __syncthreads();
-    if (k0 + KT < kbeg + kslice) fetch(k0 + KT);
-    if (sums) {   // lane (i = l % 16, part = l / 16) adds the eight kk of its part of this wave's slice (zero beyond n: adds nothing)
+  } else {
+    // A(i, kk) = W(kk, i) and B(kk, j) = dz(kk, j): both contiguous along the inner dimension
+    const T* wp = W + (long)(iok ? i : 0) * m;
+    const T* gp = dy + (long)(jok ? j : 0) * m;
+    const T* yp = relu ? y + (long)(jok ? j : 0) * m : nullptr;
+#pragma unroll 2
+    for (int kc = kbeg; kc < kend; kc += 16) {
+      T a[4], b[4];
+      mfma_load4<T, true>(a, wp, 1, kc + 4 * kq, kend, iok, vecw);
+      mfma_load4<T, true>(b, gp, 1, kc + 4 * kq, kend, jok, vecz);
+      if (relu) {
+        T yy[4];
+        mfma_load4<T, true>(yy, yp, 1, kc + 4 * kq, kend, jok, vecz);
 #pragma unroll
-      for (int q = 0; q < KT / 4; q++) rowsum = rowsum + As[w][hi_t * (KT / 4) + q][lo_t];
+        for (int c = 0; c < 4; c++) b[c] = yy[c] > T(0) ? b[c] : T(0);   // masked-out lanes hold zeros in both
+      }
+#pragma unroll
+      for (int c = 0; c < 4; c++) acc = Mfma16<T>::run(a[c], b[c], acc);
     }
-#pragma unroll 8
-    for (int kk = 0; kk < KT; kk++) {
-      const T a0 = As[w][kk][tx], a1 = As[w][kk][tx + 8], b0 = Bs[w][kk][ty], b1 = Bs[w][kk][ty + 8];
-      acc[0][0] = kfma(a0, b0, acc[0][0]); acc[1][0] = kfma(a1, b0, acc[1][0]); acc[0][1] = kfma(a0, b1, acc[0][1]); acc[1][1] = kfma(a1, b1, acc[1][1]);
-    }
-    __syncthreads();
   }
-  // partial tiles into LDS (each wave reuses its own staging area), summed in wave order; row-sum parts likewise
-  T* mine = &As[w][0][0];
+  // partial tiles into LDS, summed in wave order; row-sum parts likewise
 #pragma unroll
-  for (int a = 0; a < 2; a++)
-#pragma unroll
-    for (int b = 0; b < 2; b++) mine[(ty + 8 * b) * TS + tx + 8 * a] = acc[a][b];
-  if (sums) rs[w][hi_t][lo_t] = rowsum;
+  for (int r = 0; r < 4; r++) part[w][r16 * TS + Mfma16<T>::row(r, kq)] = acc[r];
+  if (sums) rs[w][kq][r16] = rowsum;
   __syncthreads();
   T* C = job_w ? dW : dx;
   {
     const int o = threadIdx.x;   // 256 lanes, 256 outputs
     T sum = T(0);
 #pragma unroll
-    for (int q = 0; q < KS; q++) sum += (&As[q][0][0])[o];
-    const int i = i0 + (o & (TS - 1)), j = j0 + o / TS;
-    if (i < M && j < N) C[i + (long)j * M] = sum;
+    for (int q = 0; q < KS; q++) sum += part[q][o];
+    const int oi = i0 + (o & (TS - 1)), oj = j0 + o / TS;
+    if (oi < M && oj < N) C[oi + (long)oj * M] = sum;
   }
   if (sums && threadIdx.x < TS && i0 + (int)threadIdx.x < m) {
     T r = T(0);
 #pragma unroll
     for (int q = 0; q < KS; q++)
 #pragma unroll
-      for (int part = 0; part < 4; part++) r = r + rs[q][part][threadIdx.x];
+      for (int pq = 0; pq < 4; pq++) r = r + rs[q][pq][threadIdx.x];
     db[i0 + threadIdx.x] = r;
   }
 }
@@ -129,10 +129,13 @@ inline int launch_dense_back(hipStream_t stream, int act, int m, int n, int k, c
   const int tx_m = (k + kDbTile - 1) / kDbTile, tx_n = (n + kDbTile - 1) / kDbTile;
   const int tiles_w = dW ? tw_m * tw_n : 0, tiles_x = dx ? tx_m * tx_n : 0;
   if (tiles_w + tiles_x == 0) return 0;
-  // inner dimension per wave, in whole 32-deep steps
-  auto slice = [](int K) { const int steps = (K + kGsTile - 1) / kGsTile; return ((steps + kDbWaves - 1) / kDbWaves) * kGsTile; };
+  // inner dimension per wave, in whole 16-deep steps
+  auto slice = [](int K) { const int steps = (K + 15) / 16; return ((steps + kDbWaves - 1) / kDbWaves) * 16; };
+  // 16-byte (fp64: 32-byte) loads along the inner dimension of dx = W'*dz need columns of W, dy and y that start on such a boundary
+  const bool vecw = W != nullptr && mfma_vec_ok(W, m);
+  const bool vecz = mfma_vec_ok(dy, m) && (act != 1 || mfma_vec_ok(y, m));
   hipLaunchKernelGGL((dense_back_kernel<T>), dim3((unsigned)(tiles_w + tiles_x)), dim3(kDbWaves * kWave), 0, stream, act, m, n, k, W, x, y, dy, dW, db, dx,
-                     tiles_w, tw_m, tx_m, slice(n), slice(m));
+                     tiles_w, tw_m, tx_m, slice(n), slice(m), vecw, vecz);
   return 0;
 }
 

@@ -1,15 +1,13 @@
 // Small-matrix GEMM C = alpha*op(A)*op(B) + beta*C (column-major), for products far too small to fill the
-// machine -- the 64x100x784-class products of the MNIST MLP, where the vendor library needs 15-25 us per call.  Large products
-// go to hipBLASLt (knet8_runtime.hip).  At this size a product's time is one launch (3.2 us for an empty kernel), one memory round
-// trip and a few 32-deep tile steps: what matters is how many steps run one after the other and whether partial results have to
-// leave the workgroup.  Three kernels, chosen in launch_gemm_small:
-//   * gemm_wave_kernel<.., KS, 16>: 16x16 output tile per workgroup, one wave per k slice (KS = 1..16 slices), partial tiles summed
-//     in LDS -- everything up to about 7e7 flop;
-//   * gemm_wave_kernel<.., KS, 32>: the same with 32x32 tiles (4x4 outputs per lane) for the upper end of the range, when there are
-//     at least 16 such tiles;
+// machine -- the 64x100x784-class products of the MNIST MLP, where the vendor library needs 12-25 us of host and device time per
+// call.  Large products go to hipBLASLt (knet8_runtime.hip).  At this size a product's time is one launch (3.2 us for an empty
+// kernel), one memory round trip and a short k walk: what matters is how many steps run one after the other and whether partial
+// results have to leave the workgroup.  Two kernels, chosen in launch_gemm_small:
+//   * gemm_mfma_kernel: 16x16 output tile per workgroup on the matrix cores, one wave per k slice (1..16 slices), operands straight
+//     from global memory into the instruction's registers, partial tiles summed in LDS -- every product with k <= 8192;
 //   * gemm_small_kernel: 32x32 tile per 256-lane workgroup, k split over P workgroups per tile whose partial tiles are combined, in
 //     fixed order, by the last one to finish (write-through + ticket, as in the reductions) -- few tiles with a very long k.
-// All three add the bias and apply relu in their output stage when asked (gemm_bias_act_S): same bits as separate launches.
+// Both add the bias and apply relu in their output stage when asked (gemm_bias_act_S): same bits as separate launches.
 #pragma once
 #include "knet8_device.h"
 #include "knet8_runtime.h"
@@ -105,94 +103,90 @@ __global__ __launch_bounds__(256) void gemm_small_kernel(int m, int n, int k, T 
     }
 }
 
-// ---- k split inside the workgroup ------------------------------------------------------------------------------
-// For the very small products (a few output tiles, k in the tens to hundreds) the cross-workgroup ticket costs more than the
-// arithmetic: three dependent memory round trips after the last product.  Here one wave owns the whole 32x32 tile for a slice
-// of k (4x4 outputs per lane) and the KS waves of a workgroup take KS slices; their partial tiles meet in LDS.  Every wave runs
-// the same number of k steps (loads beyond its slice or beyond k read zeros), so the workgroup barriers line up.
-// TS is the edge of a wave's output tile: 32 (4x4 outputs per lane) or 16 (2x2 per lane).  The small tile is for products with
-// so few 32x32 tiles and so long a k that even sixteen waves per tile leave most of the chip idle and each wave with a long serial
-// walk: four times the workgroups, a quarter of the arithmetic per wave.
-template <typename T, bool TA, bool TB, int KS, int TS = kGsTile>
-__global__ __launch_bounds__(KS * kWave) void gemm_wave_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda,
-                                                              const T* __restrict__ B, int ldb, T beta, T* C, int ldc, const T* bias, int act, int kslice) {
-  constexpr int KT = kGsTile;            // k elements per step
-  constexpr int Q = TS / 8;              // outputs per lane along each axis (lanes form an 8x8 grid)
-  constexpr int R = TS * KT / kWave;     // operand elements a lane stages per step
-  __shared__ T As[KS][KT][TS + 1];  // As[w][kk][i] = op(A)(i0+i, k0+kk) of wave w's current step
-  __shared__ T Bs[KS][KT][TS + 1];
+// ---- 16x16 tiles on the matrix cores, k split inside the workgroup ------------------------------------------------
+// v_mfma_{f32,f64}_16x16x4: one instruction multiplies a 16x4 by a 4x16 panel in full fp32/fp64 precision.  Lane l supplies
+// A(i = l%16, kk = l/16) and B(kk = l/16, j = l%16) and receives four outputs, column j = l%16, rows 4*(l/16) + r in fp32 and
+// 4*r + l/16 in fp64 (r = 0..3).  The operands go from global memory straight into the instruction's registers -- no LDS staging, no
+// barrier inside the k walk.  Which k a lane feeds to which of the four instructions of a 16-deep step is free as long as A and B
+// agree: lane (.., q = l/16) takes k = 4q .. 4q+3, so an operand that is contiguous along k is read with one 16-byte (fp64: 32-byte)
+// load per lane and step -- with 4-byte loads the sixteen lines a wave touches per instruction keep the CU's address unit busy four
+// times as long, and the sixteen waves of a workgroup share it.  The KS waves of a workgroup take KS slices of k (every wave of
+// the product has all its loads in flight at once) and their partial tiles meet in LDS: no combine leaves the workgroup.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+template <typename T> struct Mfma16;
+template <> struct Mfma16<float> {
+  typedef f32x4_t Acc;
+  __device__ static __forceinline__ Acc run(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  __device__ static __forceinline__ int row(int r, int kq) { return 4 * kq + r; }
+};
+template <> struct Mfma16<double> {
+  typedef f64x4_t Acc;
+  __device__ static __forceinline__ Acc run(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  __device__ static __forceinline__ int row(int r, int kq) { return 4 * r + kq; }
+};
+
+// Four consecutive k of one operand column (or row) for a lane: p points at k = 0 of it, `step` is the distance between consecutive k.
+template <typename T, bool KCONT>
+__device__ __forceinline__ void mfma_load4(T (&v)[4], const T* __restrict__ p, long step, int kk0, int kend, bool ok, bool vec) {
+  typedef T V4 __attribute__((ext_vector_type(4)));
+  if (KCONT && vec && ok && kk0 + 3 < kend) {
+    const V4 q = *reinterpret_cast<const V4*>(p + kk0);
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = q[c];
+  } else {
+#pragma unroll
+    for (int c = 0; c < 4; c++) v[c] = (ok && kk0 + c < kend) ? p[(kk0 + c) * step] : T(0);
+  }
+}
+template <typename T>
+inline bool mfma_vec_ok(const T* p, int ld) { return (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0 && ld % 4 == 0; }
+
+template <typename T, bool TA, bool TB, int KS>
+__global__ __launch_bounds__(KS * kWave) void gemm_mfma_kernel(int m, int n, int k, T alpha, const T* __restrict__ A, int lda, const T* __restrict__ B,
+                                                              int ldb, T beta, T* C, int ldc, const T* bias, int act, int kslice, bool veca, bool vecb) {
+  constexpr int TS = 16;
+  __shared__ T part[KS > 1 ? KS : 1][TS * TS];   // part[w][j*16 + i]
   const int tiles_m = (m + TS - 1) / TS;
   const int tile = blockIdx.x;
   const int i0 = (tile % tiles_m) * TS, j0 = (tile / tiles_m) * TS;
   const int w = threadIdx.x / kWave, l = threadIdx.x & (kWave - 1);
-  const int tx = l & 7, ty = l >> 3;  // outputs (tx + 8a, ty + 8b), a, b = 0..Q-1
-  // loader coordinates: `lo` runs along the operand's contiguous axis (TS long for the tile edge, KT long for k), `hi` across it
-  const int lo_t = l & (TS - 1), hi_t = l / TS;           // contiguous along the tile edge: kk = hi_t + (64/TS) r
-  const int lo_k = l & (KT - 1), hi_k = l / KT;           // contiguous along k: edge index = hi_k + (64/KT) r
+  const int r16 = l & 15, kq = l >> 4;
   const int kbeg = w * kslice;
   int kend = kbeg + kslice;
   if (kend > k) kend = k;
-  T acc[Q][Q];
+  const int i = i0 + r16, j = j0 + r16;
+  const bool iok = i < m, jok = j < n;
+  // column (or row) of each operand this lane walks; out-of-range lanes read element 0 of a valid column and are masked to zero
+  const T* ap = TA ? A + (long)(iok ? i : 0) * lda : A + (iok ? i : 0);
+  const T* bp = TB ? B + (jok ? j : 0) : B + (long)(jok ? j : 0) * ldb;
+  const long astep = TA ? 1 : lda, bstep = TB ? ldb : 1;
+  typename Mfma16<T>::Acc acc = {T(0), T(0), T(0), T(0)};
+#pragma unroll 4
+  for (int kc = kbeg; kc < kend; kc += 16) {
+    T a[4], b[4];
+    mfma_load4<T, TA>(a, ap, astep, kc + 4 * kq, kend, iok, veca);
+    mfma_load4<T, !TB>(b, bp, bstep, kc + 4 * kq, kend, jok, vecb);
 #pragma unroll
-  for (int a = 0; a < Q; a++)
-#pragma unroll
-    for (int b = 0; b < Q; b++) acc[a][b] = T(0);
-  T ga[R], gb[R];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      if (!TA) { const int i = i0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; ga[r] = (i < m && kk < kend) ? A[i + (long)kk * lda] : T(0); }
-      else     { const int kk = k0 + lo_k, i = i0 + hi_k + (kWave / KT) * r; ga[r] = (i < m && kk < kend) ? A[kk + (long)i * lda] : T(0); }
-      if (!TB) { const int kk = k0 + lo_k, j = j0 + hi_k + (kWave / KT) * r; gb[r] = (j < n && kk < kend) ? B[kk + (long)j * ldb] : T(0); }
-      else     { const int j = j0 + lo_t, kk = k0 + hi_t + (kWave / TS) * r; gb[r] = (j < n && kk < kend) ? B[j + (long)kk * ldb] : T(0); }
-    }
-  };
-  fetch(kbeg);
-  for (int k0 = kbeg; k0 < kbeg + kslice; k0 += KT) {
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      if (!TA) As[w][hi_t + (kWave / TS) * r][lo_t] = ga[r]; else As[w][lo_k][hi_k + (kWave / KT) * r] = ga[r];
-      if (!TB) Bs[w][lo_k][hi_k + (kWave / KT) * r] = gb[r]; else Bs[w][hi_t + (kWave / TS) * r][lo_t] = gb[r];
-    }
-    __syncthreads();
-    if (k0 + KT < kbeg + kslice) fetch(k0 + KT);
-#pragma unroll 8
-    for (int kk = 0; kk < KT; kk++) {
-      T av[Q], bv[Q];
-#pragma unroll
-      for (int a = 0; a < Q; a++) av[a] = As[w][kk][tx + 8 * a];
-#pragma unroll
-      for (int b = 0; b < Q; b++) bv[b] = Bs[w][kk][ty + 8 * b];
-#pragma unroll
-      for (int a = 0; a < Q; a++)
-#pragma unroll
-        for (int b = 0; b < Q; b++) acc[a][b] = kfma(av[a], bv[b], acc[a][b]);
-    }
-    __syncthreads();
+    for (int c = 0; c < 4; c++) acc = Mfma16<T>::run(a[c], b[c], acc);
   }
   if (KS > 1) {
-    // partial tiles into LDS (each wave reuses its own staging area: KT*(TS+1) >= TS*TS elements), summed in wave order
-    T* mine = &As[w][0][0];
 #pragma unroll
-    for (int a = 0; a < Q; a++)
-#pragma unroll
-      for (int b = 0; b < Q; b++) mine[(ty + 8 * b) * TS + tx + 8 * a] = acc[a][b];
+    for (int r = 0; r < 4; r++) part[w][r16 * TS + Mfma16<T>::row(r, kq)] = acc[r];
     __syncthreads();
     for (int o = threadIdx.x; o < TS * TS; o += KS * kWave) {
       T sum = T(0);
 #pragma unroll
-      for (int q = 0; q < KS; q++) sum += (&As[q][0][0])[o];
-      const int i = i0 + (o & (TS - 1)), j = j0 + o / TS;
-      if (i < m && j < n) gemm_store(C + i + (long)j * ldc, sum, alpha, beta, bias, i, act);
+      for (int q = 0; q < KS; q++) sum += part[q][o];
+      const int oi = i0 + (o & (TS - 1)), oj = j0 + o / TS;
+      if (oi < m && oj < n) gemm_store(C + oi + (long)oj * ldc, sum, alpha, beta, bias, oi, act);
     }
   } else {
 #pragma unroll
-    for (int a = 0; a < Q; a++)
-#pragma unroll
-      for (int b = 0; b < Q; b++) {
-        const int i = i0 + tx + 8 * a, j = j0 + ty + 8 * b;
-        if (i < m && j < n) gemm_store(C + i + (long)j * ldc, acc[a][b], alpha, beta, bias, i, act);
-      }
+    for (int r = 0; r < 4; r++) {
+      const int oi = i0 + Mfma16<T>::row(r, kq);
+      if (oi < m && jok) gemm_store(C + oi + (long)j * ldc, acc[r], alpha, beta, bias, oi, act);
+    }
   }
 }
 
@@ -210,47 +204,26 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
   const long tiles = (long)((m + kGsTile - 1) / kGsTile) * ((n + kGsTile - 1) / kGsTile);
   const long ksteps = (k + kGsTile - 1) / kGsTile;
   const long tiles16 = (long)((m + 15) / 16) * ((n + 15) / 16);
-  if (tiles16 * ksteps <= 4096 && tuning(kTuneGemmWaveTiles) != 1) {
-    // The smaller products (up to about 7e7 flop): 16x16 tiles, one wave per tile and k slice, as many slices per workgroup as there
-    // are 32-deep steps (up to 16), partial tiles combined in LDS -- every load of the product is in flight at once and no combine
-    // leaves the workgroup.  Measured (us per call, back-to-back launches; this path vs the 32x32-tile paths below):
-    // 64x100x784 7.6/12.1, 10x100x64 3.8/5.3, 64x784x100 NT 4.1/6.1, 128^3 3.9/6.1, 256^3 4.2/6.4, 300^3 7.5/9.6, 256x300x512 TN 7.7/10.1,
-    // 1000x10x1000 7.8/15.5, 64x4096x100 5.2/6.7; from about 1e8 flop (512x512x190: 7.8/6.9) the larger tiles win.
+  if (ksteps <= 256) {
+    // One wave per 16x16 tile and k slice, as many slices per workgroup as there are 32-deep steps (up to 16).  Kernel durations
+    // (us, rocprofv3 kernel trace, fp32; this kernel / the vendor library's kernel, which costs its caller another 12 us of host time):
+    // 64x100x784 4.6/-, 10x100x64 3.4/-, 32^3 2.5/-, 128^3 3.0/-, 256^3 3.5/-, 300^3 4.5/-, 512x300x256 4.9/6.9, 256x300x512 TN 6.1/11.6,
+    // 700x300x200 5.2/6.8, 400^3 6.3/7.3, 512^3 8.5/8.2 (NT 8.8/8.7, TN 10.7/7.0), 256x256x2048 8.6/11.4, 64x64x2000 7.5/11.1, 16x16x4000 12.0/-.
+    // Beyond k = 8192 with few tiles a wave's serial walk gets long and the cross-workgroup split below takes over.
     int ks = 1;
     while (ks < 16 && ks < ksteps) ks *= 2;
     const int kslice = (int)((ksteps + ks - 1) / ks) * kGsTile;
     const dim3 grid16((unsigned)tiles16);
-#define KNET8_GW16K(TA, TB, KSX) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KSX, 16>), grid16, dim3(KSX * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
-#define KNET8_GW16(TA, TB) do { if (ks == 1) KNET8_GW16K(TA, TB, 1); else if (ks == 2) KNET8_GW16K(TA, TB, 2); else if (ks == 4) KNET8_GW16K(TA, TB, 4); \
-                                else if (ks == 8) KNET8_GW16K(TA, TB, 8); else KNET8_GW16K(TA, TB, 16); } while (0)
-    if (!ta && !tb) KNET8_GW16(false, false);
-    else if (ta && !tb) KNET8_GW16(true, false);
-    else if (!ta && tb) KNET8_GW16(false, true);
-    else KNET8_GW16(true, true);
-#undef KNET8_GW16
-#undef KNET8_GW16K
-    return;
-  }
-  if (ksteps >= 4 && tiles >= 16 && tiles <= tuning(kTuneGemmWaveTiles)) {
-    // Enough tiles to occupy a fair share of the CUs and a k long enough that walking it serially would dominate: one wave per k
-    // slice inside the workgroup, no cross-workgroup combine.  Measured (us per call, back-to-back launches, this kernel vs the
-    // one below): 128^3 6.1/7.1, 256^3 6.3/9.9, 512x300x256 6.4/10.0, 512x256x300 NT 9.2/12.4, 256x300x512 TN 10.4/17.3.  With fewer
-    // tiles (64x100x784: 15.4/11.8) one CU's LDS bandwidth limits a 16-wave workgroup and the cross-workgroup split wins; with
-    // short k (256x300x96: 6.7/5.1) the 256-lane tiles win.
-    constexpr int kMaxKs = sizeof(T) == 4 ? 16 : 8;  // 2 * 32*33 elements of LDS per wave
-    int ks = 1;
-    while (ks < kMaxKs && ks < ksteps) ks *= 2;
-    const int kslice = (int)((ksteps + ks - 1) / ks) * kGsTile;
-    const dim3 grid((unsigned)tiles);
-#define KNET8_GW1(TA, TB, KS) hipLaunchKernelGGL((gemm_wave_kernel<T, TA, TB, KS>), grid, dim3(KS * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice)
-#define KNET8_GW(TA, TB) do { if (ks == 1) KNET8_GW1(TA, TB, 1); else if (ks == 2) KNET8_GW1(TA, TB, 2); else if (ks == 4) KNET8_GW1(TA, TB, 4); \
-                              else if (ks == 8) KNET8_GW1(TA, TB, 8); else { if constexpr (kMaxKs >= 16) KNET8_GW1(TA, TB, kMaxKs); } } while (0)
-    if (!ta && !tb) KNET8_GW(false, false);
-    else if (ta && !tb) KNET8_GW(true, false);
-    else if (!ta && tb) KNET8_GW(false, true);
-    else KNET8_GW(true, true);
-#undef KNET8_GW
-#undef KNET8_GW1
+    const bool veca = ta && mfma_vec_ok(A, lda), vecb = !tb && mfma_vec_ok(B, ldb);
+#define KNET8_GM16K(TA, TB, KSX) hipLaunchKernelGGL((gemm_mfma_kernel<T, TA, TB, KSX>), grid16, dim3(KSX * kWave), 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kslice, veca, vecb)
+#define KNET8_GM16(TA, TB) do { if (ks == 1) KNET8_GM16K(TA, TB, 1); else if (ks == 2) KNET8_GM16K(TA, TB, 2); else if (ks == 4) KNET8_GM16K(TA, TB, 4); \
+                                else if (ks == 8) KNET8_GM16K(TA, TB, 8); else KNET8_GM16K(TA, TB, 16); } while (0)
+    if (!ta && !tb) KNET8_GM16(false, false);
+    else if (ta && !tb) KNET8_GM16(true, false);
+    else if (!ta && tb) KNET8_GM16(false, true);
+    else KNET8_GM16(true, true);
+#undef KNET8_GM16
+#undef KNET8_GM16K
     return;
   }
   long P = 1;

@@ -74,7 +74,6 @@ int tuning(int key) {
       g_tune[key] = 256;
     }
   }
-  if (key == kTuneGemmWaveTiles && g_tune[key] == 0) g_tune[key] = 256;  // at most this many output tiles (and at least 16): k is split inside the workgroup (1 switches that kernel off)
   if (key == kTuneGemmSmallMflop && g_tune[key] == 0) g_tune[key] = 100;  // products up to this many MFLOP (2mnk) take the library's own kernels
   return g_tune[key];
 }

@@ -164,12 +164,12 @@ def test_allocator_pool(knet):
 def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
     rng = np.random.default_rng(54)
     rtol = 1e-5 if dt == np.float32 else 1e-13
-    # the small-product kernels: 16x16 tiles with k slices inside a workgroup (up to about 7e7 flop), above that 32x32 tiles with k
-    # slices inside a workgroup (16+ tiles) or the cross-workgroup k split (fewer tiles)
+    # the small-product kernels: 16x16 tiles on the matrix cores with k slices inside a workgroup (k <= 8192), the cross-workgroup
+    # k split beyond; operands whose k-contiguous columns are 16-byte aligned take the wide loads (k a multiple of 4), the others not
     for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000), (130, 131, 129), (512, 300, 256), (256, 300, 96), (100, 500, 97),
                       (10, 100, 500), (33, 17, 300), (1, 1, 1000), (17, 95, 225), (64, 100, 200),
                       (64, 64, 10000), (40, 33, 9000),      # few tiles, very long k: the cross-workgroup k split with its ticket
-                      (512, 512, 190), (700, 300, 200)]:    # near the upper end of the small-product range: 32x32 wave tiles
+                      (512, 512, 190), (700, 300, 200), (16, 16, 4000), (48, 20, 8192)]:    # the upper end of the small-product range
         A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
         want = oracle.gemm(A, B)
         Ad, Bd, Atd, Btd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.ascontiguousarray(A.T)), knet.KnetArray(np.ascontiguousarray(B.T))
@@ -182,6 +182,17 @@ def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
         C = knet.gemm("N", "N", 0.5, Ad, Bd, 2.0, knet.KnetArray(C0))
         assert np.linalg.norm(knet.Array(C) - (0.5 * want + 2 * C0)) <= 10 * rtol * np.linalg.norm(want)
         assert bits_equal(knet.Array(knet.transpose(Ad)), np.ascontiguousarray(A.T))
+    # operands that start at odd element offsets inside larger buffers (sub-array views): the wide loads along k must not be taken
+    for (m, n, k) in [(37, 29, 64), (64, 100, 784)]:
+        for off in (1, 2, 3):
+            A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
+            want = oracle.gemm(A, B)
+            bufa, bufb = knet.KnetArray(np.zeros(m * k + 8, dt)), knet.KnetArray(np.zeros(k * n + 8, dt))
+            at, bv = bufa.view1d(off, m * k).reshape(k, m), bufb.view1d(off, k * n).reshape(k, n)
+            knet.setindex_(bufa, knet.KnetArray(np.ascontiguousarray(A.T).ravel(order="F")), (off + 1, off + m * k))
+            knet.setindex_(bufb, knet.KnetArray(B.ravel(order="F")), (off + 1, off + k * n))
+            C = knet.gemm("T", "N", 1, at, bv, 0, knet.KnetArray(np.zeros((m, n), dt)))
+            assert np.linalg.norm(knet.Array(C) - want) <= rtol * np.linalg.norm(want), (m, n, k, off)
     with pytest.raises(ValueError):
         knet.gemm("N", "N", 1, knet.KnetArray(np.zeros((3, 4), dt)), knet.KnetArray(np.zeros((5, 2), dt)), 0, knet.KnetArray(np.zeros((3, 2), dt)))
     knet.libknet8().check()
