@@ -26,7 +26,7 @@ from .update import SGD, Momentum, Nesterov, Adagrad, Rmsprop, Adadelta, Adam, u
 from .train import (Data, minibatch, param, param0, params, gaussian, xavier, xavier_uniform, xavier_normal, Minimize, minimize, minimize_,
                     sgd, sgd_, momentum, momentum_, nesterov, nesterov_, adagrad, adagrad_, rmsprop, rmsprop_, adadelta, adadelta_,
                     adam, adam_, converge, converge_, train_, updates, epochs)
-from .linalg import dense, matmul, mat, bmm, bmm_, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
+from .linalg import dense, dense_nll, matmul, mat, bmm, bmm_, gemm, A_mul_B, A_mul_Bt, At_mul_B, axpy, scal, transpose, permutedims
 
 libknet8()  # fail loudly at import time if the HIP library is missing
 

@@ -453,6 +453,18 @@ def gen_elementwise():
                  (T + "*", "dW"), (T + "*", "db"), (T + "*", "dx")], None,
                 "reluback_S_11 + sum_S_21 + gemm! x 2, src/knetarrays/linalg.jl:11-18",
                 body="  const int rc = launch_dense_back<%s>(stream, act, m, n, k, W, x, y, dy, dW, db, dx);\n  knet8::check_launch(\"dense_back_%s\");\n  return rc;" % (T, S))
+    o.decl.append("/* dense_nll_back_S: backward pass of a classifier's output layer with the loss folded in.  z = W*x + b are the scores (m classes x n\n"
+                  "   instances, m <= 16), labels 1-based int32 (0 skips the instance).  Writes loss[j] = -logsoftmax(z)[label_j, j], mean[0] =\n"
+                  "   scale * sum(loss) (the average loss when scale = 1/count) and, with dz = scale*(softmax(z) - onehot(label)): dW = dz*x' (m x k),\n"
+                  "   db = sum(dz; dims=2), dx = W'*dz (k x n); dW, db, dx, loss, mean may be NULL (db, loss and mean need dW).  Returns 0 when done, 1 when not applicable (more than 16 classes, or too large: nothing is launched and\n"
+                  "   the caller uses nll_logsoftmax_back_S + dense_back_S), -1 on bad arguments.  No libknet8 counterpart: replaces the chain of\n"
+                  "   src/ops20/loss.jl:37-41 plus sum(dz;dims=2) and two gemm! calls (src/knetarrays/linalg.jl:11-18). */")
+    for T, S in TYPES:
+        o.entry("dense_nll_back_%s" % S, "int",
+                [("int", "m"), ("int", "n"), ("int", "k"), (T + "*", "W"), (T + "*", "x"), (T + "*", "z"), ("int*", "labels"), (T, "scale"),
+                 (T + "*", "dW"), (T + "*", "db"), (T + "*", "dx"), (T + "*", "loss"), (T + "*", "mean")], None,
+                "nll -> logsoftmax -> getindex (src/ops20/loss.jl:37-41) + sum_S_21 + gemm! x 2, src/knetarrays/linalg.jl:11-18",
+                body="  const int rc = launch_dense_nll_back<%s>(stream, m, n, k, W, x, z, labels, scale, dW, db, dx, loss, mean);\n  knet8::check_launch(\"dense_nll_back_%s\");\n  return rc;" % (T, S))
     for T, S in TYPES:
         o.entry("biasreludrop_%s" % S, "void", [("int", "m"), ("int", "n"), (T, "p"), (T + "*", "z"), (T + "*", "b"), (T + "*", "y")],
                 "launch_bias_act<%s, true>(stream, m, n, z, b, y, BiasReluDrop<%s>{p, %s(1) - p})" % (T, T, T),
@@ -635,7 +647,8 @@ KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
-   key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 100) and at most 262144 outputs take the library's own kernels, larger ones hipBLASLt */
+   key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 100) and at most 262144 outputs take the library's own kernels, larger ones hipBLASLt;
+   key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
    src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */

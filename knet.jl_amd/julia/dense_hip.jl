@@ -78,3 +78,20 @@ for (T, S) in ((Float32, 32), (Float64, 64))
         return rc == 0
     end
 end
+
+# Output layer of a classifier: from the scores z = w*x .+ b and Int32 labels (0 = skip), the mean loss (scale * sum of the losses,
+# scale = 1/count), and with dz = scale*(softmax(z) - onehot): dw = dz*x', db = sum(dz;dims=2), dx = w'*dz -- one call
+# (dense_nll_back_S) in place of nll -> logsoftmax -> getindex (src/ops20/loss.jl:37-41) and the layer's separate backward launches.
+# Returns false when the library declines (more than 16 classes or a layer beyond its small-matrix kernels).
+for (T, S) in ((Float32, 32), (Float64, 64))
+    @eval function dense_nll_back!(mean::KnetArray{$T}, dw::KnetArray{$T,2}, db::KnetArray{$T}, dx::Union{KnetArray{$T,2},Nothing},
+                                   w::KnetArray{$T,2}, x::KnetArray{$T,2}, z::KnetArray{$T,2}, labels::KnetArray{Int32}, scale::Real)
+        m, k = size(w); n = size(x, 2)
+        @assert size(x, 1) == k && size(z) == (m, n) && length(labels) == n && size(dw) == (m, k) && length(db) == m
+        rc = ccall(($("dense_nll_back_$(S)_stream"), LibKnet8.libknet8), Cint,
+                   (Cint, Cint, Cint, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{Cint}, $T, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{Cvoid}),
+                   m, n, k, w, x, z, labels, $T(scale), dw, db, dx === nothing ? C_NULL : dx, C_NULL, mean, LibKnet8.knet8_stream())
+        rc < 0 && LibKnet8.knet8_check()
+        return rc == 0
+    end
+end

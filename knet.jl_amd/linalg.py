@@ -4,6 +4,8 @@ Mirrors src/knetarrays/linalg.jl: ``A*B``, the transposition-free gradient forms
 (``:11-18``), ``gemm!`` (``:26-52``, cuBLAS there, hipBLASLt here through ``gemm_S``), ``axpy!`` (``:58-73``)
 and ``scal!`` (``:75-90``).
 """
+import numpy as np
+
 from .autograd import primitive, selective
 from .karray import KnetArray
 from .libknet8 import knet8, libknet8
@@ -93,6 +95,59 @@ def dense(w, x, b, act=None):
             dz, db = dy, (reduce_op("sum", dy, 2).reshape(b.dims) if need[2] else None)
         return (A_mul_Bt(dz, x2) if need[0] else None, At_mul_B(w, dz).reshape(x.dims) if need[1] else None, db)
     return y, selective(back)
+
+
+def _dense_nll_fits(m, n, k):
+    # the range dense_nll_back_S accepts: at most 16 classes, products of the small-kernel class
+    return m <= 16 and 2.0 * m * n * k <= 2.7e8 and m * k <= 262144 and k * n <= 262144
+
+
+@primitive
+def _dense_nll(w, x, b, labels, count):
+    x2 = x if x.ndims == 2 else x.reshape(x.length // x.size(x.ndims), x.size(x.ndims))
+    m, k, n = _size2(w, 1), _size2(w, 2), x2.size(2)
+    lib = libknet8()
+    c = w.ctype
+    z = w.similar((m, n))
+    rc = lib.call("gemm_bias_act_%s" % w.suffix, b"N", b"N", m, n, k, c(1), w.ptr, m, x2.ptr, k, b.ptr, 0, z.ptr, m)
+    if rc != 0:
+        lib.check()
+        raise RuntimeError("gemm_bias_act failed")
+    dW, db, dx, mean = w.similar((m, k)), b.similar(), x2.similar(), w.similar((1,))
+    T = w.dtype.type
+    scale = T(1) / T(count) if count else T(np.inf)
+    rc = lib.call("dense_nll_back_%s" % w.suffix, m, n, k, w.ptr, x2.ptr, z.ptr, labels.ptr, c(scale), dW.ptr, db.ptr, dx.ptr, None, mean.ptr)
+    if rc != 0:
+        lib.check()
+        raise RuntimeError("dense_nll_back declined (%d)" % rc)
+
+    def back(dy):
+        if float(dy) != 1.0:
+            for g in (dW, db, dx):
+                scal(float(dy), g)
+        return (dW.reshape(w.dims), dx.reshape(x.dims), db, None, None)
+    return mean, back
+
+
+def dense_nll(w, x, b, labels, count=None):
+    """``nll(w*x .+ b, labels)`` for a classifier's output layer: the average loss as a 1-element ``KnetArray`` (nothing synchronises
+    with the host).  ``labels``: Int32 ``KnetArray`` of 1-based classes, 0 = skip; ``count``: number of non-zero labels (default: all).
+    With at most 16 classes and a layer of the small-kernel class the loss and the layer's three gradients come out of ONE launch
+    after the product (``dense_nll_back_S``: softmax, loss, dW, db and dx); otherwise this is ``nll(dense(w, x, b), labels; fused)``.
+    The reference runs the chain of src/ops20/loss.jl:37-41 and src/knetarrays/linalg.jl:11-18 for it."""
+    from .autograd import value as _value
+    wv, xv = _value(w), _value(x)
+    if not isinstance(labels, KnetArray) or labels.dtype != np.int32:
+        raise TypeError("MethodError: dense_nll takes Int32 device labels")
+    m, k = _size2(wv, 1), _size2(wv, 2)
+    n = xv.size(xv.ndims)
+    if labels.length != n:
+        raise ValueError("DimensionMismatch: %d labels for %d instances" % (labels.length, n))
+    count = n if count is None else int(count)
+    if _dense_nll_fits(m, n, k):
+        return _dense_nll(w, x, b, labels, count)
+    from .loss import nll
+    return nll(dense(w, x, b), labels, fused=True, count=count)
 
 
 def bmm_(transA, transB, alpha, A, B, beta, C):

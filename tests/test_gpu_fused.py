@@ -246,3 +246,99 @@ def test_dense_back_one_launch_per_layer(knet, dt):
     with pytest.raises(RuntimeError):
         lib.check()
     lib.check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_dense_nll_back_loss_and_layer_gradients_in_one_launch(knet, dt):
+    """dense_nll_back_S: from the scores z = W*x + b and the labels, the per-instance loss, its mean and the output layer's dW, db, dx in
+    one launch, against fp64 numpy: loss_j = logsumexp(z_j) - z[label_j, j], dz = scale*(softmax(z) - onehot), dW = dz*x', db = row sums,
+    dx = W'*dz.  Skipped instances (label 0), every class count up to 16, ragged sizes, wanted-output combinations; more than 16
+    classes are declined."""
+    rng = np.random.default_rng(46)
+    lib = knet.libknet8()
+    tol = 2e-5 if dt == np.float32 else 1e-12
+    c = knet.KnetArray(np.zeros(1, dt)).ctype
+    for m, n, k in ((10, 100, 64), (16, 37, 33), (3, 5, 7), (1, 4, 4), (2, 1, 1), (13, 257, 100), (10, 16, 784)):
+        W = rng.standard_normal((m, k)).astype(dt)
+        x = rng.standard_normal((k, n)).astype(dt)
+        z = (3 * rng.standard_normal((m, n))).astype(dt)
+        labels = rng.integers(1, m + 1, size=n).astype(np.int32)
+        if n > 3:
+            labels[rng.integers(0, n, size=max(1, n // 10))] = 0            # skipped instances
+        count = max(int(np.count_nonzero(labels)), 1)
+        scale = 1.0 / count
+        z64 = z.astype(np.float64)
+        zmax = z64.max(axis=0)
+        lse = zmax + np.log(np.exp(z64 - zmax).sum(axis=0))
+        keep = labels > 0
+        want_loss = np.where(keep, lse - z64[np.maximum(labels, 1) - 1, np.arange(n)], 0.0)
+        p = np.exp(z64 - lse)
+        onehot = np.zeros((m, n))
+        onehot[np.maximum(labels, 1) - 1, np.arange(n)] = 1
+        dz = np.where(keep, (p - onehot) * scale, 0.0)
+        want = (dz @ x.astype(np.float64).T, dz.sum(axis=1), W.astype(np.float64).T @ dz)
+        Wd, xd, zd, ld = knet.KnetArray(W), knet.KnetArray(x), knet.KnetArray(z), knet.KnetArray(labels)
+        for wantb, wantx, wantl, wantm in ((True, True, True, True), (False, True, True, False), (True, False, False, True), (False, False, False, False)):
+            dW = knet.KnetArray(np.full((m, k), 7, dt))
+            db = knet.KnetArray(np.full((m,), 7, dt)) if wantb else None
+            dx = knet.KnetArray(np.full((k, n), 7, dt)) if wantx else None
+            loss = knet.KnetArray(np.full((n,), 7, dt)) if wantl else None
+            mean = knet.KnetArray(np.full((1,), 7, dt)) if wantm else None
+            rc = lib.call("dense_nll_back_%s" % Wd.suffix, m, n, k, Wd.ptr, xd.ptr, zd.ptr, ld.ptr, c(scale), dW.ptr, db.ptr if db else None,
+                          dx.ptr if dx else None, loss.ptr if loss else None, mean.ptr if mean else None)
+            assert rc == 0
+            for got, w in ((dW, want[0]), (db, want[1]), (dx, want[2]), (loss, want_loss), (mean, np.array([want_loss.sum() * scale]))):
+                if got is not None:
+                    g = knet.Array(got)
+                    assert np.abs(g - w.reshape(g.shape)).max() <= tol * max(np.abs(w).max(), 1.0) * 4, (m, n, k)
+        # dx alone (no dW): the tiles of dx do not need the losses
+        dx = knet.KnetArray(np.full((k, n), 7, dt))
+        assert lib.call("dense_nll_back_%s" % Wd.suffix, m, n, k, Wd.ptr, xd.ptr, zd.ptr, ld.ptr, c(scale), None, None, dx.ptr, None, None) == 0
+        assert np.abs(knet.Array(dx) - want[2]).max() <= tol * max(np.abs(want[2]).max(), 1.0) * 4
+    # agrees with the separate launches it replaces (nll_logsoftmax_back_S + dense_back_S) to rounding
+    m, n, k = 10, 100, 64
+    W, x, z = (rng.standard_normal(s).astype(dt) for s in ((m, k), (k, n), (m, n)))
+    labels = rng.integers(1, m + 1, size=n).astype(np.int32)
+    Wd, xd, zd, ld = knet.KnetArray(W), knet.KnetArray(x), knet.KnetArray(z), knet.KnetArray(labels)
+    dz, lossv = knet.KnetArray(np.zeros((m, n), dt)), knet.KnetArray(np.zeros(n, dt))
+    knet.knet8("nll_logsoftmax_back_%s" % Wd.suffix, m, n, zd.ptr, ld.ptr, c(1.0 / n), dz.ptr, lossv.ptr)
+    sep = [knet.KnetArray(np.zeros(s, dt)) for s in ((m, k), (m,), (k, n))]
+    assert lib.call("dense_back_%s" % Wd.suffix, 0, m, n, k, Wd.ptr, xd.ptr, zd.ptr, dz.ptr, sep[0].ptr, sep[1].ptr, sep[2].ptr) == 0
+    one = [knet.KnetArray(np.zeros(s, dt)) for s in ((m, k), (m,), (k, n), (n,))]
+    assert lib.call("dense_nll_back_%s" % Wd.suffix, m, n, k, Wd.ptr, xd.ptr, zd.ptr, ld.ptr, c(1.0 / n), one[0].ptr, one[1].ptr, one[2].ptr, one[3].ptr, None) == 0
+    for a, b in zip(one, sep + [lossv]):
+        ga, gb = knet.Array(a).astype(np.float64), knet.Array(b).astype(np.float64)
+        assert np.abs(ga - gb).max() <= (1e-6 if dt == np.float32 else 1e-14) * max(np.abs(gb).max(), 1.0) * 4
+    # more than 16 classes, or the losses without dW: declined, nothing written
+    big = knet.KnetArray(np.zeros((17, 17), dt))
+    out = knet.KnetArray(np.full((17, 17), 7, dt))
+    lab17 = knet.KnetArray(np.ones(17, np.int32))
+    assert lib.call("dense_nll_back_%s" % big.suffix, 17, 17, 17, big.ptr, big.ptr, big.ptr, lab17.ptr, c(1.0), out.ptr, None, None, None, None) == 1
+    assert lib.call("dense_nll_back_%s" % big.suffix, 4, 4, 4, big.ptr, big.ptr, big.ptr, lab17.ptr, c(1.0), None, None, out.ptr, out.ptr, None) == 1
+    assert np.all(knet.Array(out) == 7)
+    lib.check()
+
+
+def test_dense_nll_on_the_tape_matches_the_separate_primitives(knet):
+    """``dense_nll(w, x, b, labels)`` against ``nll(dense(w, x, b), labels; fused)``: same loss and gradients (to rounding), for an output
+    layer inside the fused range and for one outside it (more than 16 classes: the composition itself runs)."""
+    rng = np.random.default_rng(47)
+    for m, n, k in ((10, 100, 64), (40, 30, 20)):
+        W, b, x = (rng.standard_normal(s).astype(np.float32) for s in ((m, k), (m, 1), (k, n)))
+        labels_h = rng.integers(1, m + 1, size=n)
+        labels_h[:3] = 0
+        labels = knet.KnetArray(labels_h.astype(np.int32))
+        count = int(np.count_nonzero(labels_h))
+        res = []
+        for fused in (True, False):
+            pw, pb, px = knet.Param(knet.KnetArray(W)), knet.Param(knet.KnetArray(b)), knet.Param(knet.KnetArray(x))
+            if fused:
+                J = knet.diff(lambda: knet.dense_nll(pw, px, pb, labels, count=count))
+            else:
+                J = knet.diff(lambda: knet.nll(knet.dense(pw, px, pb), labels, fused=True, count=count))
+            res.append([knet.Array(knet.value(J))] + [knet.Array(knet.grad(J, p)) for p in (pw, pb, px)])
+        for a, c in zip(*res):
+            assert a.shape == c.shape and np.abs(a.astype(np.float64) - c).max() <= 2e-6 * max(np.abs(c).max(), 1.0)
+    with pytest.raises(TypeError):
+        knet.dense_nll(knet.KnetArray(W), knet.KnetArray(x), knet.KnetArray(b), labels_h)
+    knet.libknet8().check()
