@@ -370,7 +370,8 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=F
                 J = K.diff(loss)
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
-            lossv = float(K.value(J))
+            v = K.value(J)
+            lossv = float(K.Array(v).ravel()[0]) if isinstance(v, K.KnetArray) else float(v)
         lib.check()
     finally:
         lib.stream = old_stream
@@ -530,6 +531,8 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
             "config1 same graph with dense layers (product, bias and relu in one launch)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
+            "config1 eager with dense layers and dense_nll (4 launches per step, loss left on the device)":
+                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 1000, True, layers=True, head=True),
             "config1 same graph, output layer's loss and gradients in one launch (dense_nll: 4 launches per step)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True, head=True),
             "config1 same step from a compiled C99 host through the C ABI (eager, 4 launches: fused layer kernels forward and backward, loss folded into the output layer's backward)": c_host_steps(K),

@@ -169,3 +169,42 @@ def test_mat_dims_as_the_reference_tests_them(knet, rec):
     assert knet.mat(x, dims=0).dims == (1, 384)
     m = arr((5, 7))
     assert knet.mat(m) is m
+
+
+def test_minibatch_params_converge_and_fans_on_the_host(knet):
+    """The host logic of the training callers (src/train20/data.jl, train.jl, distributions.jl) with batches kept as host arrays:
+    nothing touches the device."""
+    from knet_jl_amd import train as T
+    rng = np.random.default_rng(3)
+    x, y = rng.random((2, 3, 11)), np.arange(11)
+    d = knet.minibatch(x, y, 4, xtype=np.asarray)
+    assert len(d) == 2 and [b[0].shape for b in d] == [(2, 3, 4)] * 2 and (list(d)[1][1] == y[4:8]).all()
+    assert np.array_equal(list(d)[1][0], x[:, :, 4:8])
+    p = knet.minibatch(x, y, 4, xtype=np.asarray, partial=True)
+    assert len(p) == 3 and [b[1].tolist() for b in p][-1] == [8, 9, 10]
+    s = knet.minibatch(x, y, 5, xtype=np.asarray, shuffle=True, rng=np.random.default_rng(1))
+    got = np.concatenate([b[1] for b in s])
+    assert len(got) == 10 and len(set(got.tolist())) == 10          # one epoch without the partial batch: ten distinct instances
+    for xb, yb in s:
+        assert all(np.array_equal(xb[:, :, j], x[:, :, yb[j]]) for j in range(5))        # x and y stay paired
+    flat = list(knet.minibatch(x, 11, xtype=np.asarray, xsize=(6, 11)))
+    assert len(flat) == 1 and np.array_equal(flat[0], x.reshape((6, 11), order="F"))
+    with pytest.raises(ValueError):
+        knet.minibatch(x, y[:5], 2)
+    with pytest.raises(ValueError):
+        knet.minibatch(x, y, 0)
+    # fan-in / fan-out of the initialisers (distributions.jl:27-36)
+    assert T._fans((7,)) == (7, 1) and T._fans((3, 5)) == (5, 3) and T._fans((3, 3, 16, 32)) == (3 * 3 * 16, 3 * 3 * 32)
+    # params: attributes, sequences and dict values, each Param once
+    a, b = knet.Param(None), knet.Param(None)
+
+    class M:
+        def __init__(self):
+            self.layers, self.extra, self.name = [a, (b, 3)], {"again": a}, "m"
+    assert knet.params(M()) == [a, b]
+    # converge, updates, epochs
+    assert list(knet.converge(iter([3.0, 2.0, 1.0, 0.5]), alpha=0.1)) == [3.0, 2.0, 1.0, 0.5]
+    assert list(knet.converge(iter([1.0, 2.0, 3.0]))) == [1.0]
+    cb = knet.updates(3)
+    assert [cb(None) for _ in range(4)] == [True, True, False, False]
+    assert [knet.epochs(d, 2)(None) for _ in range(1)] == [True]
