@@ -647,7 +647,7 @@ KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
-   key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 100) and at most 262144 outputs take the library's own kernels, larger ones hipBLASLt;
+   key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 270) take the library's own kernels, larger ones hipBLASLt;
    key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,

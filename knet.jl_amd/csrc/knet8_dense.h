@@ -255,7 +255,7 @@ inline int launch_dense_back_impl(hipStream_t stream, int act, int m, int n, int
   // both products have 2*m*n*k flop; kernel durations against reluback_biasgrad + two gemm launches (us, kernel trace): 64x100x784
   // 3.6/11.3, 256^3 5.2/12.6, 300^3 7.3/14.8, 512x128x512 9.6/14.1, 400^3 11.9/18.8, 512^3 20.8/26.2 -- one launch wins over the whole range of
   // the small-product kernels (2.7e8 flop); beyond it the separate launches reach the vendor library's large tiles
-  if (2.0 * m * n * (double)k > 1.0e6 * tuning(kTuneDenseBackMflop) || (long)m * k > 262144 || (long)k * n > 262144 || (db != nullptr && dW == nullptr)) return 1;
+  if (2.0 * m * n * (double)k > 1.0e6 * tuning(kTuneDenseBackMflop) || (db != nullptr && dW == nullptr)) return 1;
   const int tw_m = (m + kDbTile - 1) / kDbTile, tw_n = (k + kDbTile - 1) / kDbTile;
   const int tx_m = (k + kDbTile - 1) / kDbTile, tx_n = (n + kDbTile - 1) / kDbTile;
   const int tiles_w = dW ? tw_m * tw_n : 0, tiles_x = dx ? tx_m * tx_n : 0;

@@ -190,12 +190,14 @@ __global__ __launch_bounds__(KS * kWave) void gemm_mfma_kernel(int m, int n, int
   }
 }
 
-// True if this product should use the small kernel.
-// hipBLASLt has a floor of about 12 us per call on this chip; the kernels here stay below it up to about 1e8 flop in general and
-// 2.7e8 flop when k <= 512 (512^3: 10.4 vs 12.0 us; 256x256x2048: 28 vs 12.6 us -- long k runs serially inside a wave).
+// True if this product should use the library's own kernels.  Against the vendor library's kernels (durations by kernel trace, fp32,
+// us; own / vendor): 1000x100x1000 8.5/9.0 (TN 8.4/10.2, dW form 1000x1000x100 NT 9.1/7.5), 1024x128x1024 8.1/8.2, 512x256x512 5.4/6.6,
+// 2048x64x784 7.1/8.2, 768x768x128 6.3/6.2 -- level up to about 2.7e8 flop whatever the shape, and the vendor call costs its caller another
+// 12 us of host time; beyond that its large LDS tiles win clearly (640^3 15.5/9.8, 2048x128x2048 28/15, 4096x100x4096 141/34).
 inline bool gemm_is_small(int m, int n, int k) {
   const double flop = 2.0 * m * n * (double)k, limit = 1.0e6 * tuning(kTuneGemmSmallMflop);
-  return (flop <= limit || (flop <= 2.7 * limit && k <= 512)) && (long)m * n <= 262144;
+  if (k > 8192) return flop <= limit && (long)m * n <= 262144;   // cross-workgroup split: its partial tiles live in the stream's scratch
+  return flop <= limit;
 }
 
 template <typename T>

@@ -74,7 +74,7 @@ int tuning(int key) {
       g_tune[key] = 256;
     }
   }
-  if (key == kTuneGemmSmallMflop && g_tune[key] == 0) g_tune[key] = 100;
+  if (key == kTuneGemmSmallMflop && g_tune[key] == 0) g_tune[key] = 270;
   if (key == kTuneDenseBackMflop && g_tune[key] == 0) g_tune[key] = 270;  // layers whose products have up to this many MFLOP each run their backward pass in one launch  // products up to this many MFLOP (2mnk) take the library's own kernels
   return g_tune[key];
 }

@@ -99,7 +99,7 @@ def dense(w, x, b, act=None):
 
 def _dense_nll_fits(m, n, k):
     # the range dense_nll_back_S accepts: at most 16 classes, products of the small-kernel class
-    return m <= 16 and 2.0 * m * n * k <= 2.7e8 and m * k <= 262144 and k * n <= 262144
+    return m <= 16 and 2.0 * m * n * k <= 2.7e8
 
 
 @primitive

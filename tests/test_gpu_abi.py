@@ -169,7 +169,7 @@ def test_gemm_all_transposes_and_transpose_kernel(knet, oracle, dt, S):
     for (m, n, k) in [(64, 100, 784), (10, 100, 64), (33, 17, 5), (1, 7, 9), (257, 129, 1000), (130, 131, 129), (512, 300, 256), (256, 300, 96), (100, 500, 97),
                       (10, 100, 500), (33, 17, 300), (1, 1, 1000), (17, 95, 225), (64, 100, 200),
                       (64, 64, 10000), (40, 33, 9000),      # few tiles, very long k: the cross-workgroup k split with its ticket
-                      (512, 512, 190), (700, 300, 200), (16, 16, 4000), (48, 20, 8192)]:    # the upper end of the small-product range
+                      (512, 512, 190), (700, 300, 200), (16, 16, 4000), (48, 20, 8192), (1000, 100, 1000), (1024, 1024, 100)]:    # the upper end of the small-product range
         A, B = rng.standard_normal((m, k)).astype(dt), rng.standard_normal((k, n)).astype(dt)
         want = oracle.gemm(A, B)
         Ad, Bd, Atd, Btd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.ascontiguousarray(A.T)), knet.KnetArray(np.ascontiguousarray(B.T))

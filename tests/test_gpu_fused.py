@@ -213,7 +213,7 @@ def test_dense_back_one_launch_per_layer(knet, dt):
     rng = np.random.default_rng(45)
     lib = knet.libknet8()
     tol = 2e-5 if dt == np.float32 else 1e-12
-    for m, n, k in ((64, 100, 784), (10, 100, 64), (33, 65, 31), (1, 1, 1), (32, 32, 32), (100, 7, 300)):
+    for m, n, k in ((64, 100, 784), (10, 100, 64), (33, 65, 31), (1, 1, 1), (32, 32, 32), (100, 7, 300), (1000, 64, 1000)):
         W = rng.standard_normal((m, k)).astype(dt)
         x = rng.standard_normal((k, n)).astype(dt)
         y = rng.standard_normal((m, n)).astype(dt)
