@@ -38,13 +38,52 @@ template <typename T> __host__ __device__ __forceinline__ bool aligned16(const T
 }
 
 // ---- wave64 reductions -------------------------------------------------------------------------
-// Butterfly over the 64 lanes with ds_bpermute-free cross-lane moves (__shfl_xor lowers to DPP /
-// ds_swizzle / permlane on gfx950).  Every lane ends with the full result, in a fixed order, so
-// results are deterministic run to run.
-template <typename T, typename Merge> __device__ __forceinline__ T wave_reduce(T v, Merge merge) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v = merge(v, __shfl_xor(v, off, kWave));
+// Cross-lane moves by DPP (data-parallel primitives: a modifier of an ordinary ALU move, full rate, no LDS traffic).  __shfl_xor
+// goes through ds_bpermute, a dependent LDS round trip per step: measured on a latency-bound kernel, sixteen such steps cost 0.5 us.
+//   row_ror:n   (0x120 + n) rotate within each row of 16 lanes
+//   row_bcast15 (0x142)     lane 15 of each row to every lane of the next row (rows chosen by the row mask)
+//   row_bcast31 (0x143)     lane 31 to every lane of rows 2 and 3
+template <int CTRL, int ROW_MASK, typename T> __device__ __forceinline__ T dpp_move(T v) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "dpp_move: 4- or 8-byte values");
+  if constexpr (sizeof(T) == 4) {
+    const int b = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(b, b, CTRL, ROW_MASK, 0xf, false));
+  } else {
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = (int)b, hi = (int)(b >> 32);
+    const int nlo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+    const int nhi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(T, ((long long)nhi << 32) | (unsigned int)nlo);
+  }
+}
+template <typename T> __device__ __forceinline__ T wave_read_lane63(T v) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+  } else {
+    const long long b = __builtin_bit_cast(long long, v);
+    const int lo = __builtin_amdgcn_readlane((int)b, 63), hi = __builtin_amdgcn_readlane((int)(b >> 32), 63);
+    return __builtin_bit_cast(T, ((long long)hi << 32) | (unsigned int)lo);
+  }
+}
+// All-reduce over the 16 lanes of each row by rotations (every lane of a row ends with the row's result).
+template <typename T, typename Merge> __device__ __forceinline__ T row16_reduce(T v, Merge merge) {
+  v = merge(v, dpp_move<0x128, 0xf>(v));
+  v = merge(v, dpp_move<0x124, 0xf>(v));
+  v = merge(v, dpp_move<0x122, 0xf>(v));
+  v = merge(v, dpp_move<0x121, 0xf>(v));
   return v;
+}
+// All-reduce over the 64 lanes: rows first, then row 0 into row 1 and row 2 into row 3, then rows 0+1 into row 3, whose last lane is
+// read back to everyone.  A fixed order, every lane the same bits: results are deterministic run to run.  Must be called by all 64
+// lanes of the wave (no divergence around it).
+template <typename T, typename Merge> __device__ __forceinline__ T wave_reduce(T v, Merge merge) {
+  v = row16_reduce(v, merge);
+  const int row = (threadIdx.x & (kWave - 1)) >> 4;
+  T t = dpp_move<0x142, 0xa>(v);
+  v = (row & 1) ? merge(v, t) : v;
+  t = dpp_move<0x143, 0xc>(v);
+  v = (row >= 2) ? merge(v, t) : v;
+  return wave_read_lane63(v);
 }
 
 // Reduce over a workgroup of NWAVES*64 threads.  `lds` must hold NWAVES elements.  Every thread

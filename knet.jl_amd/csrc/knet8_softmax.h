@@ -225,13 +225,12 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_merge(MaxSum<T> a,
   MaxSum<T> r = {M, sa + sb};
   return r;
 }
+// Over a wave: the max first, one rescaling of the lane's sum to it, then the sums -- one exp per lane instead of two per butterfly step.
 template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum<T> v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    MaxSum<T> o = {__shfl_xor(v.m, off, kWave), __shfl_xor(v.s, off, kWave)};
-    v = ms_merge(v, o);
-  }
-  return v;
+  const T M = wave_reduce(v.m, [](T a, T b) { return a > b ? a : b; });
+  const T s = v.m == M ? v.s : v.s * dev_exp(v.m - M);   // a lane holding only -inf padding has s = 0: 0 * exp(-inf) = 0
+  MaxSum<T> r = {M, wave_reduce(s, [](T a, T b) { return a + b; })};
+  return r;
 }
 
 // The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
@@ -403,8 +402,12 @@ __global__ __launch_bounds__(1024) void softmax_col_stream_kernel(long m, long n
     }
   }
   if (Algo::kNeedMax) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) maxsum_merge(mx, s, __shfl_xor(mx, off), __shfl_xor(s, off));
+    {
+      MaxSum<T> ms = {mx, s};
+      ms = ms_wave_reduce(ms);
+      mx = ms.m;
+      s = ms.s;
+    }
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     if (lane == 0) { lds[0][wave] = mx; lds[1][wave] = s; }
     __syncthreads();
