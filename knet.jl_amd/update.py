@@ -79,6 +79,23 @@ def update_(w, g, p=None, lr=0.1, gclip=0):
     ``update!(x::Param, g)`` uses the parameter's own optimizer ``x.opt``; without any optimizer the step is SGD with
     ``lr`` and ``gclip`` (src/train20/update.jl:470-476); a gradient of ``None`` (the parameter took no part) changes nothing."""
     from .autograd import Param
+    if isinstance(w, dict):                      # update!(w::AbstractDict, g::AbstractDict, p::AbstractDict): g may have fewer keys (update.jl:497-503)
+        if not isinstance(g, dict) or not isinstance(p, dict):
+            raise TypeError("MethodError: update! of a Dict needs Dicts of gradients and optimizers")
+        for key in g:
+            update_(w[key], g[key], p[key])
+        return w
+    if isinstance(w, (list, tuple)):             # arrays, tuples, iterators in general (update.jl:479-494)
+        if g is None:
+            return w
+        ps = [p] * len(w) if (p is None or isinstance(p, _Opt)) else list(p)
+        if isinstance(p, _Opt) and not isinstance(p, SGD):
+            raise TypeError("Bad args: one optimizer state for several weight arrays")
+        if not (len(w) == len(g) == len(ps)):
+            raise ValueError("weight, gradient, and optimization parameters not the same length.")
+        for wi, gi, pi in zip(w, g, ps):
+            update_(wi, gi, pi, lr=lr, gclip=gclip)
+        return w
     if isinstance(w, Param):
         if p is None:
             p = w.opt

@@ -75,3 +75,58 @@ def test_training_loop_reduces_the_loss(knet):
             for p in ws:
                 knet.update_(p.value, knet.grad(J, p), p.opt)
         assert losses[-1] < 0.6 * losses[0], (type(opt).__name__, losses[0], losses[-1])
+
+
+def _rosenbrock(knet, x):
+    """sum(abs2.(1 .- x[1:end-1]) .+ 100 .* abs2.(x[2:end] .- abs2.(x[1:end-1])))  (test/update.jl:11), through the tape."""
+    n = knet.value(x).length
+    a, b = knet.getindex(x, (1, n - 1)), knet.getindex(x, (2, n))
+    t1 = knet.sub(1, a)
+    t2 = knet.sub(b, knet.mul(a, a))
+    return knet.sum(knet.add(knet.mul(t1, t1), knet.mul(100, knet.mul(t2, t2))))
+
+
+def _rosenopt(knet, weights, opts, form, ftol=1e-1, xtol=1e-10, maxiter=10000):
+    """The loop of test/update.jl:27-46: gradient and value of the summed Rosenbrock functions, then update!(w, g, p) with the weights,
+    gradients and optimizers held as one array, a tuple, a list or a dict."""
+    ps = [knet.Param(knet.KnetArray(w.copy())) for w in weights]
+    i, prev, cur = 1, 0.0, 1.0
+    while i <= maxiter and abs(cur - prev) > xtol and cur > ftol:
+        prev = cur
+        J = knet.diff(lambda: _rosenbrock(knet, ps[0]) if len(ps) == 1 else knet.add(_rosenbrock(knet, ps[0]), _rosenbrock(knet, ps[1])))
+        cur = float(knet.value(J))
+        ws, gs = [p.value for p in ps], [knet.grad(J, p) for p in ps]
+        if form == "array":
+            knet.update_(ws[0], gs[0], opts[0])
+        elif form == "tuple":
+            knet.update_(tuple(ws), tuple(gs), tuple(opts))
+        elif form == "list":
+            knet.update_(ws, gs, list(opts))
+        else:
+            knet.update_(dict(a=ws[0], b=ws[1]), dict(a=gs[0], b=gs[1]), dict(a=opts[0], b=opts[1]))
+        i += 1
+    return cur <= ftol, i - 1
+
+
+def test_every_optimizer_minimises_the_rosenbrock_function(knet):
+    """test/update.jl:48-75 on KnetArrays: each optimizer with the reference's hyper-parameters brings the 6-dimensional Rosenbrock
+    function below 0.1 within 10 000 steps, for a single array and for tuples, lists and dicts of arrays.  (The reference notes that
+    the test depends on the random start; this start converges for all of them in a CPU simulation of the same loop.)"""
+    rng = np.random.default_rng(7)
+    w, v = rng.standard_normal(6), 10 * rng.standard_normal(6)
+    adam = lambda: knet.Adam(lr=0.005, beta1=0.9, beta2=0.95, eps=1e-8)
+    for make in (lambda: knet.SGD(lr=0.001), lambda: knet.Momentum(lr=0.00025, gamma=0.95), lambda: knet.Nesterov(lr=0.00025, gamma=0.95), adam,
+                 lambda: knet.Adagrad(lr=0.4, eps=1e-6), lambda: knet.Adadelta(lr=0.4, rho=0.5, eps=1e-6), lambda: knet.Rmsprop(lr=0.005, rho=0.9, eps=1e-6)):
+        ok, steps = _rosenopt(knet, [w], [make()], "array")
+        assert ok, (type(make()).__name__, steps)
+    for form in ("tuple", "list", "dict"):
+        ok, steps = _rosenopt(knet, [w, v], [adam(), adam()], form)
+        assert ok, (form, steps)
+    # update! with mismatched containers is an error; a missing gradient leaves the weights alone
+    a = knet.KnetArray(w.copy())
+    with pytest.raises(ValueError):
+        knet.update_([a, a], [a], [adam(), adam()])
+    with pytest.raises(TypeError):
+        knet.update_(dict(a=a), [a], dict(a=adam()))
+    assert knet.update_([a], None, [adam()]) == [a]
+    knet.libknet8().check()
