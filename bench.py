@@ -439,42 +439,45 @@ def cpu_side_table():
 
 
 def cpu_baseline():
-    """The oracle's *back loops (plain C, one thread) on a bounded sample of the config-2 workload."""
+    """The oracle's *back loops (plain C, one thread) on one pass of the config-2 workload at its real size (about 4 s of timed loops,
+    20-30 s with the generation of the inputs and the forward passes that produce y)."""
     from oracle import knet_oracle as ko
     rng = np.random.default_rng(0)
     total_bytes, total_s = 0, 0.0
-    for dt, n in ((np.float32, 1 << 25), (np.float64, 1 << 24)):
-        x = rng.standard_normal(n).astype(dt)
-        dy = rng.standard_normal(n).astype(dt)
+    x32 = rng.standard_normal(1 << 28, dtype=np.float32)
+    dy32 = rng.standard_normal(1 << 28, dtype=np.float32)
+    for dt, n in ((np.float32, 1 << 28), (np.float64, 1 << 27)):
+        x = x32 if dt == np.float32 else x32[:n].astype(dt)
+        dy = dy32 if dt == np.float32 else dy32[:n].astype(dt)
+        out = np.zeros(n, dt)   # touched once: the timed loops write into resident pages, as the GPU kernels do
         for back, fwd in OPS:
             y = ko.unary(fwd, x)
             ko.back11(back, dy[:1024], y[:1024])
             t0 = time.perf_counter()
-            ko.back11(back, dy, y)
+            ko.back11(back, dy, y, out=out)
             total_s += time.perf_counter() - t0
             total_bytes += 3 * n * x.itemsize
     # The same loops over 16 equal slices in 16 threads (ctypes drops the interpreter lock during the call): what the port reaches
     # on the host share of a one-GPU box when every core streams; a restatement's figure, not Knet's, whose Array path is one thread.
     from concurrent.futures import ThreadPoolExecutor
     threads = 16
-    x = rng.standard_normal(1 << 25).astype(np.float32)
-    dy = rng.standard_normal(1 << 25).astype(np.float32)
+    x, dy, out32 = x32[:1 << 27], dy32[:1 << 27], np.zeros(1 << 27, np.float32)
     cut = np.linspace(0, x.size, threads + 1).astype(np.int64)
     par_bytes, par_s = 0, 0.0
     with ThreadPoolExecutor(threads) as pool:
         for back, fwd in OPS:
             y = ko.unary(fwd, x)
-            parts = [(dy[a:b], y[a:b]) for a, b in zip(cut[:-1], cut[1:])]
+            parts = [(dy[a:b], y[a:b], out32[a:b]) for a, b in zip(cut[:-1], cut[1:])]
             list(pool.map(lambda p: ko.back11(back, p[0][:1024], p[1][:1024]), parts))
             t0 = time.perf_counter()
-            list(pool.map(lambda p: ko.back11(back, p[0], p[1]), parts))
+            list(pool.map(lambda p: ko.back11(back, p[0], p[1], out=p[2]), parts))
             par_s += time.perf_counter() - t0
             par_bytes += 3 * x.size * x.itemsize
     return {"value": total_bytes / total_s * 1e-9, "unit": "GB/s", "cores": 1, "kind": "port",
             "all_cores": {"value": par_bytes / par_s * 1e-9, "unit": "GB/s", "cores": threads,
-                          "sample": "the five fp32 *back loops on 2^25 elements cut into 16 slices, one thread each"},
-            "sample": "the five *back loops of oracle/knet_cpu.c (gcc -O2, no contraction) on 2^25 fp32 and 2^24 fp64 elements, one pass each, "
-                      "timed through ctypes including the output allocation; Knet's CPU Array path for these ops is single-threaded broadcast"}
+                          "sample": "the five fp32 *back loops on 2^27 elements cut into 16 slices, one thread each"},
+            "sample": "one pass of the whole config-2 workload: the five *back loops of oracle/knet_cpu.c (gcc -O2, no contraction) on 2^28 fp32 and 2^27 fp64 elements, "
+                      "timed through ctypes, outputs written into touched memory; Knet's CPU Array path for these ops is single-threaded broadcast"}
 
 
 def main():
