@@ -18,7 +18,7 @@ from .softmax import logsoftmax, softmax, logp, logsumexp, logsoftmaxback, softm
 from .cat import cat, hcat, vcat
 from .statistics import mean, var, std, varm, stdm, norm, isequal, isapprox
 from .random import seed_, rand_, randn_, RngState
-from .loss import nll, findindices, accuracy, ungetindex, bce, logistic
+from .loss import nll, findindices, accuracy, zeroone, ungetindex, bce, logistic
 from .indexing import (getcols, getrows, setcols_, setrows_, addcols_, addrows_, setents_, getindex2, setindex2_, icat, concat,
                        getindex, setindex_)
 from .dropout import dropout, dropback, dropout_, dropback_

@@ -124,12 +124,26 @@ def _nll_fused(scores, labels, dims=1, count=None):
     return loss, back
 
 
-def nll(scores, labels, dims=1, average=True, fused=False, count=None):
-    """``nll(scores, labels; dims=1, average=true)`` (src/ops20/loss.jl:37-41).
+def _over_data(fn, model, data, dims, average, kw):
+    """``sum``/``count`` of ``fn(model(x), y; average=false)`` over an iterable of ``(x, y)`` pairs (src/ops20/loss.jl:159-166,185-193)."""
+    total, cnt = 0, 0
+    for x, y in data:
+        z, n = fn(model(x, **kw), y, dims=dims, average=False)
+        total, cnt = total + z, cnt + n
+    return total / cnt if average else (total, cnt)
+
+
+def nll(scores, labels=None, dims=1, average=True, fused=False, count=None, data=None, **kw):
+    """``nll(scores, labels; dims=1, average=true)`` (src/ops20/loss.jl:37-41), and ``nll(model; data, dims, average, o...)``
+    (``:159-166``; also the deprecated two-argument ``nll(model, data)``, ``:199-202``): the loss of a callable model over a dataset.
 
     ``fused=False`` follows the reference step by step (logsoftmax, gather, sum); ``fused=True`` computes the loss
     and, when recording, the gradient with the single-pass kernel (same result within rounding).
     """
+    if callable(scores) and not isinstance(scores, KnetArray):
+        return _over_data(nll, scores, data if data is not None else labels, dims, average, kw)
+    if kw:
+        raise TypeError("MethodError: nll got unexpected keyword arguments %r" % sorted(kw))
     if isinstance(labels, KnetArray) and not fused:
         raise TypeError("MethodError: nll takes host labels (an integer array), as in the reference; device labels need fused=True")
     if fused and average:
@@ -183,9 +197,18 @@ def logistic(scores, labels, average=True):
     return bce(scores, (np.asarray(labels) + 1) // 2, average=average)
 
 
-def accuracy(scores, labels, dims=1, average=True):
+def zeroone(*a, **kw):
+    """``zeroone(x...) = 1 - accuracy(x...)`` (src/ops20/loss.jl:232-235)."""
+    return 1 - accuracy(*a, **kw)
+
+
+def accuracy(scores, labels=None, dims=1, average=True, data=None, **kw):
     """Ratio of instances whose labelled class has the largest score (src/ops20/loss.jl:52-62); as in the
-    reference the scores are brought to the host for ``findmax``."""
+    reference the scores are brought to the host for ``findmax``.  ``accuracy(model; data, ...)`` (``:185-193``) sums over a dataset."""
+    if callable(scores) and not isinstance(scores, KnetArray):
+        return _over_data(accuracy, scores, data if data is not None else labels, dims, average, kw)
+    if kw:
+        raise TypeError("MethodError: accuracy got unexpected keyword arguments %r" % sorted(kw))
     s = value(scores).to_numpy()
     lab = np.asarray(labels).ravel(order="F")
     pred = s.argmax(axis=0 if dims == 1 else s.ndim - 1).ravel(order="F") + 1

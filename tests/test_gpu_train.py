@@ -191,3 +191,30 @@ def test_params_update_of_a_param_converge_and_train(knet):
     knet.train_(net2, knet.minibatch(X, labels, 10))                          # one epoch of Adam: epochs(data, 1) stops before the 4th update
     assert net2.w.opt.t == 3 and not bits_equal(knet.Array(net2.w.value), w0)
     knet.libknet8().check()
+
+
+def test_nll_and_accuracy_of_a_model_over_a_dataset(knet):
+    """``nll(model; data)``, ``accuracy(model; data)`` (src/ops20/loss.jl:159-193) and ``zeroone``: totals over the minibatches divided by
+    the number of instances that were not skipped, against numpy on the whole dataset."""
+    rng = np.random.default_rng(84)
+    X = rng.standard_normal((6, 40)).astype(np.float32)
+    W = rng.standard_normal((3, 6)).astype(np.float32)
+    labels = rng.integers(1, 4, size=40)
+    labels[[3, 17, 29]] = 0                                   # skipped instances
+    wd = knet.KnetArray(W)
+    model = lambda x: knet.matmul(wd, x)
+    z = W.astype(np.float64) @ X.astype(np.float64)
+    lse = np.log(np.exp(z - z.max(axis=0)).sum(axis=0)) + z.max(axis=0)
+    keep = labels > 0
+    want_nll = float((lse - z[np.maximum(labels, 1) - 1, np.arange(40)])[keep].sum() / keep.sum())
+    want_acc = float(((z.argmax(axis=0) + 1) == labels)[keep].mean())
+    data = knet.minibatch(X, labels, 8)
+    assert abs(float(knet.nll(model, data=data)) - want_nll) <= 1e-5 * want_nll
+    total, cnt = knet.nll(model, data=data, average=False)
+    assert cnt == 37 and abs(float(total) / cnt - want_nll) <= 1e-5 * want_nll
+    assert abs(knet.accuracy(model, data=data) - want_acc) <= 1e-12 and knet.accuracy(model, data=data, average=False)[1] == 37
+    assert abs(knet.nll(model, data) - knet.nll(model, data=data)) == 0 and knet.accuracy(model, data) == knet.accuracy(model, data=data)
+    assert abs(knet.zeroone(model, data=data) - (1 - want_acc)) <= 1e-12
+    scores = model(knet.KnetArray(X))
+    assert abs(knet.zeroone(scores, labels) - (1 - want_acc)) <= 1e-12
+    knet.libknet8().check()
