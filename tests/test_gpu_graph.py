@@ -145,3 +145,41 @@ def test_a_product_first_seen_under_capture_is_planned_without_timing(knet):
         lib.check()
     finally:
         lib.fn["knet8_stream_destroy"](stream)
+
+
+def test_captured_step_with_fused_layers_matches_the_oracle_on_every_replay(knet, oracle):
+    """The same MLP step written with the one-launch layers (``dense`` forward/backward, ``dense_nll`` for the output layer: four launches)
+    captured and replayed, with an optimizer step between replays."""
+    rng = np.random.default_rng(83)
+    lib = knet.libknet8()
+    old_stream = lib.stream
+    try:
+        sizes = [784, 64, 10]
+        ws = []
+        for i in range(2):
+            ws += [(rng.standard_normal((sizes[i + 1], sizes[i])) * 0.05).astype(np.float32), (rng.standard_normal((sizes[i + 1], 1)) * 0.1).astype(np.float32)]
+        params = [knet.Param(knet.KnetArray(w)) for w in ws]
+        x = knet.KnetArray(rng.random((784, 100), dtype=np.float32))
+        labels_h = rng.integers(1, 11, size=100)
+        labels = knet.KnetArray(labels_h.astype(np.int32))
+
+        def step():
+            J = knet.diff(lambda: knet.dense_nll(params[2], knet.dense(params[0], x, params[1], act="relu"), params[3], labels, count=100))
+            return [J.value] + [knet.grad(J, p) for p in params]
+
+        g = knet.capture(step)
+        for r in range(3):
+            loss_ref, grads_ref = oracle.mlp_backward(ws, knet.Array(x), labels_h)
+            g.replay()
+            knet.synchronize()
+            out = [knet.Array(o) for o in g.outputs]
+            assert abs(float(out[0][0]) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref)), r
+            for got, want in zip(out[1:], grads_ref):
+                assert rel(got.reshape(want.shape), want) <= 1e-4, r
+            for p, gr in zip(params, g.outputs[1:]):
+                knet.update_(p.value, gr, knet.SGD(lr=0.2))
+            ws = [knet.Array(p.value) for p in params]
+        del g
+        lib.check()
+    finally:
+        lib.stream = old_stream
