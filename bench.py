@@ -310,7 +310,7 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=F
     """Forward + backward of an MLP through KnetArray and the tape.  graph=True: the step is captured once into a hipGraph
     (labels resident on the device, loss kept on the device) and `steps` replays are timed.  layers=True: each hidden layer's
     bias add, relu and dropout (and their gradients plus the bias gradient) run as one fused launch each way.  head=True: the
-    output layer's loss and gradients come from one launch after its product (dense_nll)."""
+    output layer's product, loss and gradients come from one launch (dense_nll)."""
     rng = np.random.default_rng(0)
     lib = K.libknet8()
     old_stream = lib.stream
@@ -534,11 +534,11 @@ def main():
             "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
             "config1 same graph with dense layers (product, bias and relu in one launch)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
-            "config1 eager with dense layers and dense_nll (4 launches per step, loss left on the device)":
+            "config1 eager with dense layers and dense_nll (3 launches per step, loss left on the device)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 1000, True, layers=True, head=True),
-            "config1 same graph, output layer's loss and gradients in one launch (dense_nll: 4 launches per step)":
+            "config1 same graph, output layer forward + loss + gradients in one launch (dense_nll: 3 launches per step)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True, head=True),
-            "config1 same step from a compiled C99 host through the C ABI (eager, 4 launches: fused layer kernels forward and backward, loss folded into the output layer's backward)": c_host_steps(K),
+            "config1 same step from a compiled C99 host through the C ABI (eager, 3 launches: hidden layer forward, output layer forward + loss + backward, hidden layer backward)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),

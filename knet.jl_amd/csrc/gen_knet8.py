@@ -465,6 +465,16 @@ def gen_elementwise():
                  (T + "*", "dW"), (T + "*", "db"), (T + "*", "dx"), (T + "*", "loss"), (T + "*", "mean")], None,
                 "nll -> logsoftmax -> getindex (src/ops20/loss.jl:37-41) + sum_S_21 + gemm! x 2, src/knetarrays/linalg.jl:11-18",
                 body="  const int rc = launch_dense_nll_back<%s>(stream, m, n, k, W, x, z, labels, scale, dW, db, dx, loss, mean);\n  knet8::check_launch(\"dense_nll_back_%s\");\n  return rc;" % (T, S))
+    o.decl.append("/* dense_head_S: a classifier's output layer forward and backward in one launch.  From W (m x k), bias (m), the layer's input x (k x n)\n"
+                  "   and the labels: the scores z = W*x + bias (written to z when z is not NULL), and everything dense_nll_back_S writes from them\n"
+                  "   (loss, mean, dW, db, dx).  m <= 16 classes, n <= 512 instances (fp64: 256), dW required; returns 0 when done, 1 when not applicable\n"
+                  "   (nothing launched: use gemm_bias_act_S + dense_nll_back_S), -1 on bad arguments.  No libknet8 counterpart. */")
+    for T, S in TYPES:
+        o.entry("dense_head_%s" % S, "int",
+                [("int", "m"), ("int", "n"), ("int", "k"), (T + "*", "W"), (T + "*", "bias"), (T + "*", "x"), ("int*", "labels"), (T, "scale"),
+                 (T + "*", "dW"), (T + "*", "db"), (T + "*", "dx"), (T + "*", "loss"), (T + "*", "mean"), (T + "*", "z")], None,
+                "gemm! + bias broadcast (src/knetarrays/linalg.jl:26-52, binary.jl:61-95) + the chain of src/ops20/loss.jl:37-41 + sum_S_21 + gemm! x 2",
+                body="  const int rc = launch_dense_head<%s>(stream, m, n, k, W, bias, x, labels, scale, dW, db, dx, loss, mean, z);\n  knet8::check_launch(\"dense_head_%s\");\n  return rc;" % (T, S))
     for T, S in TYPES:
         o.entry("biasreludrop_%s" % S, "void", [("int", "m"), ("int", "n"), (T, "p"), (T + "*", "z"), (T + "*", "b"), (T + "*", "y")],
                 "launch_bias_act<%s, true>(stream, m, n, z, b, y, BiasReluDrop<%s>{p, %s(1) - p})" % (T, T, T),

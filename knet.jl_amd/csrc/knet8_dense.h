@@ -64,15 +64,21 @@ __device__ __forceinline__ T nll_dz(T e, T sum, int lab, int cls, T scale) {
   return ((cls + 1 == lab) ? -scale : T(0)) + e * (nll_rcp(sum) * scale);
 }
 
-// NLL = false: y and dy are the layer's output and its gradient.  NLL = true: y holds the scores, dy is unused, dz comes from
-// (labels, scale) and the per-column loss goes to `loss` (m <= 16: a column's classes fit one tile edge).
-template <typename T, bool NLL>
+// MODE 0: y and dy are the layer's output and its gradient.  MODE 1 (loss form): y holds the scores, dy is unused, dz comes from
+// (labels, scale) and the per-column loss goes to `loss` (m <= 16: a column's classes fit one tile edge).  MODE 2 (head form): as 1, but
+// the scores are not read: every workgroup first computes the scores of the columns it needs, z = W*x + bias, into LDS (all n
+// columns for a tile of dW, its own sixteen for a tile of dx) -- the output layer's forward product rides in its backward launch.
+template <typename T> struct DenseHead { static constexpr int kCols = 32768 / (int)sizeof(T) / kDbTile; };   // 32 KB of scores in LDS
+
+template <typename T, int MODE>
 __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, int m, int n, int k, const T* __restrict__ W, const T* __restrict__ x,
                                                                       const T* __restrict__ y, const T* __restrict__ dy, T* __restrict__ dW,
                                                                       T* __restrict__ db, T* __restrict__ dx, int tiles_w, int tiles_w_m, int tiles_x_m,
                                                                       int kslice_w, int kslice_x, bool vecw, bool vecz, const int* __restrict__ labels, T scale,
-                                                                      T* __restrict__ loss, T* __restrict__ mean) {
+                                                                      T* __restrict__ loss, T* __restrict__ mean, const T* __restrict__ bias, T* __restrict__ zout) {
   constexpr int TS = kDbTile, KS = kDbWaves;
+  constexpr bool NLL = MODE >= 1, HEAD = MODE == 2;
+  __shared__ T zs[HEAD ? DenseHead<T>::kCols * TS : 1];   // zs[column * 16 + class]
   __shared__ T part[KS][TS * TS];      // part[w][j*16 + i]
   __shared__ T rs[KS][4][TS];          // row-sum parts
   __shared__ T ls[KS];                 // loss parts
@@ -96,6 +102,36 @@ __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, i
   const bool first = job_w && j0 == 0;          // the tiles that walk all of dz once: row sums and, in the loss form, the losses
   const bool sums = first && db != nullptr;
   const T ninf = T(-INFINITY);
+  // Head form: the scores of the columns this workgroup needs, into LDS.  Called once by every wave (it contains a barrier), after the
+  // loads of the second phase that do not depend on the scores have been issued, so that the two memory round trips overlap.
+  auto compute_scores = [&]() {
+    const int c0 = job_w ? 0 : j0;
+    const int c1 = job_w ? n : (j0 + TS < n ? j0 + TS : n);
+    const bool rok = r16 < m;                       // lane's class row of W
+    for (int t = w; 16 * t < c1 - c0; t += KS) {   // one wave per tile of sixteen columns
+      const int col = c0 + 16 * t + r16;
+      const bool cok = col < c1;
+      const T* wp = W + (rok ? r16 : 0);
+      const T* xp = x + (long)(cok ? col : 0) * k;
+      typename Mfma16<T>::Acc za = {T(0), T(0), T(0), T(0)};
+#pragma unroll 4
+      for (int kc = 0; kc < k; kc += 16) {
+        T a[4], b[4];
+        mfma_load4<T, false>(a, wp, m, kc + 4 * kq, k, rok, false);   // W(class, kk): contiguous along the classes
+        mfma_load4<T, true>(b, xp, 1, kc + 4 * kq, k, cok, vecz);     // x(kk, col): contiguous along kk
+#pragma unroll
+        for (int c = 0; c < 4; c++) za = Mfma16<T>::run(a[c], b[c], za);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int row = Mfma16<T>::row(r, kq);
+        zs[(16 * t + r16) * TS + row] = (row < m && cok) ? za[r] + bias[row] : ninf;
+      }
+    }
+    __syncthreads();
+    if (first && zout != nullptr)
+      for (long o = threadIdx.x; o < (long)m * n; o += KS * kWave) zout[o] = zs[(o / m) * TS + (o % m)];
+  };
   if (job_w) {
     // A(i, kk) = dz(i, kk) and B(kk, j) = x(j, kk): both contiguous along the tile edge
     const T* gp = NLL ? nullptr : dy + (iok ? i : 0);
@@ -113,12 +149,29 @@ __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, i
         for (int c = 0; c < NC; c++) {
           const int kk = col(kc, c);
           const bool kok = kk < kend;
-          zn[c] = (iok && kok) ? y[i + (long)kk * m] : ninf;
+          if (HEAD) zn[c] = (iok && kok) ? zs[kk * TS + i] : ninf;
+          else zn[c] = (iok && kok) ? y[i + (long)kk * m] : ninf;
           ln[c] = kok ? labels[kk] : 0;
           xn[c] = (jok && kok) ? xp[(long)kk * k] : T(0);
         }
       };
-      fetch(kbeg);
+      if (HEAD) {   // labels and x of the first step first, the scores' product behind them, then the scores from LDS
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+          const int kk = col(kbeg, c);
+          const bool kok = kk < kend;
+          ln[c] = kok ? labels[kk] : 0;
+          xn[c] = (jok && kok) ? xp[(long)kk * k] : T(0);
+        }
+        compute_scores();
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+          const int kk = col(kbeg, c);
+          zn[c] = (iok && kk < kend) ? zs[kk * TS + i] : ninf;
+        }
+      } else {
+        fetch(kbeg);
+      }
       for (int kc = kbeg; kc < kend; kc += 16 * CH) {
         T z[NC], a[NC], b[NC], lj[NC];
         int lab[NC];
@@ -176,13 +229,19 @@ __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, i
   } else {
     // A(i, kk) = W(kk, i) and B(kk, j) = dz(kk, j): both contiguous along the inner dimension
     const T* wp = W + (long)(iok ? i : 0) * m;
-    const T* gp = (NLL ? y : dy) + (long)(jok ? j : 0) * m;
+    const T* gp = HEAD ? nullptr : (NLL ? y : dy) + (long)(jok ? j : 0) * m;
     const T* yp = relu ? y + (long)(jok ? j : 0) * m : nullptr;
+    if (HEAD) compute_scores();   // every wave, also those whose slice of the (short) inner dimension is empty
 #pragma unroll 2
     for (int kc = kbeg; kc < kend; kc += 16) {
       T a[4], b[4];
       mfma_load4<T, true>(a, wp, 1, kc + 4 * kq, kend, iok, vecw);
-      mfma_load4<T, true>(b, gp, 1, kc + 4 * kq, kend, jok, vecz);
+      if (HEAD) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) b[c] = (jok && kc + 4 * kq + c < kend) ? zs[r16 * TS + kc + 4 * kq + c] : T(0);
+      } else {
+        mfma_load4<T, true>(b, gp, 1, kc + 4 * kq, kend, jok, vecz);
+      }
       if (NLL) {
         // m <= 16: this one step holds every class of column j, four per lane in the lanes j, j+16, j+32, j+48
         T z[4], mx = ninf;
@@ -249,9 +308,10 @@ __global__ __launch_bounds__(kDbWaves * kWave) void dense_back_kernel(int act, i
 
 // 0: done.  1: not applicable (a product too large for the small kernels, or db wanted without dW): nothing was launched and the
 // caller takes the separate launches.  -1: bad arguments (recorded).
-template <typename T, bool NLL>
+template <typename T, int MODE>
 inline int launch_dense_back_impl(hipStream_t stream, int act, int m, int n, int k, const T* W, const T* x, const T* y, const T* dy, T* dW, T* db, T* dx,
-                                  const int* labels, T scale, T* loss, T* mean) {
+                                  const int* labels, T scale, T* loss, T* mean, const T* bias = nullptr, T* zout = nullptr) {
+  constexpr bool NLL = MODE >= 1;
   // both products have 2*m*n*k flop; kernel durations against reluback_biasgrad + two gemm launches (us, kernel trace): 64x100x784
   // 3.6/11.3, 256^3 5.2/12.6, 300^3 7.3/14.8, 512x128x512 9.6/14.1, 400^3 11.9/18.8, 512^3 20.8/26.2 -- one launch wins over the whole range of
   // the small-product kernels (2.7e8 flop); beyond it the separate launches reach the vendor library's large tiles
@@ -264,9 +324,10 @@ inline int launch_dense_back_impl(hipStream_t stream, int act, int m, int n, int
   auto slice = [](int K) { const int steps = (K + 15) / 16; return ((steps + kDbWaves - 1) / kDbWaves) * 16; };
   // 16-byte (fp64: 32-byte) loads along the inner dimension of dx = W'*dz need columns of W, dy and y that start on such a boundary
   const bool vecw = W != nullptr && mfma_vec_ok(W, m);
-  const bool vecz = NLL ? mfma_vec_ok(y, m) : (mfma_vec_ok(dy, m) && (act != 1 || mfma_vec_ok(y, m)));
-  hipLaunchKernelGGL((dense_back_kernel<T, NLL>), dim3((unsigned)(tiles_w + tiles_x)), dim3(kDbWaves * kWave), 0, stream, act, m, n, k, W, x, y, dy, dW, db, dx,
-                     tiles_w, tw_m, tx_m, slice(n), slice(m), vecw, vecz, labels, scale, loss, mean);
+  // (head form: the flag covers the loads of x along its inner dimension instead)
+  const bool vecz = MODE == 2 ? mfma_vec_ok(x, k) : NLL ? mfma_vec_ok(y, m) : (mfma_vec_ok(dy, m) && (act != 1 || mfma_vec_ok(y, m)));
+  hipLaunchKernelGGL((dense_back_kernel<T, MODE>), dim3((unsigned)(tiles_w + tiles_x)), dim3(kDbWaves * kWave), 0, stream, act, m, n, k, W, x, y, dy, dW, db, dx,
+                     tiles_w, tw_m, tx_m, slice(n), slice(m), vecw, vecz, labels, scale, loss, mean, bias, zout);
   return 0;
 }
 
@@ -278,7 +339,7 @@ inline int launch_dense_back(hipStream_t stream, int act, int m, int n, int k, c
     record_error("dense_back: missing operand");
     return -1;
   }
-  return launch_dense_back_impl<T, false>(stream, act, m, n, k, W, x, y, dy, dW, db, dx, nullptr, T(0), nullptr, nullptr);
+  return launch_dense_back_impl<T, 0>(stream, act, m, n, k, W, x, y, dy, dW, db, dx, nullptr, T(0), nullptr, nullptr);
 }
 
 // The classifier's output layer: scores z = W*x + b (m classes x n instances) and labels in, the loss per instance and the layer's
@@ -292,7 +353,21 @@ inline int launch_dense_nll_back(hipStream_t stream, int m, int n, int k, const 
     return -1;
   }
   if (m > kDbTile || ((loss != nullptr || mean != nullptr) && dW == nullptr)) return 1;
-  return launch_dense_back_impl<T, true>(stream, 0, m, n, k, W, x, z, nullptr, dW, db, dx, labels, scale, loss, mean);
+  return launch_dense_back_impl<T, 1>(stream, 0, m, n, k, W, x, z, nullptr, dW, db, dx, labels, scale, loss, mean);
+}
+
+// The head form: forward product included.  W (m x k), bias (m), x (k x n) in; the scores themselves are written to z when asked for.
+// At most 16 classes and DenseHead<T>::kCols instances (512 in fp32, 256 in fp64: their scores stay in LDS); dW is required.
+template <typename T>
+inline int launch_dense_head(hipStream_t stream, int m, int n, int k, const T* W, const T* bias, const T* x, const int* labels, T scale, T* dW, T* db,
+                             T* dx, T* loss, T* mean, T* z) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  if (W == nullptr || bias == nullptr || x == nullptr || labels == nullptr) {
+    record_error("dense_head: missing operand");
+    return -1;
+  }
+  if (m > kDbTile || n > DenseHead<T>::kCols || dW == nullptr) return 1;
+  return launch_dense_back_impl<T, 2>(stream, 0, m, n, k, W, x, nullptr, nullptr, dW, db, dx, labels, scale, loss, mean, bias, z);
 }
 
 }  // namespace knet8

@@ -95,3 +95,20 @@ for (T, S) in ((Float32, 32), (Float64, 64))
         return rc == 0
     end
 end
+
+# The same with the output layer's forward product inside the launch (dense_head_S): scores z = w*x .+ b are formed in the kernel (and
+# written to `z` when given).  At most 16 classes and 512 instances (Float64: 256); returns false when the library declines.
+for (T, S) in ((Float32, 32), (Float64, 64))
+    @eval function dense_head!(mean::KnetArray{$T}, dw::KnetArray{$T,2}, db::KnetArray{$T}, dx::Union{KnetArray{$T,2},Nothing},
+                               w::KnetArray{$T,2}, b::KnetArray{$T}, x::KnetArray{$T,2}, labels::KnetArray{Int32}, scale::Real;
+                               z::Union{KnetArray{$T,2},Nothing}=nothing)
+        m, k = size(w); n = size(x, 2)
+        @assert size(x, 1) == k && length(b) == m && length(labels) == n && size(dw) == (m, k) && length(db) == m
+        rc = ccall(($("dense_head_$(S)_stream"), LibKnet8.libknet8), Cint,
+                   (Cint, Cint, Cint, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{Cint}, $T, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{$T}, Ptr{Cvoid}),
+                   m, n, k, w, b, x, labels, $T(scale), dw, db, dx === nothing ? C_NULL : dx, C_NULL, mean, z === nothing ? C_NULL : z,
+                   LibKnet8.knet8_stream())
+        rc < 0 && LibKnet8.knet8_check()
+        return rc == 0
+    end
+end

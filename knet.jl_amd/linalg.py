@@ -108,15 +108,19 @@ def _dense_nll(w, x, b, labels, count):
     m, k, n = _size2(w, 1), _size2(w, 2), x2.size(2)
     lib = libknet8()
     c = w.ctype
-    z = w.similar((m, n))
-    rc = lib.call("gemm_bias_act_%s" % w.suffix, b"N", b"N", m, n, k, c(1), w.ptr, m, x2.ptr, k, b.ptr, 0, z.ptr, m)
-    if rc != 0:
-        lib.check()
-        raise RuntimeError("gemm_bias_act failed")
     dW, db, dx, mean = w.similar((m, k)), b.similar(), x2.similar(), w.similar((1,))
     T = w.dtype.type
     scale = T(1) / T(count) if count else T(np.inf)
-    rc = lib.call("dense_nll_back_%s" % w.suffix, m, n, k, w.ptr, x2.ptr, z.ptr, labels.ptr, c(scale), dW.ptr, db.ptr, dx.ptr, None, mean.ptr)
+    # forward product included when the scores of all instances fit the kernel's LDS (dense_head_S); else product, then dense_nll_back_S
+    rc = 1
+    if n <= (512 if w.dtype == np.float32 else 256):
+        rc = lib.call("dense_head_%s" % w.suffix, m, n, k, w.ptr, b.ptr, x2.ptr, labels.ptr, c(scale), dW.ptr, db.ptr, dx.ptr, None, mean.ptr, None)
+    if rc == 1:
+        z = w.similar((m, n))
+        if lib.call("gemm_bias_act_%s" % w.suffix, b"N", b"N", m, n, k, c(1), w.ptr, m, x2.ptr, k, b.ptr, 0, z.ptr, m) != 0:
+            lib.check()
+            raise RuntimeError("gemm_bias_act failed")
+        rc = lib.call("dense_nll_back_%s" % w.suffix, m, n, k, w.ptr, x2.ptr, z.ptr, labels.ptr, c(scale), dW.ptr, db.ptr, dx.ptr, None, mean.ptr)
     if rc != 0:
         lib.check()
         raise RuntimeError("dense_nll_back declined (%d)" % rc)
@@ -132,8 +136,9 @@ def _dense_nll(w, x, b, labels, count):
 def dense_nll(w, x, b, labels, count=None):
     """``nll(w*x .+ b, labels)`` for a classifier's output layer: the average loss as a 1-element ``KnetArray`` (nothing synchronises
     with the host).  ``labels``: Int32 ``KnetArray`` of 1-based classes, 0 = skip; ``count``: number of non-zero labels (default: all).
-    With at most 16 classes and a layer of the small-kernel class the loss and the layer's three gradients come out of ONE launch
-    after the product (``dense_nll_back_S``: softmax, loss, dW, db and dx); otherwise this is ``nll(dense(w, x, b), labels; fused)``.
+    With at most 16 classes and a layer of the small-kernel class the loss and the layer's three gradients come out of ONE launch,
+    product included (``dense_head_S``, up to 512 instances; beyond, the product and then ``dense_nll_back_S``: softmax, loss, dW, db and
+    dx); otherwise this is ``nll(dense(w, x, b), labels; fused)``.
     The reference runs the chain of src/ops20/loss.jl:37-41 and src/knetarrays/linalg.jl:11-18 for it."""
     from .autograd import value as _value
     wv, xv = _value(w), _value(x)

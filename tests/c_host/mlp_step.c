@@ -26,17 +26,17 @@ static void up(void *d, const void *h, size_t bytes) {
 }
 
 struct net {
-  float *W1, *b1, *W2, *b2, *x, *y1, *s, *mean, *db2, *dW2, *dy1, *db1, *dW1;
+  float *W1, *b1, *W2, *b2, *x, *y1, *mean, *db2, *dW2, *dy1, *db1, *dW1;
   int *labels;
 };
 
 static void step(struct net *n, hipStream_t st) {
-  /* forward: y1 = relu(W1*x .+ b1); s = W2*y1 .+ b2 */
+  /* hidden layer forward: y1 = relu(W1*x .+ b1) */
   gemm_bias_act_32_stream('N', 'N', D1, NB, D0, 1.0f, n->W1, D1, n->x, D0, n->b1, 1, n->y1, D1, st);
-  gemm_bias_act_32_stream('N', 'N', D2, NB, D1, 1.0f, n->W2, D2, n->y1, D1, n->b2, 0, n->s, D2, st);
-  /* backward: one launch per layer (these entry points return 1 for layers outside the range of their kernel; these are not).
-   * Output layer: the mean loss, ds = (softmax(s) - onehot)/NB, dW2 = ds*y1', db2, dy1 = W2'*ds; hidden layer: dz1 = relu'(y1).*dy1, dW1, db1 */
-  if (dense_nll_back_32_stream(D2, NB, D1, n->W2, n->y1, n->s, n->labels, 1.0f / NB, n->dW2, n->db2, n->dy1, NULL, n->mean, st) != 0 ||
+  /* output layer, forward and backward in one launch: s = W2*y1 .+ b2 (kept inside the kernel), the mean loss, ds = (softmax(s) - onehot)/NB,
+   * dW2 = ds*y1', db2, dy1 = W2'*ds; then the hidden layer's backward: dz1 = relu'(y1).*dy1, dW1, db1.
+   * (These entry points return 1 for layers outside the range of their kernel; these are not.) */
+  if (dense_head_32_stream(D2, NB, D1, n->W2, n->b2, n->y1, n->labels, 1.0f / NB, n->dW2, n->db2, n->dy1, NULL, n->mean, NULL, st) != 0 ||
       dense_back_32_stream(1, D1, NB, D0, n->W1, n->x, n->y1, n->dy1, n->dW1, n->db1, NULL, st) != 0) {
     fprintf(stderr, "dense_back declined or failed\n");
     exit(4);
@@ -63,7 +63,7 @@ int main(int argc, char **argv) {
   if (knet8_device_count() < 1) { fprintf(stderr, "no device\n"); return 3; }
   struct net n;
   n.W1 = dev(nW1); n.b1 = dev(D1); n.W2 = dev(nW2); n.b2 = dev(D2); n.x = dev(nx);
-  n.y1 = dev(D1 * NB); n.s = dev(D2 * NB); n.mean = dev(1);
+  n.y1 = dev(D1 * NB); n.mean = dev(1);
   n.db2 = dev(D2); n.dW2 = dev(nW2); n.dy1 = dev(D1 * NB); n.db1 = dev(D1); n.dW1 = dev(nW1);
   n.labels = (int *)knet8_malloc(NB * sizeof(int));
   const float *p = h;

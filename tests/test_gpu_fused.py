@@ -323,7 +323,7 @@ def test_dense_nll_on_the_tape_matches_the_separate_primitives(knet):
     """``dense_nll(w, x, b, labels)`` against ``nll(dense(w, x, b), labels; fused)``: same loss and gradients (to rounding), for an output
     layer inside the fused range and for one outside it (more than 16 classes: the composition itself runs)."""
     rng = np.random.default_rng(47)
-    for m, n, k in ((10, 100, 64), (40, 30, 20)):
+    for m, n, k in ((10, 100, 64), (40, 30, 20), (10, 600, 20)):     # one launch; the composition; product + one launch (too many instances for one)
         W, b, x = (rng.standard_normal(s).astype(np.float32) for s in ((m, k), (m, 1), (k, n)))
         labels_h = rng.integers(1, m + 1, size=n)
         labels_h[:3] = 0
@@ -342,3 +342,54 @@ def test_dense_nll_on_the_tape_matches_the_separate_primitives(knet):
     with pytest.raises(TypeError):
         knet.dense_nll(knet.KnetArray(W), knet.KnetArray(x), knet.KnetArray(b), labels_h)
     knet.libknet8().check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_dense_head_forward_and_backward_of_the_output_layer_in_one_launch(knet, dt):
+    """dense_head_S: scores z = W*x + bias computed inside the launch that turns them into loss and gradients; against fp64 numpy and against
+    gemm_bias_act_S + dense_nll_back_S.  Ragged sizes, the instance limit (512 / 256 columns of scores in LDS), declined cases."""
+    rng = np.random.default_rng(48)
+    lib = knet.libknet8()
+    tol = 2e-5 if dt == np.float32 else 1e-12
+    c = knet.KnetArray(np.zeros(1, dt)).ctype
+    cols = 512 if dt == np.float32 else 256
+    for m, n, k in ((10, 100, 64), (16, 37, 33), (3, 5, 7), (1, 4, 4), (13, cols, 100), (10, 17, 784), (2, 1, 1)):
+        W = rng.standard_normal((m, k)).astype(dt)
+        b = rng.standard_normal(m).astype(dt)
+        x = rng.standard_normal((k, n)).astype(dt)
+        labels = rng.integers(1, m + 1, size=n).astype(np.int32)
+        if n > 3:
+            labels[rng.integers(0, n, size=max(1, n // 10))] = 0
+        count = max(int(np.count_nonzero(labels)), 1)
+        scale = 1.0 / count
+        z64 = W.astype(np.float64) @ x.astype(np.float64) + b.astype(np.float64)[:, None]
+        zmax = z64.max(axis=0)
+        lse = zmax + np.log(np.exp(z64 - zmax).sum(axis=0))
+        keep = labels > 0
+        want_loss = np.where(keep, lse - z64[np.maximum(labels, 1) - 1, np.arange(n)], 0.0)
+        onehot = np.zeros((m, n))
+        onehot[np.maximum(labels, 1) - 1, np.arange(n)] = 1
+        dz = np.where(keep, (np.exp(z64 - lse) - onehot) * scale, 0.0)
+        want = (dz @ x.astype(np.float64).T, dz.sum(axis=1), W.astype(np.float64).T @ dz, want_loss, np.array([want_loss.sum() * scale]), z64)
+        Wd, bd, xd, ld = knet.KnetArray(W), knet.KnetArray(b), knet.KnetArray(x), knet.KnetArray(labels)
+        for full in (True, False):
+            outs = [knet.KnetArray(np.full(s, 7, dt)) for s in ((m, k), (m,), (k, n), (n,), (1,), (m, n))]
+            ptrs = [o.ptr for o in outs] if full else [outs[0].ptr, None, outs[2].ptr, None, outs[4].ptr, None]
+            assert lib.call("dense_head_%s" % Wd.suffix, m, n, k, Wd.ptr, bd.ptr, xd.ptr, ld.ptr, c(scale), *ptrs) == 0
+            for idx, (got, w) in enumerate(zip(outs, want)):
+                if ptrs[idx] is not None:
+                    g = knet.Array(got)
+                    zscale = max(np.abs(w).max(), 1.0) * (np.sqrt(k) if idx == 5 else 1.0)
+                    assert np.abs(g - w.reshape(g.shape)).max() <= tol * zscale * 4, (m, n, k, idx)
+                else:
+                    assert np.all(knet.Array(got) == 7)
+    # one column too many, more than 16 classes, no dW: declined, nothing written
+    m, n, k = 4, cols + 1, 8
+    big = [knet.KnetArray(np.zeros(s, dt)) for s in ((m, k), (m,), (k, n))]
+    lab = knet.KnetArray(np.ones(n, np.int32))
+    out = knet.KnetArray(np.full((m, k), 7, dt))
+    assert lib.call("dense_head_%s" % out.suffix, m, n, k, big[0].ptr, big[1].ptr, big[2].ptr, lab.ptr, c(1.0), out.ptr, None, None, None, None, None) == 1
+    assert lib.call("dense_head_%s" % out.suffix, 17, 4, 4, big[0].ptr, big[1].ptr, big[2].ptr, lab.ptr, c(1.0), out.ptr, None, None, None, None, None) == 1
+    assert lib.call("dense_head_%s" % out.suffix, 4, 4, 4, big[0].ptr, big[1].ptr, big[2].ptr, lab.ptr, c(1.0), None, None, out.ptr, None, None, None) == 1
+    assert np.all(knet.Array(out) == 7)
+    lib.check()
