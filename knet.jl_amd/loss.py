@@ -6,9 +6,9 @@ Mirrors src/ops20/loss.jl:37-41,116-140 and the device side of ``x[indices]`` an
 """
 import numpy as np
 
-from .autograd import primitive, recording, track, value
+from .autograd import primitive, value
 from .karray import KnetArray
-from .libknet8 import knet8, libknet8
+from .libknet8 import knet8
 from . import reduction as R
 from .softmax import logsoftmax
 

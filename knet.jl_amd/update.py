@@ -7,8 +7,6 @@ arrays, ``gclip`` gradient clipping, and one ``update_(w, g, p)`` per parameter.
 """
 import math
 
-import numpy as np
-
 from .binary import zero
 from .karray import KnetArray
 from .libknet8 import knet8
