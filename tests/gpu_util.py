@@ -8,7 +8,8 @@ def ulp_diff(a, b, scale=None):
     dt = a.dtype
     ref = np.abs(np.asarray(b if scale is None else scale, dtype=np.float64))
     sp = np.spacing(np.maximum(ref, np.finfo(dt).tiny).astype(dt)).astype(np.float64)
-    d = np.abs(a.astype(np.float64) - np.asarray(b, np.float64)) / sp
+    with np.errstate(invalid="ignore"):      # inf - inf for matching infinities: set to 0 below
+        d = np.abs(a.astype(np.float64) - np.asarray(b, np.float64)) / sp
     both_nan = np.isnan(a) & np.isnan(np.asarray(b))
     same_inf = np.isinf(a) & (a == np.asarray(b))
     d[both_nan | same_inf] = 0
