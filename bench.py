@@ -538,6 +538,8 @@ def main():
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 1000, True, layers=True, head=True),
             "config1 same graph, output layer forward + loss + gradients in one launch (dense_nll: 3 launches per step)":
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True, head=True),
+            "beside the configs: MLP 784-512-512-10 batch 128, graph with dense layers and dense_nll (own MFMA kernels throughout)":
+                mlp_steps(torch, K, [784, 512, 512, 10], 128, 0.0, 1000, True, graph=True, layers=True, head=True),
             "config1 same step from a compiled C99 host through the C ABI (eager, 3 launches: hidden layer forward, output layer forward + loss + backward, hidden layer backward)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
