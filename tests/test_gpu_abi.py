@@ -294,3 +294,26 @@ def test_transpose_and_batched_permutation(knet, dt, S):
             knet.knet8("transpose_%s" % S, m, n, xd.ptr, y2.ptr)
             assert bits_equal(knet.Array(y2), knet.Array(yd).reshape(n, m)), (m, n)
     knet.libknet8().check()
+
+
+def test_product_routing_knob_both_routes_agree(knet, oracle):
+    """knet8_tune key 3 (products of up to that many MFLOP run on the library's own kernels): the same product through the own MFMA
+    kernel and through hipBLASLt gives the same matrix to rounding; the knob reads back and restores."""
+    fn = knet.libknet8().fn
+    rng = np.random.default_rng(55)
+    m, n, k = 96, 130, 300                                    # 7.5 MFLOP
+    A, B = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((k, n)).astype(np.float32)
+    want = oracle.gemm(A, B)
+    Ad, Bd = knet.KnetArray(A), knet.KnetArray(B)
+    old = fn["knet8_tune"](3, 1)                              # 1 MFLOP: this product now goes to the vendor library
+    try:
+        assert fn["knet8_tune"](3, -1) == 1                   # a negative value only reads
+        vendor = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
+    finally:
+        fn["knet8_tune"](3, old)                              # 0 (never set) restores the default
+    own = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
+    for got in (vendor, own):
+        assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
+    assert np.abs(vendor - own).max() <= 1e-4 * np.abs(want).max()
+    assert fn["knet8_tune"](99, 1) == -1                      # unknown key
+    knet.libknet8().check()
