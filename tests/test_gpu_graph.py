@@ -148,7 +148,7 @@ def test_a_product_first_seen_under_capture_is_planned_without_timing(knet):
 
 
 def test_captured_step_with_fused_layers_matches_the_oracle_on_every_replay(knet, oracle):
-    """The same MLP step written with the one-launch layers (``dense`` forward/backward, ``dense_nll`` for the output layer: four launches)
+    """The same MLP step written with the one-launch layers (``dense`` forward/backward, ``dense_nll`` for the output layer: three launches)
     captured and replayed, with an optimizer step between replays."""
     rng = np.random.default_rng(83)
     lib = knet.libknet8()
