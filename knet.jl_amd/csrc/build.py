@@ -20,6 +20,19 @@ FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hi
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
 
 
+def source_id():
+    """Hash of everything the binary is made from: the hand-written headers and sources, the generator and this script (flags
+    included).  build() bakes it into the library (knet8_build_id()); the loader compares the two and refuses a stale binary."""
+    import hashlib
+    h = hashlib.sha256()
+    names = sorted(f for f in os.listdir(HERE) if f.endswith((".h", ".hip")) or f in ("gen_knet8.py", "build.py"))
+    for name in names:
+        h.update(name.encode())
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def sources():
     sys.path.insert(0, HERE)
     import gen_knet8
@@ -31,7 +44,7 @@ def sources():
 
 def compile_one(src):
     obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + ["-DKNET8_BUILD_ID=\"%s\"" % source_id(), "-c", src, "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:

@@ -655,10 +655,15 @@ KNET8_API void knet8_graph_destroy(void* graph);
 /* last recorded failure as text (NULL if none); reading clears it */
 KNET8_API const char* knet8_last_error(void);
 KNET8_API int knet8_version(void);
+/* hash of the sources the binary was built from (csrc headers and .hip files, the generator, the build script), baked in by build.py:
+   a loader compares it with the working tree and refuses a stale library */
+KNET8_API const char* knet8_build_id(void);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
-   key 3: products of up to this many MFLOP (2*m*n*k/1e6, default 270) take the library's own kernels, larger ones hipBLASLt;
-   key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270) */
+   key 3: products of up to this many MFLOP (2*m*n*k/1e6) take the library's own small-product kernels instead of hipBLASLt (default 0: off,
+   every product of gemm_S / gemm_bias_act_S goes to hipBLASLt);
+   key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270);
+   key 5: non-zero makes the library behave as if the scratch memory of split launches could not be allocated (for tests of that error path) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
    src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */
@@ -676,7 +681,8 @@ KNET8_API int bmm_64_stream(char transa, char transb, int m, int n, int k, doubl
 KNET8_API int bmm_64(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, long long strideA, double* B, int ldb, long long strideB, double beta, double* C, int ldc, long long strideC, int batch);
 /* dense layer in one call: C = act(alpha*op(A)*op(B) + bias[i]) with bias of length m and act 0 (none) or 1 (relu).  No counterpart in
    the reference, which runs gemm!, the bias broadcast (src/knetarrays/binary.jl:61-95) and relu (src/ops20_gpu/activation.jl:17-29) as
-   three launches; same bits as that chain.  Small products fold bias and relu into the product kernel's output stage. */
+   three launches.  Bias and relu run in the output stage of the hipBLASLt product (its BIAS / RELU_BIAS epilogues), so the result is
+   written once; where hipBLASLt has no such kernel the product is followed by one in-place pass. */
 KNET8_API int gemm_bias_act_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc, hipStream_t stream);
 KNET8_API int gemm_bias_act_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc);
 KNET8_API int gemm_bias_act_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias, int act, double* C, int ldc, hipStream_t stream);

@@ -160,7 +160,10 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   P = (unsigned)ceil_div(n, jchunk > 0 ? jchunk : 1);
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
-  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)atiles * P * tile, (size_t)atiles);
+  if (P > 1) {
+    ws = workspace_for(stream, sizeof(T) * (size_t)atiles * P * tile, (size_t)atiles);
+    if (!scratch_ready(ws, "activation gradient + bias gradient: no scratch memory for a split launch")) return;
+  }
   const dim3 grid((unsigned)(atiles * P));
   T* partial = static_cast<T*>(ws.partial);
   const bool big = jchunk >= 64;

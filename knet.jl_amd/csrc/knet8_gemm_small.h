@@ -238,7 +238,10 @@ inline void launch_gemm_small(hipStream_t stream, bool ta, bool tb, int m, int n
   P = (k + kchunk - 1) / kchunk;
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
-  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)tiles * P * kGsTile * kGsTile, (size_t)tiles);
+  if (P > 1) {
+    ws = workspace_for(stream, sizeof(T) * (size_t)tiles * P * kGsTile * kGsTile, (size_t)tiles);
+    if (!scratch_ready(ws, "gemm (small, k split): no scratch memory for a split launch")) return;
+  }
   const dim3 grid((unsigned)(tiles * P)), block(256);
   T* partial = static_cast<T*>(ws.partial);
 #define KNET8_GS(TA, TB) hipLaunchKernelGGL((gemm_small_kernel<T, TA, TB>), grid, block, 0, stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act, kchunk, (unsigned)P, partial, ws.counters)

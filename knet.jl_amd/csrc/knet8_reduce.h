@@ -280,7 +280,7 @@ inline unsigned plan_parts(long groups, long units_per_group, long min_units_per
 }
 
 template <typename T, typename Op>
-inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y) {
+inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y, const ScratchSource* scratch = nullptr) {
   if (ny <= 0) return;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
@@ -291,7 +291,10 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   P = (unsigned)ceil_div(units, chunk > 0 ? chunk : 1);
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
-  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)ny * P, (size_t)ny);
+  if (P > 1) {
+    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)ny * P, (size_t)ny);
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
+  }
   T* partial = static_cast<T*>(ws.partial);
   // workgroup size by the work of one part: a wave for short runs, 512 lanes when there is plenty
   const int bt = chunk <= 2 * kWave ? 64 : chunk <= 4096 ? 256 : 512;
@@ -309,7 +312,7 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
 }
 
 template <typename T, typename Op>
-inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y) {
+inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr) {
   if (s1 <= 0 || nb <= 0) return;
   constexpr int N = Vec16<T>::N;
   if (s1 < kWave) {
@@ -320,7 +323,10 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
     P = (unsigned)ceil_div(total, chunk > 0 ? chunk : 1);
     if (P < 1) P = 1;
     Workspace ws = {nullptr, nullptr};
-    if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)nb * P * s1, (size_t)nb);
+    if (P > 1) {
+      ws = take_scratch(scratch, stream, sizeof(T) * (size_t)nb * P * s1, (size_t)nb);
+      if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
+    }
     hipLaunchKernelGGL((reduce_strided_small_kernel<T, Op>), dim3((unsigned)(nb * P)), dim3(kRedBlock), 0, stream, x, (int)s1, d,
                        chunk, P, y, static_cast<T*>(ws.partial), ws.counters);
     return;
@@ -335,7 +341,10 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   P = (unsigned)ceil_div(d, kchunk > 0 ? kchunk : 1);
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
-  if (P > 1) ws = workspace_for(stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups);
+  if (P > 1) {
+    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups);
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
+  }
   const dim3 grid((unsigned)(groups * P));
   T* partial = static_cast<T*>(ws.partial);
   const bool big = kchunk >= 128;  // sixteen waves share a tile when each still gets >= 8 rows
@@ -348,13 +357,13 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
 
 // `_21` contract: x[i] goes into y[(i/sy)%ny]  (src/libknet8/cuda21.jl:23).
 template <typename T, typename Op>
-inline void reduce_21(hipStream_t stream, long nx, const T* x, long sy, long ny, T* y) {
+inline void reduce_21(hipStream_t stream, long nx, const T* x, long sy, long ny, T* y, const ScratchSource* scratch = nullptr) {
   if (ny <= 0 || sy <= 0 || nx < 0) return;
   if (nx % (sy * ny) != 0) { record_error("reduce _21: nx is not a multiple of sy*ny"); return; }
   const long no = nx / (sy * ny);
-  if (ny == 1) launch_reduce_run<T, Op>(stream, x, nx, 1, 1, y);
-  else if (sy == 1) launch_reduce_strided<T, Op>(stream, x, ny, no, 1, y);
-  else launch_reduce_run<T, Op>(stream, x, sy, ny, no, y);
+  if (ny == 1) launch_reduce_run<T, Op>(stream, x, nx, 1, 1, y, scratch);
+  else if (sy == 1) launch_reduce_strided<T, Op>(stream, x, ny, no, 1, y, scratch);
+  else launch_reduce_run<T, Op>(stream, x, sy, ny, no, y, scratch);
 }
 
 // `_22` contract: output bi reduces x[lower + k*s1], k = 0..xd1, lower = bi%s1 + (bi/s1)*s2

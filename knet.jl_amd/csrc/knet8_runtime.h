@@ -24,6 +24,22 @@ struct Workspace {
   unsigned* counters;
 };
 Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters);
+// Where a split launch takes its scratch from: the per-stream buffers above (a null source) or a caller-supplied provider.  A provider
+// that cannot serve the request records why and returns null pointers.
+struct ScratchSource {
+  Workspace (*get)(void* ctx, hipStream_t stream, size_t partial_bytes, size_t ncounters);
+  void* ctx;
+};
+inline Workspace take_scratch(const ScratchSource* src, hipStream_t stream, size_t partial_bytes, size_t ncounters) {
+  return src ? src->get(src->ctx, stream, partial_bytes, ncounters) : workspace_for(stream, partial_bytes, ncounters);
+}
+// A launch split over several workgroups stores partial results and draws tickets through these pointers: without them it must not be
+// issued at all (out of device memory is an error to report, src/knetarrays/kptr.jl:114-141, not a fault on the device).
+inline bool scratch_ready(const Workspace& ws, const char* who) {
+  if (ws.partial != nullptr && ws.counters != nullptr) return true;
+  record_error(who);   // the allocation's own failure, recorded first, is the message that is kept
+  return false;
+}
 // Device slot for the result of a `_20` reduction on this stream, and the blocking copy that fetches it.
 void* scalar_slot(hipStream_t stream);
 void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes);
@@ -31,7 +47,7 @@ void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes
 // State of the default random stream (knet8_seed): hands out `blocks` consecutive generator counters under the current seed.
 void rng_take(unsigned long long blocks, unsigned long long* seed, unsigned long long* offset);
 
-enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneGemmSmallMflop = 3, kTuneDenseBackMflop = 4, kTuneCount = 8 };
+enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneGemmSmallMflop = 3, kTuneDenseBackMflop = 4, kTuneFailScratch = 5, kTuneCount = 8 };
 int tuning(int key);
 
 }  // namespace knet8

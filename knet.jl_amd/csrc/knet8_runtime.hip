@@ -74,8 +74,9 @@ int tuning(int key) {
       g_tune[key] = 256;
     }
   }
-  if (key == kTuneGemmSmallMflop && g_tune[key] == 0) g_tune[key] = 270;
-  if (key == kTuneDenseBackMflop && g_tune[key] == 0) g_tune[key] = 270;  // layers whose products have up to this many MFLOP each run their backward pass in one launch  // products up to this many MFLOP (2mnk) take the library's own kernels
+  // kTuneGemmSmallMflop stays 0 unless a caller opts in: gemm_S and gemm_bias_act_S go to hipBLASLt (the matrix cores are used through the
+  // vendor library only).  A positive value sends products of up to that many MFLOP (2mnk) to the library's own small-product kernels.
+  if (key == kTuneDenseBackMflop && g_tune[key] == 0) g_tune[key] = 270;  // dense_back_S and its relatives accept layers whose products have up to this many MFLOP each
   return g_tune[key];
 }
 
@@ -85,7 +86,6 @@ struct StreamScratch {
   size_t partial_bytes = 0;
   unsigned* counters = nullptr;
   size_t ncounters = 0;
-  void* scalar = nullptr;
   std::vector<void*> retired;
   hipEvent_t t0 = nullptr, t1 = nullptr;
 };
@@ -104,6 +104,11 @@ __global__ __launch_bounds__(256) void zero_counters_kernel(unsigned* c, size_t 
 }
 
 Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounters) {
+  if (g_tune[kTuneFailScratch] != 0) {   // set by tests: behave as if the device were out of memory, without touching it
+    record_error("reduction scratch: allocation refused (knet8_tune key 5 is set)");
+    Workspace none = {nullptr, nullptr};
+    return none;
+  }
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   StreamScratch& s = scratch_of(stream);
   // Buffers that have become too small are retired, not freed: launches already queued on the stream, and graphs
@@ -133,11 +138,16 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
   return w;
 }
 
+// One slot per (host thread, device, stream): two threads that call a `_20` entry point on the same stream (the plain twins all use the
+// null stream; the reference builds with --default-stream per-thread, src/libknet8/build.jl:5) must not read each other's result.
+// 256 bytes each, kept until the process ends.
 void* scalar_slot(hipStream_t stream) {
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  StreamScratch& s = scratch_of(stream);
-  if (!s.scalar) ok(hipMalloc(&s.scalar, 256), "hipMalloc(scalar slot)");
-  return s.scalar;
+  thread_local std::map<std::pair<int, hipStream_t>, void*> slots;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  void*& p = slots[std::make_pair(dev, stream)];
+  if (!p && !ok(hipMalloc(&p, 256), "hipMalloc(scalar slot)")) p = nullptr;
+  return p;
 }
 
 void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes) {
@@ -325,7 +335,6 @@ KNET8_API void knet8_stream_destroy(hipStream_t stream) {
       StreamScratch& s = it->second;
       if (s.partial) (void)hipFree(s.partial);
       if (s.counters) (void)hipFree(s.counters);
-      if (s.scalar) (void)hipFree(s.scalar);
       for (void* p : s.retired) (void)hipFree(p);
       if (s.t0) (void)hipEventDestroy(s.t0);
       if (s.t1) (void)hipEventDestroy(s.t1);
@@ -419,7 +428,14 @@ KNET8_API const char* knet8_last_error(void) {
   return g_err_out.c_str();
 }
 
-KNET8_API int knet8_version(void) { return 100; }
+KNET8_API int knet8_version(void) { return 200; }
+
+// Hash of the sources this binary was built from (csrc/*.h, *.hip, gen_knet8.py, build.py), written by build.py: lets a loader refuse a
+// stale library.
+#ifndef KNET8_BUILD_ID
+#define KNET8_BUILD_ID "unknown"
+#endif
+KNET8_API const char* knet8_build_id(void) { return KNET8_BUILD_ID; }
 
 KNET8_API void knet8_seed(unsigned long long seed) {
   std::lock_guard<std::mutex> lock(g_rng_mu);
@@ -445,11 +461,11 @@ struct GemmBatch {   // strided batch: product b uses A + b*sa, B + b*sb, C + b*
   long long sa = 0, sb = 0, sc = 0;
 };
 struct GemmKey {
-  int dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch;
+  int dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch, epilogue;
   long long sa, sb, sc;
   bool operator<(const GemmKey& o) const {
-    return std::tie(dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch, sa, sb, sc) <
-           std::tie(o.dev, o.dtype, o.ta, o.tb, o.m, o.n, o.k, o.lda, o.ldb, o.ldc, o.batch, o.sa, o.sb, o.sc);
+    return std::tie(dev, dtype, ta, tb, m, n, k, lda, ldb, ldc, batch, epilogue, sa, sb, sc) <
+           std::tie(o.dev, o.dtype, o.ta, o.tb, o.m, o.n, o.k, o.lda, o.ldb, o.ldc, o.batch, o.epilogue, o.sa, o.sb, o.sc);
   }
 };
 struct GemmPlan {
@@ -457,8 +473,9 @@ struct GemmPlan {
   hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
-  bool valid = false;   // descriptors and an algorithm exist
-  bool timed = false;   // the algorithm was chosen by timing the candidates (not possible while the stream is being captured)
+  bool valid = false;        // descriptors and an algorithm exist
+  bool timed = false;        // the algorithm was chosen by timing the candidates (not possible while the stream is being captured)
+  bool unsupported = false;  // the vendor library has no kernel for this problem with this epilogue: callers take the separate bias pass
 };
 static std::mutex g_gemm_mutex;
 static std::map<int, hipblasLtHandle_t> g_lt;
@@ -474,37 +491,26 @@ static bool lt_ok(hipblasStatus_t s, const char* what) {
   return false;
 }
 
-// bias != nullptr / act != 0: the dense-layer form C = act(alpha*op(A)*op(B) + bias[i]) (beta must be 0).  Small products fold it
-// into the output stage of the product kernel; large ones run the vendor product and then one in-place bias+activation pass.
+static void destroy_plan(GemmPlan& p) {
+  if (p.la) (void)hipblasLtMatrixLayoutDestroy(p.la);
+  if (p.lb) (void)hipblasLtMatrixLayoutDestroy(p.lb);
+  if (p.lc) (void)hipblasLtMatrixLayoutDestroy(p.lc);
+  if (p.desc) (void)hipblasLtMatmulDescDestroy(p.desc);
+  p = GemmPlan();
+}
+
+// bias != nullptr / act != 0: the dense-layer form C = act(alpha*op(A)*op(B) + bias[i]) (beta must be 0).
 struct EpiNone { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb; } };
 struct EpiRelu { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb != zb ? zb : (zb > T(0) ? zb : T(0)); } };
 
+enum { kEpiNone = 0, kEpiBias = 1, kEpiReluBias = 2 };
+constexpr int kGemmNoFusedForm = 2;   // gemm_lt: the vendor library has no kernel for this problem (with this epilogue); nothing was launched
+
+// One product through hipBLASLt.  epilogue != kEpiNone: bias (length m, added to every column) and optionally relu are applied by the
+// product kernel's own output stage, so the m x n result is written once and never read back.
 template <typename T>
-static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
-                hipStream_t stream, const T* bias = nullptr, int act = 0, GemmBatch batch = GemmBatch()) {
-  if (m <= 0 || n <= 0 || batch.count <= 0) return 0;
-  const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
-  const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
-  if (batch.count > 1 && (bias || act)) { record_error("gemm: the bias/activation form takes no batch"); return -1; }
-  if (batch.count == 1 && gemm_is_small(m, n, k)) {
-    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act);
-    check_launch("gemm (small)");
-    return 0;
-  }
-  if (bias || act) {
-    if (ldc != m) { record_error("gemm_bias_act: ldc must equal m for large products"); return -1; }
-    const int rc = gemm<T>(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, stream);
-    if (rc != 0) return rc;
-    if (bias) {
-      if (act == 1) launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiRelu());
-      else launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiNone());
-    } else {
-      record_error("gemm_bias_act: an activation without a bias is not provided");
-      return -1;
-    }
-    check_launch("gemm_bias_act (bias pass)");
-    return 0;
-  }
+static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc, hipStream_t stream,
+                   int epilogue, const T* bias, GemmBatch batch) {
   const hipDataType dt = sizeof(T) == 4 ? HIP_R_32F : HIP_R_64F;
   const hipblasComputeType_t ct = sizeof(T) == 4 ? HIPBLAS_COMPUTE_32F : HIPBLAS_COMPUTE_64F;
   int dev = 0;
@@ -514,35 +520,51 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   if (!h && !lt_ok(hipblasLtCreate(&h), "create")) return -1;
   void*& ws = g_gemm_ws[std::make_pair(dev, stream)];
   if (!ws && !ok(hipMalloc(&ws, kGemmWorkspace), "hipMalloc(gemm workspace)")) return -1;
-  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, batch.sa, batch.sb, batch.sc};
+  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, epilogue, batch.sa, batch.sb, batch.sc};
   GemmPlan& p = g_plans[key];
+  if (p.unsupported) return kGemmNoFusedForm;
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (stream) (void)hipStreamIsCapturing(stream, &cap);
   const bool capturing = cap != hipStreamCaptureStatusNone;
+  // A plan whose creation fails half way is taken out of the cache again: the next call must not find a descriptor without layouts.
+  auto fail = [&]() { destroy_plan(p); g_plans.erase(key); return -1; };
   if (!p.desc) {
     const hipblasOperation_t opa = ta ? HIPBLAS_OP_T : HIPBLAS_OP_N, opb = tb ? HIPBLAS_OP_T : HIPBLAS_OP_N;
-    if (!lt_ok(hipblasLtMatmulDescCreate(&p.desc, ct, dt), "desc create")) return -1;
-    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &opa, sizeof(opa)), "set transa")) return -1;
-    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &opb, sizeof(opb)), "set transb")) return -1;
-    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.la, dt, ta ? k : m, ta ? m : k, lda), "layout A")) return -1;
-    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lb, dt, tb ? n : k, tb ? k : n, ldb), "layout B")) return -1;
-    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lc, dt, m, n, ldc), "layout C")) return -1;
+    if (!lt_ok(hipblasLtMatmulDescCreate(&p.desc, ct, dt), "desc create")) return fail();
+    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &opa, sizeof(opa)), "set transa")) return fail();
+    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &opb, sizeof(opb)), "set transb")) return fail();
+    if (epilogue != kEpiNone) {
+      const hipblasLtEpilogue_t ep = epilogue == kEpiReluBias ? HIPBLASLT_EPILOGUE_RELU_BIAS : HIPBLASLT_EPILOGUE_BIAS;
+      if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof(ep)) != HIPBLAS_STATUS_SUCCESS ||
+          hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &dt, sizeof(dt)) != HIPBLAS_STATUS_SUCCESS) {
+        destroy_plan(p);
+        p.unsupported = true;
+        return kGemmNoFusedForm;
+      }
+    }
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.la, dt, ta ? k : m, ta ? m : k, lda), "layout A")) return fail();
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lb, dt, tb ? n : k, tb ? k : n, ldb), "layout B")) return fail();
+    if (!lt_ok(hipblasLtMatrixLayoutCreate(&p.lc, dt, m, n, ldc), "layout C")) return fail();
     if (batch.count > 1) {
       const int32_t bc = batch.count;
       const int64_t st[3] = {batch.sa, batch.sb, batch.sc};
       hipblasLtMatrixLayout_t lay[3] = {p.la, p.lb, p.lc};
       for (int q = 0; q < 3; q++) {
-        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &bc, sizeof(bc)), "batch count")) return -1;
-        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &st[q], sizeof(st[q])), "batch stride")) return -1;
+        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_BATCH_COUNT, &bc, sizeof(bc)), "batch count")) return fail();
+        if (!lt_ok(hipblasLtMatrixLayoutSetAttribute(lay[q], HIPBLASLT_MATRIX_LAYOUT_STRIDED_BATCH_OFFSET, &st[q], sizeof(st[q])), "batch stride")) return fail();
       }
     }
+  }
+  if (epilogue != kEpiNone) {   // the bias vector changes from call to call; the descriptor is only used under this lock
+    const void* bp = bias;
+    if (!lt_ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp)), "set bias pointer")) return fail();
   }
   // Choose the algorithm: at the first call, and again at the first call that is allowed to time the candidates if the earlier
   // choice had to be made without (a stream under capture cannot be synchronised; a call with beta != 0 would accumulate into C).
   const bool can_time = !capturing && beta == T(0);
   if (!p.valid || (!p.timed && can_time)) {
     hipblasLtMatmulPreference_t pref = nullptr;
-    if (!lt_ok(hipblasLtMatmulPreferenceCreate(&pref), "pref create")) return -1;
+    if (!lt_ok(hipblasLtMatmulPreferenceCreate(&pref), "pref create")) return fail();
     size_t wsbytes = kGemmWorkspace;
     lt_ok(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsbytes, sizeof(wsbytes)), "pref workspace");
     // Ask for several candidates and time each once on this problem: the first heuristic answer is far from the
@@ -550,11 +572,12 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
     constexpr int kCand = 8;
     hipblasLtMatmulHeuristicResult_t res[kCand];
     int found = 0;
-    const bool got = lt_ok(hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, kCand, res, &found), "heuristic");
+    const hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, kCand, res, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
-    if (!got || found < 1) {
-      record_error("hipBLASLt: no algorithm for this GEMM shape");
-      return -1;
+    if (hs != HIPBLAS_STATUS_SUCCESS || found < 1) {
+      destroy_plan(p);   // not an error: the caller falls back on the library's own product kernels, and remembers it
+      p.unsupported = true;
+      return kGemmNoFusedForm;
     }
     int best = 0;
     if (found > 1 && can_time) {
@@ -588,6 +611,45 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
     p.timed = can_time;
   }
   return lt_ok(hipblasLtMatmul(h, p.desc, &alpha, A, p.la, B, p.lb, &beta, C, p.lc, C, p.lc, &p.algo, ws, kGemmWorkspace, stream), "matmul") ? 0 : -1;
+}
+
+template <typename T>
+static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T* A, int lda, const T* B, int ldb, T beta, T* C, int ldc,
+                hipStream_t stream, const T* bias = nullptr, int act = 0, GemmBatch batch = GemmBatch()) {
+  if (m <= 0 || n <= 0 || batch.count <= 0) return 0;
+  const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
+  const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
+  if (batch.count > 1 && (bias || act)) { record_error("gemm: the bias/activation form takes no batch"); return -1; }
+  if ((long long)m * n >= (1LL << 31) || (long long)m * k >= (1LL << 31) || (long long)k * n >= (1LL << 31)) {
+    record_error("gemm: an operand has 2^31 or more elements; the 32-bit indices of the library's kernels do not reach that far");
+    return -1;
+  }
+  if (batch.count == 1 && (k <= 0 || gemm_is_small(m, n, k))) {   // empty products (C = beta*C [+ bias]), and small ones when a caller has opted in (knet8_tune key 3)
+    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act);
+    check_launch("gemm (small)");
+    return 0;
+  }
+  // Products the vendor library has no kernel for (seen with some fp64 shapes) run on the library's own tiles, whatever their size.
+  auto plain = [&](T bt) {
+    int rc = gemm_lt<T>(ta, tb, m, n, k, alpha, A, lda, B, ldb, bt, C, ldc, stream, kEpiNone, nullptr, batch);
+    if (rc != kGemmNoFusedForm) return rc;
+    if (batch.count > 1) { record_error("hipBLASLt: no algorithm for this batched product"); return -1; }
+    launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, bt, C, ldc, nullptr, 0);
+    check_launch("gemm (own kernel: no vendor algorithm)");
+    return 0;
+  };
+  if (!bias && !act) return plain(beta);
+  if (!bias) { record_error("gemm_bias_act: an activation without a bias is not provided"); return -1; }
+  int rc = gemm_lt<T>(ta, tb, m, n, k, alpha, A, lda, B, ldb, T(0), C, ldc, stream, act == 1 ? kEpiReluBias : kEpiBias, bias, batch);
+  if (rc != kGemmNoFusedForm) return rc;
+  // no fused form in the vendor library for this type or shape: the product, then one in-place pass over it
+  if (ldc != m) { record_error("gemm_bias_act: ldc must equal m when the vendor library has no fused form for the product"); return -1; }
+  rc = plain(T(0));
+  if (rc != 0) return rc;
+  if (act == 1) launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiRelu());
+  else launch_bias_act<T, false>(stream, m, n, C, bias, C, EpiNone());
+  check_launch("gemm_bias_act (bias pass)");
+  return 0;
 }
 
 

@@ -44,6 +44,18 @@ def parse_header(path=HEADER_PATH):
     return out
 
 
+def source_build_id():
+    """The id build.py would bake into a library built from the sources next to this package (None when they are not there)."""
+    import importlib.util
+    path = os.path.join(_PKG, "csrc", "build.py")
+    if not os.path.exists(path):
+        return None
+    spec = importlib.util.spec_from_file_location("knet8_build_for_id", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.source_id()
+
+
 class LibKnet8:
     def __init__(self, path=LIB_PATH):
         if not os.path.exists(path):
@@ -59,6 +71,11 @@ class LibKnet8:
             f.argtypes = [_CTYPES[a] for a in args]
             self.fn[name] = f
         self.stream = None  # current stream handle (None = null stream), cf. CUDA.stream() in the reference
+        self.build_id = self.fn["knet8_build_id"]().decode()
+        want = source_build_id()
+        if want is not None and want != self.build_id and not os.environ.get("KNET8_ALLOW_STALE"):
+            raise OSError("libknet8.so at %s was built from other sources (library %s, working tree %s): rebuild it "
+                          "(python __graft_entry__.py build)" % (path, self.build_id, want))
 
     def check(self):
         msg = self.fn["knet8_last_error"]()

@@ -297,23 +297,71 @@ def test_transpose_and_batched_permutation(knet, dt, S):
 
 
 def test_product_routing_knob_both_routes_agree(knet, oracle):
-    """knet8_tune key 3 (products of up to that many MFLOP run on the library's own kernels): the same product through the own MFMA
-    kernel and through hipBLASLt gives the same matrix to rounding; the knob reads back and restores."""
+    """gemm_S goes to hipBLASLt unless a caller opts in: knet8_tune key 3 (products of up to that many MFLOP run on the library's own
+    small-product kernels) is 0 by default.  The same product through both routes gives the same matrix to rounding; the knob reads
+    back and restores."""
     fn = knet.libknet8().fn
     rng = np.random.default_rng(55)
     m, n, k = 96, 130, 300                                    # 7.5 MFLOP
     A, B = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((k, n)).astype(np.float32)
     want = oracle.gemm(A, B)
     Ad, Bd = knet.KnetArray(A), knet.KnetArray(B)
-    old = fn["knet8_tune"](3, 1)                              # 1 MFLOP: this product now goes to the vendor library
+    assert fn["knet8_tune"](3, -1) == 0                       # default: every product goes to the vendor library
+    vendor = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
+    old = fn["knet8_tune"](3, 270)                            # opt in: this product now runs on the library's own kernel
     try:
-        assert fn["knet8_tune"](3, -1) == 1                   # a negative value only reads
-        vendor = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
+        assert old == 0 and fn["knet8_tune"](3, -1) == 270    # a negative value only reads
+        own = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
     finally:
-        fn["knet8_tune"](3, old)                              # 0 (never set) restores the default
-    own = knet.Array(knet.gemm("N", "N", 1, Ad, Bd, 0, knet.KnetArray(np.zeros((m, n), np.float32))))
+        fn["knet8_tune"](3, 0)
     for got in (vendor, own):
         assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
     assert np.abs(vendor - own).max() <= 1e-4 * np.abs(want).max()
     assert fn["knet8_tune"](99, 1) == -1                      # unknown key
     knet.libknet8().check()
+
+
+def test_split_launch_without_scratch_is_refused_on_the_host(knet):
+    """When the scratch memory of a split launch cannot be had (out of device memory; forced here through knet8_tune key 5) the
+    launch must not happen at all: the failure is recorded, as "Out of gpu memory" is an error and not a crash in the reference
+    (src/knetarrays/kptr.jl:114-141), and the output keeps what it held.  Nothing touches the device on this path."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    rng = np.random.default_rng(56)
+    sentinel = np.float32(-777.0)
+    x = rng.integers(-3, 4, size=(256, 4096)).astype(np.float32)          # one row tile, 4096 columns: the planner splits the columns
+    xd = knet.KnetArray(x)
+    dy, yv = rng.standard_normal((256, 4096)).astype(np.float32), rng.standard_normal((256, 4096)).astype(np.float32)
+    dyd, yd = knet.KnetArray(dy), knet.KnetArray(yv)
+
+    def sum_dims2(out):
+        fn["sum_32_21_stream"](x.size, xd.ptr, 1, 256, out.ptr, lib.stream)
+
+    def sum_all(out):     # run view, one output: split over the whole array
+        fn["sum_32_21_stream"](x.size, xd.ptr, x.size, 1, out.ptr, lib.stream)
+
+    def sum_small_rows(out):   # short contiguous axis
+        fn["sum_32_21_stream"](x.size, xd.ptr, 1, 8, out.ptr, lib.stream)
+
+    def bias_grad(out):
+        dz = knet.KnetArray(dtype=np.float32, dims=(256, 4096))
+        fn["reluback_biasgrad_32_stream"](256, 4096, dyd.ptr, yd.ptr, dz.ptr, out.ptr, lib.stream)
+
+    cases = [(sum_dims2, 256), (sum_all, 1), (sum_small_rows, 8), (bias_grad, 256)]
+    assert fn["knet8_tune"](5, 1) == 0
+    try:
+        for launch, ny in cases:
+            out = knet.KnetArray(np.full(ny, sentinel, np.float32))
+            launch(out)
+            assert fn["knet8_synchronize"](lib.stream) == 0
+            msg = fn["knet8_last_error"]()
+            assert msg is not None and b"scratch" in msg, (launch.__name__, msg)
+            assert np.all(knet.Array(out) == sentinel), launch.__name__      # no kernel ran on it
+    finally:
+        fn["knet8_tune"](5, 0)
+    for launch, ny in cases[:3]:                                             # with the knob back the same calls work
+        out = knet.KnetArray(np.full(ny, sentinel, np.float32))
+        launch(out)
+        want = x.sum(axis=1) if ny == 256 else (x.sum() if ny == 1 else x.reshape(-1, order="F").reshape(8, -1, order="F").sum(axis=1))
+        assert np.array_equal(knet.Array(out).ravel(), np.atleast_1d(want).astype(np.float32)), launch.__name__
+    lib.check()

@@ -158,14 +158,9 @@ def test_fused_layers_in_the_mlp_match_oracle(knet, oracle):
     knet.libknet8().check()
 
 
-@pytest.mark.parametrize("dt", [np.float32, np.float64])
-def test_gemm_bias_act_carries_the_bits_of_the_three_launch_chain(knet, dt):
-    """C = act(alpha*op(A)*op(B) + bias) in one call against gemm, add_12 and relu through the same library: identical bits, over
-    the product kernels' plans (cross-workgroup split, in-workgroup k slices, plain tiles) and a vendor-library size."""
-    rng = np.random.default_rng(55)
+def _gemm_bias_act_cases(knet, dt, rng, shapes):
     S = sfx(dt)
     lib = knet.libknet8()
-    shapes = [(64, 100, 784), (10, 100, 64), (33, 17, 5), (130, 131, 129), (512, 300, 256), (256, 300, 96), (1000, 700, 300)]
     for (m, n, k) in shapes:
         for ta, tb in (("N", "N"), ("T", "N"), ("N", "T")):
             a = rng.standard_normal((m, k) if ta == "N" else (k, m)).astype(dt)
@@ -174,15 +169,54 @@ def test_gemm_bias_act_carries_the_bits_of_the_three_launch_chain(knet, dt):
             A, B, bd = knet.KnetArray(a), knet.KnetArray(b), knet.KnetArray(bias)
             z = knet.gemm(ta, tb, 1, A, B, 0, knet.KnetArray(np.zeros((m, n), dt)))
             zb = knet.add(z, bd)
-            for act, want in ((0, knet.Array(zb)), (1, knet.Array(knet.relu(zb)))):
+            ref = (a if ta == "N" else a.T).astype(np.float64) @ (b if tb == "N" else b.T).astype(np.float64) + bias.astype(np.float64)
+            for act, chain, ref_act in ((0, knet.Array(zb), ref), (1, knet.Array(knet.relu(zb)), np.maximum(ref, 0))):
                 C = knet.KnetArray(np.full((m, n), np.nan, dt))
                 rc = lib.call("gemm_bias_act_%s" % S, ta.encode(), tb.encode(), m, n, k, A.ctype(1), A.ptr, a.shape[0], B.ptr, b.shape[0],
                               bd.ptr, act, C.ptr, m)
                 assert rc == 0
-                assert bits_equal(knet.Array(C), want), (m, n, k, ta, tb, act)
-    lib.call("gemm_bias_act_%s" % S, b"N", b"N", 4, 4, 4, A.ctype(1), A.ptr, 4, B.ptr, 4, bd.ptr, 7, C.ptr, 4)
+                yield (m, n, k, ta, tb, act), knet.Array(C), chain, ref_act
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gemm_bias_act_in_the_vendor_epilogue_matches_the_three_launch_chain(knet, dt):
+    """C = act(alpha*op(A)*op(B) + bias) in one call (bias and relu in the output stage of the hipBLASLt product) against gemm, add_12
+    and relu as three launches and against an fp64 product.  Not bit for bit: hipBLASLt runs a different kernel for the product with
+    an epilogue than for the plain product, and the two sum over k in different orders, so the comparison is at the tolerance of the
+    product itself (1e-5 of the matrix norm in fp32, 1e-13 in fp64); what is exact is the relu: never a negative output, and 0 wherever the
+    fp64 value is below zero by more than that tolerance."""
+    rng = np.random.default_rng(55)
+    lib = knet.libknet8()
+    rtol = 1e-5 if dt == np.float32 else 1e-13
+    shapes = [(64, 100, 784), (10, 100, 64), (33, 17, 5), (130, 131, 129), (512, 300, 256), (1000, 700, 300), (4096, 256, 512)]
+    for case, got, chain, ref in _gemm_bias_act_cases(knet, dt, rng, shapes):
+        tol = rtol * np.linalg.norm(ref) if np.linalg.norm(ref) > 0 else rtol
+        assert np.linalg.norm(got - ref) <= tol, case
+        assert np.linalg.norm(got - chain) <= 2 * tol, case
+        if case[-1] == 1:
+            assert got.min() >= 0, case
+            eps = rtol * np.abs(ref).max() * 10
+            assert np.all(got[ref < -eps] == 0) and np.all(got[ref > eps] > 0), case
+    A = knet.KnetArray(np.zeros((4, 4), dt))
+    lib.call("gemm_bias_act_%s" % sfx(dt), b"N", b"N", 4, 4, 4, A.ctype(1), A.ptr, 4, A.ptr, 4, A.ptr, 7, A.ptr, 4)
     with pytest.raises(RuntimeError):
         lib.check()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gemm_bias_act_on_the_own_kernels_carries_the_bits_of_the_three_launch_chain(knet, dt):
+    """With the library's own small-product kernels switched on (knet8_tune key 3) both the one-call form and the chain run on them, and
+    bias and relu in the kernel's output stage give identical bits, over its plans (cross-workgroup split, k slices, plain tiles)."""
+    rng = np.random.default_rng(55)
+    fn = knet.libknet8().fn
+    old = fn["knet8_tune"](3, 270)
+    try:
+        shapes = [(64, 100, 784), (10, 100, 64), (33, 17, 5), (130, 131, 129), (512, 300, 256), (256, 300, 96)]
+        for case, got, chain, _ in _gemm_bias_act_cases(knet, dt, rng, shapes):
+            assert bits_equal(got, chain), case
+    finally:
+        fn["knet8_tune"](3, old)
+    knet.libknet8().check()
 
 
 def test_dense_primitive_in_the_mlp_matches_oracle(knet, oracle):
