@@ -658,6 +658,14 @@ KNET8_API int knet8_version(void);
 /* hash of the sources the binary was built from (csrc headers and .hip files, the generator, the build script), baked in by build.py:
    a loader compares it with the working tree and refuses a stale library */
 KNET8_API const char* knet8_build_id(void);
+/* No counterpart in the reference.  sum_32_21 for callers that cannot allocate device memory -- code under hipGraph capture, tight
+   serving loops, harnesses that forbid hipMalloc: the same kernels and the same result, bit for bit, with the partial results and
+   tickets of a split launch in a fixed array inside the library (1 MiB of partials + 4096 tickets per GPU, held until the process
+   ends) instead of the per-stream buffers that sum_32_21 grows through hipMalloc.  Calls no hipMalloc, hipFree or other allocating
+   routine.  A shape whose split needs more than the array holds is refused: the error is recorded and y is left untouched.  All calls
+   on one GPU share the array, so calls that overlap in time on one GPU (other streams, other threads) race; calls on one stream are
+   ordered and safe. */
+KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hipStream_t stream);
 /* launch-heuristic knobs; returns the old value; value 0 restores the default, a negative value only reads.  Key 0: number of compute units the reduction planner aims at (default: asked from the
    device); key 1: longest softmax column kept resident in registers, longer ones take the two-pass streaming kernel (default 0: the register capacity);
    key 3: products of up to this many MFLOP (2*m*n*k/1e6) take the library's own small-product kernels instead of hipBLASLt (default 0: off,

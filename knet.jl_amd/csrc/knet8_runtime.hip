@@ -138,6 +138,56 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
   return w;
 }
 
+// ---- scratch for callers that cannot allocate ---------------------------------------------------------------------
+// sum_32_21_noalloc runs the same kernels as sum_32_21 with the partial results and tickets of a split launch in this fixed array
+// instead of the per-stream buffers above (which grow through hipMalloc).  Every GPU the library runs on holds its own copy, at its
+// own address, until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel
+// can use is asked from the runtime once per device and kept.
+constexpr size_t kStaticPartialBytes = size_t(1) << 20;
+constexpr size_t kStaticCounters = 4096;
+static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(unsigned)];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_static_mutex;
+static unsigned char* g_static_ptr[kMaxDevices] = {nullptr};
+
+static unsigned char* static_scratch_ptr() {
+  int dev = -1;
+  if (!ok(hipGetDevice(&dev), "hipGetDevice") || dev < 0 || dev >= kMaxDevices) {
+    record_error("sum_32_21_noalloc: no current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_ptr[dev] == nullptr) {
+    unsigned char* ptr = nullptr;
+    if (!ok(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)") || ptr == nullptr) return nullptr;
+    g_static_ptr[dev] = ptr;
+  }
+  return g_static_ptr[dev];
+}
+
+static Workspace static_scratch_get(void*, hipStream_t stream, size_t partial_bytes, size_t ncounters) {
+  Workspace none = {nullptr, nullptr};
+  if (partial_bytes > kStaticPartialBytes || ncounters > kStaticCounters) {
+    char buf[256];
+    snprintf(buf, sizeof(buf), "sum_32_21_noalloc: the split of this shape needs %zu bytes of partial results and %zu tickets; the library's fixed scratch "
+             "holds %zu bytes and %zu tickets (use sum_32_21)", partial_bytes, ncounters, kStaticPartialBytes, kStaticCounters);
+    record_error(buf);
+    return none;
+  }
+  unsigned char* base = static_scratch_ptr();
+  if (base == nullptr) return none;
+  unsigned* counters = reinterpret_cast<unsigned*>(base + kStaticPartialBytes);
+  // The array keeps whatever the last call on this GPU left in it: the tickets this launch draws start from zero by a fill kernel on
+  // the same stream (a kernel, not a memset node, so the call can be captured into a graph).
+  if (ncounters > 0) {
+    hipLaunchKernelGGL(zero_counters_kernel, dim3((unsigned)((ncounters + 255) / 256)), dim3(256), 0, stream, counters, ncounters);
+    if (!ok(hipGetLastError(), "zero_counters_kernel")) return none;
+  }
+  Workspace w = {base, counters};
+  return w;
+}
+
 // One slot per (host thread, device, stream): two threads that call a `_20` entry point on the same stream (the plain twins all use the
 // null stream; the reference builds with --default-stream per-thread, src/libknet8/build.jl:5) must not read each other's result.
 // 256 bytes each, kept until the process ends.
@@ -436,6 +486,12 @@ KNET8_API int knet8_version(void) { return 200; }
 #define KNET8_BUILD_ID "unknown"
 #endif
 KNET8_API const char* knet8_build_id(void) { return KNET8_BUILD_ID; }
+
+KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hipStream_t stream) {
+  const ScratchSource src = {static_scratch_get, nullptr};
+  reduce_21<float, RedSum<float>>(stream, nx, x, sy, ny, y, &src);
+  check_launch("sum_32_21_noalloc");
+}
 
 KNET8_API void knet8_seed(unsigned long long seed) {
   std::lock_guard<std::mutex> lock(g_rng_mu);
