@@ -379,8 +379,11 @@ def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=F
 
 
 def c_host_steps(K, steps=5000):
-    """The config-1 step driven by a compiled C99 host through the C ABI (tests/c_host/mlp_step.c), eager, no graph: what a host
-    with ccall-like call overhead (the reference's Julia) reaches.  None if no C compiler is at hand."""
+    """The config-1 step driven by compiled C99 hosts through the C ABI, eager, no graph: what a host with ccall-like call overhead (the
+    reference's Julia) reaches.  mlp_ref_sequence.c issues the launch sequence an unchanged Knet model emits (reference-named entry
+    points only: 18 launches, one upload and one blocking download per step), with every product on hipBLASLt (the default) and with the
+    library's own small-product kernels switched on; mlp_step.c is the same step through the fused layer entry points (3 launches).  None
+    if no C compiler is at hand."""
     import shutil
     import subprocess
     import tempfile
@@ -389,23 +392,37 @@ def c_host_steps(K, steps=5000):
     here = os.path.dirname(os.path.abspath(__file__))
     libdir = os.path.dirname(K.LIB_PATH)
     rng = np.random.default_rng(0)
+    out = {}
     with tempfile.TemporaryDirectory() as tmp:
-        exe, fin, fout = os.path.join(tmp, "mlp_step"), os.path.join(tmp, "in.bin"), os.path.join(tmp, "out.bin")
-        subprocess.check_call(["gcc", "-std=c99", "-D_POSIX_C_SOURCE=199309L", "-O2", "-I", os.path.join(here, "include"),
-                               os.path.join(here, "tests", "c_host", "mlp_step.c"), "-o", exe, "-L", libdir, "-lknet8",
-                               "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
+        fin, fout = os.path.join(tmp, "in.bin"), os.path.join(tmp, "out.bin")
         with open(fin, "wb") as f:
             for shape, scale in (((64, 784), 0.01), ((64, 1), 0.0), ((10, 64), 0.01), ((10, 1), 0.0)):
                 f.write((rng.standard_normal(shape) * scale).astype(np.float32).tobytes(order="F"))
             f.write(rng.random((784, 100), dtype=np.float32).tobytes(order="F"))
             f.write(rng.integers(1, 11, size=100).astype(np.int32).tobytes())
-        r = subprocess.run([exe, fin, fout, str(steps)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
-        if r.returncode != 0:
-            raise RuntimeError("mlp_step failed: " + r.stderr)
-        rates = dict(line.split() for line in r.stdout.strip().splitlines())
+
+        def run(name, extra):
+            exe = os.path.join(tmp, name)
+            if not os.path.exists(exe):
+                subprocess.check_call(["gcc", "-std=c99", "-D_POSIX_C_SOURCE=199309L", "-O2", "-I", os.path.join(here, "include"),
+                                       os.path.join(here, "tests", "c_host", name + ".c"), "-o", exe, "-L", libdir, "-lknet8",
+                                       "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
+            r = subprocess.run([exe, fin, fout] + extra, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=180)
+            if r.returncode != 0:
+                raise RuntimeError(name + " failed: " + r.stderr)
+            rates = dict(line.split() for line in r.stdout.strip().splitlines())
+            return rates, float(np.fromfile(fout, dtype=np.float32, count=1)[0])
+        for label, own in (("config1 reference launch sequence (C host): 18 launches of reference-named entry points, products on hipBLASLt (default routing)", 0),
+                           ("config1 reference launch sequence (C host), products on the library's own kernels (knet8_tune key 3 = 270)", 270)):
+            rates, loss = run("mlp_ref_sequence", [str(max(steps // 2, 1)), str(own)])
+            rate = float(rates["steps_per_sec"])
+            out[label] = {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "loss": loss}
+        rates, loss = run("mlp_step", [str(steps)])
         rate = float(rates["steps_per_sec"])
-        loss = float(np.fromfile(fout, dtype=np.float32, count=1)[0])
-    return {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "graph_replay_steps_per_sec": float(rates["graph_steps_per_sec"]), "loss": loss}
+        out["config1 same step through the fused layer entry points (C host, eager, 3 launches: hidden layer forward, output layer forward + loss + backward, "
+            "hidden layer backward; opt-in API, own MFMA kernels in the two backward launches)"] = {
+            "steps_per_sec": rate, "ms_per_step": 1e3 / rate, "graph_replay_steps_per_sec": float(rates["graph_steps_per_sec"]), "loss": loss}
+    return out
 
 
 def cpu_side_table():
@@ -540,13 +557,15 @@ def main():
                 mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True, head=True),
             "beside the configs: MLP 784-512-512-10 batch 128, graph with dense layers and dense_nll (own MFMA kernels throughout)":
                 mlp_steps(torch, K, [784, 512, 512, 10], 128, 0.0, 1000, True, graph=True, layers=True, head=True),
-            "config1 same step from a compiled C99 host through the C ABI (eager, 3 launches: hidden layer forward, output layer forward + loss + backward, hidden layer backward)": c_host_steps(K),
             "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),
             "config5 same graph with fused bias+relu+dropout layers":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True, layers=True),
         }
+        ch = c_host_steps(K)
+        if ch:
+            line["mlp"].update(ch)
     line["cpu_baseline"] = cpu_baseline()
     if not args.no_extras:
         line["cpu_oracle_config3_4_5 (1 thread, algorithmic GB/s)"] = cpu_side_table()

@@ -485,8 +485,18 @@ def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None, gemm=None):
         else:
             saved.append((h, None, None))
             h = z
-    loss = nll(h, labels)
-    dz = nll_back(h, labels)
+    return nll(h, labels), mlp_backward_given_forward(weights, saved, h, labels, pdrop=pdrop, gemm=gemm)
+
+
+def mlp_backward_given_forward(weights, saved, scores, labels, pdrop=0.0, gemm=None):
+    """The backward half of ``mlp_backward`` on a forward pass that is handed in: ``saved[l] = (input of layer l, relu output or None,
+    dropout output or None)`` and the output layer's ``scores``.  With the activations of a device run as ``saved`` the masks of relu
+    and dropout are the device's own, so a comparison of the gradients measures the gradient kernels and not which side of zero a
+    pre-activation fell on under two GEMM accumulation orders.  Same expressions as above (src/knetarrays/linalg.jl:11-18,
+    ``sum(dy;dims=2)``, ``reluback``, ``dropback``, ``ko_nll_back``)."""
+    gemm = gemm or globals()["gemm"]
+    nl = len(weights) // 2
+    dz = nll_back(scores, labels)
     grads = [None] * (2 * nl)
     for l in reversed(range(nl)):
         hin, y, yd = saved[l]
@@ -498,4 +508,4 @@ def mlp_backward(weights, x, labels, pdrop=0.0, uniforms=None, gemm=None):
         grads[2 * l] = gemm(dz, hin, tb=True)
         if l > 0:
             dz = gemm(weights[2 * l], dz, ta=True)
-    return loss, grads
+    return grads

@@ -94,17 +94,40 @@ def test_config5_deep_mlp_full_size(knet, oracle):
     params = build(knet, ws)
     xd = knet.KnetArray(x)
     unid = [knet.KnetArray(u) for u in uni]
-    J = knet.diff(lambda: knet.nll(predict(knet, params, xd, 0.5, unid), labels, fused=True))
+    kept = []   # the device's own activations: (relu output, dropout output) per hidden layer, then the scores
+
+    def forward():
+        h = xd
+        for i in range(0, len(params), 2):
+            h = knet.add(knet.matmul(params[i], h), params[i + 1])
+            if i < len(params) - 2:
+                y = knet.relu(h)
+                h = knet.dropout(y, 0.5, uniform=unid[i // 2])
+                kept.append((knet.value(y), knet.value(h)))
+        kept.append(knet.value(h))
+        return h
+    J = knet.diff(lambda: knet.nll(forward(), labels, fused=True))
     assert abs(float(knet.value(J)) - float(loss_ref)) <= 1e-5 * abs(float(loss_ref))
     errs = [rel(knet.Array(knet.grad(J, p)), g) for p, g in zip(params, grads_ref)]
-    print("config5 relative gradient errors (dW1, db1, ..., dW8, db8):", ["%.1e" % e for e in errs])
-    # Two fp32 GEMM implementations differ in accumulation order (k = 4096), so of the 8.4 M pre-activations of a
-    # hidden layer the handful that lie within rounding of zero land on different sides of relu's step.  Each such
-    # flip is a 100 % error on one element of the upstream gradient: sqrt(flips / 8.4e6) ~ 1e-3 norm-wise, which is
-    # what layers 1-7 show.  The output layer has no relu between it and the loss and must agree to 1e-4
-    # (measured: 2e-6), which is the check that the GEMM, bias-gradient and fused nll kernels themselves are right.
+    print("config5 relative gradient errors against the oracle's own forward pass (dW1, db1, ..., dW8, db8):", ["%.1e" % e for e in errs])
+    # Against the oracle's OWN forward pass only the output layer can be held tightly: two fp32 GEMM implementations differ in
+    # accumulation order (k = 4096), so of the 8.4 M pre-activations of a hidden layer the handful within rounding of zero land on
+    # different sides of relu's step, each a 100 % error on one element of the upstream gradient (sqrt(flips / 8.4e6) ~ 1e-3 norm-wise).
     assert max(errs[-2:]) <= 1e-4, errs
     assert max(errs) <= 5e-3, errs
+    # The sharp check: the oracle's backward pass on the DEVICE's activations (its relu outputs, dropout outputs and scores, downloaded).
+    # The masks are then the same on both sides, the flips cancel, and every one of the 16 gradients -- the whole dropback / reluback /
+    # bias-gradient / product chain at (4096,2048) -- must agree to 1e-4 norm-wise.
+    saved, hin = [], x
+    for y, yd in kept[:-1]:
+        ya, yda = knet.Array(y), knet.Array(yd)
+        saved.append((hin, ya, yda))
+        hin = yda
+    saved.append((hin, None, None))
+    grads_dev = oracle.mlp_backward_given_forward(ws, saved, knet.Array(kept[-1]), labels, pdrop=0.5, gemm=blas_gemm)
+    errs2 = [rel(knet.Array(knet.grad(J, p)), g) for p, g in zip(params, grads_dev)]
+    print("config5 relative gradient errors against the oracle's backward pass on the device's activations:", ["%.1e" % e for e in errs2])
+    assert max(errs2) <= 1e-4, errs2
     knet.libknet8().check()
 
 
