@@ -30,10 +30,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of reluback_32_11 on 2^28 elements from the two `rocprofv3 --pmc` runs summarised in
-# profiles/libknet8_kernels_profile_pass.txt: FETCH_SIZE x 2.0000 -> 2048.0 MiB + WRITE_SIZE x 0.9996 -> 1023.6 MiB, each scaled by
-# what the same counter reads for the 1 GiB + 1 GiB copy kernel of that run.  (Algorithmic: 3 * 4 * 2^28 = 3221225472.)
-RELUBACK_32_TRAFFIC_BYTES = int((2048.0 + 1023.6) * (1 << 20))
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "libknet8_kernels_profile_pass.txt")
+
+
+def profiled_traffic(kernel):
+    """HBM bytes per launch of `kernel` as the committed rocprofv3 summary holds them (a line `traffic <kernel> <bytes> ...`, written from
+    two `rocprofv3 --pmc` runs of `bench.py --profile-pass`: FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for the
+    1 GiB + 1 GiB copy kernel of that run).  Not measured in the run that prints the bench line; None if the summary is not there."""
+    try:
+        for line in open(PROFILE_SUMMARY):
+            f = line.split()
+            if len(f) >= 3 and f[0] == "traffic" and f[1] == kernel:
+                return int(f[2])
+    except OSError:
+        pass
+    return None
+
+
 OPS = [("reluback", "relu"), ("sigmback", "sigm"), ("tanhback", "tanh"), ("eluback", "elu"), ("seluback", "selu")]
 
 
@@ -121,9 +134,12 @@ def config2(torch, K, steps, warmup):
     return (t1 - t0), total_bytes, per_kernel
 
 
-def time_kernel(K, torch, make_launch, nbytes, footprints, reps=20):
-    """Warm: `reps` back-to-back launches on one buffer set.  Cold: rotate over enough distinct buffer sets to
-    exceed 1 GB, so that no launch finds its inputs in the Infinity Cache."""
+def time_kernel(K, torch, make_launch, nbytes, footprints, reps=24):
+    """Warm: `reps` back-to-back launches on one buffer set.  Cold: rotate over enough distinct buffer sets to exceed 1 GB, so that
+    no launch finds its inputs in the Infinity Cache.  Two figures per mode, both from HIP events on the launch stream:
+      us_batch_mean    one event pair around `reps` back-to-back launches, divided by their number -- the average launch duration;
+                       `us`, GBps and frac_of_peak are computed from this one;
+      us_event_median  median over event pairs around single launches (includes the gap the event records themselves add)."""
     out = {}
     for mode, sets in (("warm", footprints[:1]), ("cold", footprints)):
         launches = [make_launch(s) for s in sets]
@@ -134,14 +150,13 @@ def time_kernel(K, torch, make_launch, nbytes, footprints, reps=20):
         n = max(reps, len(launches) * 2)
         ids = [ev.time(launches[i % len(launches)]) for i in range(n)]
         torch.cuda.synchronize()
-        ms = float(np.median([ev.ms(i) for i in ids]))
-        # event pairs around single ~20 us launches include a few us of dispatch gap: also time them as one batch
-        b = ev.time(lambda: [launches[i % len(launches)]() for i in range(n)])
+        med = float(np.median([ev.ms(i) for i in ids]))
+        batches = [ev.time(lambda: [launches[i % len(launches)]() for i in range(n)]) for _ in range(3)]
         torch.cuda.synchronize()
-        msb = ev.ms(b) / n
+        mean = float(np.median([ev.ms(b) for b in batches])) / n
         ev.close()
-        best = min(ms, msb)
-        out[mode] = {"us": best * 1e3, "GBps": nbytes / best * 1e-6, "frac_of_peak": nbytes / best * 1e-6 / HBM_PEAK_GBS}
+        out[mode] = {"us": mean * 1e3, "us_batch_mean": mean * 1e3, "us_event_median": med * 1e3, "launches": n,
+                     "GBps": nbytes / mean * 1e-6, "frac_of_peak": nbytes / mean * 1e-6 / HBM_PEAK_GBS}
     return out
 
 
@@ -185,125 +200,179 @@ def neighbours(torch, K):
     return res
 
 
-def extras(torch, K):
-    res = {}
+def kernel_cases(torch, K, widths=("32", "64")):
+    """The kernels of benchmark configs 3, 4 and 5 at their full shapes: yields (label, algorithmic bytes per launch, number of buffer sets,
+    make_launch) where make_launch(i) returns a function that launches the kernel on buffer set i.  Enough sets that one round over them
+    exceeds 1 GB.  fp32 is the configs' own width; the fp64 rows are the same kernels at the reference's other element type."""
+    for S in widths:
+        dt, sz = (torch.float32, 4) if S == "32" else (torch.float64, 8)
+        # config 3: unbroadcast reductions
+        nsets = 10 if S == "32" else 5
+        mats = [device_randn(torch, K, 4096 * 8192, dt, 10 + i, dims=(4096, 8192)) for i in range(nsets)]
+        for d, ny in ((1, 8192), (2, 4096)):
+            outs = [m.similar((ny,)) for m in mats]
+            sy = 4096 if d == 1 else 1
+            yield ("sum_%s_21 (4096,8192) dims=%d" % (S, d), sz * (4096 * 8192 + ny), nsets,
+                   lambda i, sy=sy, ny=ny, outs=outs: (lambda: K.knet8("sum_%s_21" % S, 4096 * 8192, mats[i].ptr, sy, ny, outs[i].ptr)))
+        del mats, outs
+        nn = 56 * 56 * 256 * 64
+        nsets = 6 if S == "32" else 4
+        mats = [device_randn(torch, K, nn, dt, 30 + i) for i in range(nsets)]
+        outs = [m.similar((256,)) for m in mats]
+        yield ("sum_%s_21 NCHW (56,56,256,64)->(1,1,256,1)" % S, sz * (nn + 256), nsets,
+               lambda i: (lambda: K.knet8("sum_%s_21" % S, nn, mats[i].ptr, 3136, 256, outs[i].ptr)))
+        del mats, outs
+        # config 4: logsoftmax backward and fused nll backward
+        for C, N in ((32000, 512), (1000, 4096)):
+            nsets = (8 if C == 32000 else 24) // (1 if S == "32" else 2)
+            ys = [device_randn(torch, K, C * N, dt, 50 + i, scale=2.0) for i in range(nsets)]
+            dys = [device_randn(torch, K, C * N, dt, 90 + i) for i in range(nsets)]
+            dxs = [y.similar() for y in ys]
+            labels = K.KnetArray(np.random.default_rng(0).integers(1, C + 1, size=N).astype(np.int32))
+            loss = ys[0].similar((N,))
+            scale = (ctypes.c_float if S == "32" else ctypes.c_double)(1.0 / N)
+            yield ("logsoftmaxback_%s (%d,%d)" % (S, C, N), 3 * sz * C * N, nsets,
+                   lambda i: (lambda: K.knet8("logsoftmaxback_%s" % S, C, N, ys[i].ptr, dys[i].ptr, dxs[i].ptr)))
+            yield ("nll_logsoftmax_back_%s (%d,%d)" % (S, C, N), 2 * sz * C * N + sz * N, nsets,
+                   lambda i: (lambda: K.knet8("nll_logsoftmax_back_%s" % S, C, N, ys[i].ptr, labels.ptr, scale, dxs[i].ptr, loss.ptr)))
+            if S == "32":
+                # yardsticks: plain elementwise kernels moving the same bytes over the same buffers -- what this chip delivers to
+                # any kernel of this size, launch ramp and drain included
+                yield ("yardstick reluback_32_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (C * N, C, N), 12 * C * N, nsets,
+                       lambda i: (lambda: K.knet8("reluback_32_11", C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)))
+                yield ("yardstick relu_32 n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (C * N, C, N), 8 * C * N, nsets,
+                       lambda i: (lambda: K.knet8("relu_32", C * N, ys[i].ptr, dxs[i].ptr)))
+            del ys, dys, dxs
+    # config 5 per-layer kernels (fp32): dropback, then the fused layer passes: bias + relu + dropout forward (z, u -> y) and
+    # dropback + reluback + bias gradient (dy, y -> dz, db)
     f32 = torch.float32
-    # config 3: unbroadcast reductions
-    nsets = 10
-    mats = [device_randn(torch, K, 4096 * 8192, f32, 10 + i, dims=(4096, 8192)) for i in range(nsets)]
-    for d, ny in ((1, 8192), (2, 4096)):
-        outs = [m.similar((ny,)) for m in mats]
-        sy = 4096 if d == 1 else 1
-
-        def mk(i, sy=sy, ny=ny, outs=outs):
-            return lambda: K.knet8("sum_32_21", 4096 * 8192, mats[i].ptr, sy, ny, outs[i].ptr)
-        res["sum_32_21 (4096,8192) dims=%d" % d] = time_kernel(K, torch, mk, 4 * (4096 * 8192 + ny), list(range(nsets)))
-    del mats
-    nn = 56 * 56 * 256 * 64
-    mats = [device_randn(torch, K, nn, f32, 30 + i) for i in range(6)]
-    outs = [m.similar((256,)) for m in mats]
-    res["sum_32_21 NCHW (56,56,256,64)->(1,1,256,1)"] = time_kernel(
-        K, torch, lambda i: (lambda: K.knet8("sum_32_21", nn, mats[i].ptr, 3136, 256, outs[i].ptr)), 4 * (nn + 256), list(range(6)))
-    del mats
-    # config 4: logsoftmax backward and fused nll backward
-    for C, N in ((32000, 512), (1000, 4096)):
-        nsets = 8 if C == 32000 else 24
-        ys = [device_randn(torch, K, C * N, f32, 50 + i, scale=2.0) for i in range(nsets)]
-        dys = [device_randn(torch, K, C * N, f32, 90 + i) for i in range(nsets)]
-        dxs = [y.similar() for y in ys]
-        res["logsoftmaxback_32 (%d,%d)" % (C, N)] = time_kernel(
-            K, torch, lambda i: (lambda: K.knet8("logsoftmaxback_32", C, N, ys[i].ptr, dys[i].ptr, dxs[i].ptr)), 12 * C * N, list(range(nsets)))
-        rng = np.random.default_rng(0)
-        labels = K.KnetArray(rng.integers(1, C + 1, size=N).astype(np.int32))
-        loss = ys[0].similar((N,))
-        res["nll_logsoftmax_back_32 (%d,%d)" % (C, N)] = time_kernel(
-            K, torch, lambda i: (lambda: K.knet8("nll_logsoftmax_back_32", C, N, ys[i].ptr, labels.ptr, ctypes.c_float(1.0 / N), dxs[i].ptr, loss.ptr)),
-            8 * C * N + 4 * N, list(range(nsets)))
-        # yardsticks: plain elementwise kernels moving the same bytes over the same buffers -- what this chip delivers to
-        # any kernel of this size, launch ramp and drain included
-        res["yardstick reluback_32_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (C * N, C, N)] = time_kernel(
-            K, torch, lambda i: (lambda: K.knet8("reluback_32_11", C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)), 12 * C * N, list(range(nsets)))
-        res["yardstick relu_32 n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (C * N, C, N)] = time_kernel(
-            K, torch, lambda i: (lambda: K.knet8("relu_32", C * N, ys[i].ptr, dxs[i].ptr)), 8 * C * N, list(range(nsets)))
-        del ys, dys, dxs
-    # config 5 per-layer dropback
     n5 = 4096 * 2048
     ys = [device_randn(torch, K, n5, f32, 130 + i) for i in range(40)]
     dys = [device_randn(torch, K, n5, f32, 180 + i) for i in range(40)]
     dxs = [y.similar() for y in ys[:4]]
-    res["dropback_32 (4096,2048)"] = time_kernel(
-        K, torch, lambda i: (lambda: K.knet8("dropback_32", n5, ctypes.c_float(0.5), ys[i].ptr, ys[i].ptr, dys[i].ptr, dxs[i % 4].ptr)), 12 * n5, list(range(40)))
-    # config 5 fused layer passes: bias + relu + dropout forward (z, u -> y) and dropback + reluback + bias gradient (dy, y -> dz, db)
-    zs = dys
+    half = ctypes.c_float(0.5)
+    yield ("dropback_32 (4096,2048)", 12 * n5, 40,
+           lambda i: (lambda: K.knet8("dropback_32", n5, half, ys[i].ptr, ys[i].ptr, dys[i].ptr, dxs[i % 4].ptr)))
     us = [device_randn(torch, K, n5, f32, 230 + i) for i in range(4)]
     bias = device_randn(torch, K, 4096, f32, 229)
     db = bias.similar()
-    res["biasreludrop_32 (4096,2048)"] = time_kernel(
-        K, torch, lambda i: (lambda: K.knet8("biasreludrop_32", 4096, 2048, ctypes.c_float(0.5), zs[i].ptr, bias.ptr, us[i % 4].ptr)),
-        12 * n5 + 4 * 4096, list(range(40)))
-    res["dropreluback_biasgrad_32 (4096,2048)"] = time_kernel(
-        K, torch, lambda i: (lambda: K.knet8("dropreluback_biasgrad_32", 4096, 2048, ctypes.c_float(0.5), dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr, db.ptr)),
-        12 * n5 + 4 * 4096, list(range(40)))
-    K.libknet8().check()
+    yield ("biasreludrop_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
+           lambda i: (lambda: K.knet8("biasreludrop_32", 4096, 2048, half, dys[i].ptr, bias.ptr, us[i % 4].ptr)))
+    yield ("dropreluback_biasgrad_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
+           lambda i: (lambda: K.knet8("dropreluback_biasgrad_32", 4096, 2048, half, dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr, db.ptr)))
+
+
+def extras(torch, K):
+    res = {}
+    for label, nbytes, nsets, make_launch in kernel_cases(torch, K):
+        res[label] = time_kernel(K, torch, make_launch, nbytes, list(range(nsets)))
+        K.libknet8().check()
     return res
 
 
-def profile_pass(torch, K):
-    """One launch of every kernel the roofline tables quote, preceded by a copy kernel of known size (1 GiB read +
-    1 GiB written) against which the HBM byte counters of a `rocprofv3 --pmc` run are scaled."""
+PROFILE_REPS = 24
+
+
+def profile_pass(torch, K, mode, plan_path):
+    """For `rocprofv3` runs: PROFILE_REPS launches of every kernel the roofline tables quote, config 2 first (after a copy kernel of known
+    size, 1 GiB read + 1 GiB written, against which the HBM byte counters of a `--pmc` run are scaled), then configs 3-5 either warm
+    (the same buffers every time) or cold (rotating over more than 1 GB of buffers, as the bench table's cold column does).  The plan
+    -- label, algorithmic bytes and launch count of each group, in launch order -- goes to `plan_path` for --summarize-profile."""
+    plan = []
     f32 = torch.float32
     n = 1 << 28
     x = device_randn(torch, K, n, f32, 1)
     dy = device_randn(torch, K, n, f32, 2)
     dx = x.similar()
-    for _ in range(3):
+    for _ in range(PROFILE_REPS):
         K.knet8("copy_32", n, x.ptr, dx.ptr)
+    plan.append(["copy_32 n=2^28 (1 GiB read + 1 GiB written: the yardstick of the byte counters)", 8 * n, PROFILE_REPS])
     for back, fwd in OPS:
         y = K.unary_op(fwd, x)
-        for _ in range(3):
+        for _ in range(PROFILE_REPS):
             K.knet8("%s_32_11" % back, n, dy.ptr, y.ptr, dx.ptr)
+        plan.append(["%s_32_11 n=2^28" % back, 12 * n, PROFILE_REPS])
         del y
+    del x, dy, dx
     xd = device_randn(torch, K, 1 << 27, torch.float64, 3)
     dyd = device_randn(torch, K, 1 << 27, torch.float64, 4)
-    yd = K.unary_op("sigm", xd)
-    for _ in range(3):
-        K.knet8("sigmback_64_11", 1 << 27, dyd.ptr, yd.ptr, xd.ptr)
-    del xd, dyd, yd, x, dy, dx
+    dxd = xd.similar()
+    for back, fwd in OPS:
+        yd = K.unary_op(fwd, xd)
+        for _ in range(PROFILE_REPS):
+            K.knet8("%s_64_11" % back, 1 << 27, dyd.ptr, yd.ptr, dxd.ptr)
+        plan.append(["%s_64_11 n=2^27" % back, 24 << 27, PROFILE_REPS])
+        del yd
+    del xd, dyd, dxd
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     K.libknet8().fn["knet8_trim"]()
-    m = device_randn(torch, K, 4096 * 8192, f32, 5)
-    o = m.similar((8192,))
-    for _ in range(3):
-        K.knet8("sum_32_21", 4096 * 8192, m.ptr, 4096, 8192, o.ptr)
-        K.knet8("sum_32_21", 4096 * 8192, m.ptr, 1, 4096, o.ptr)
-    nn = 56 * 56 * 256 * 64
-    m = device_randn(torch, K, nn, f32, 6)
-    for _ in range(3):
-        K.knet8("sum_32_21", nn, m.ptr, 3136, 256, o.ptr)
-    for C, N in ((32000, 512), (1000, 4096)):
-        y = device_randn(torch, K, C * N, f32, 7, scale=2.0)
-        dyy = device_randn(torch, K, C * N, f32, 8)
-        dxx = y.similar()
-        labels = K.KnetArray(np.random.default_rng(0).integers(1, C + 1, size=N).astype(np.int32))
-        loss = y.similar((N,))
-        for _ in range(3):
-            K.knet8("logsoftmaxback_32", C, N, y.ptr, dyy.ptr, dxx.ptr)
-            K.knet8("nll_logsoftmax_back_32", C, N, y.ptr, labels.ptr, ctypes.c_float(1.0 / N), dxx.ptr, loss.ptr)
-    n5 = 4096 * 2048
-    y = device_randn(torch, K, n5, f32, 9)
-    dyy = device_randn(torch, K, n5, f32, 10)
-    dxx = y.similar()
-    for _ in range(3):
-        K.knet8("dropback_32", n5, ctypes.c_float(0.5), y.ptr, y.ptr, dyy.ptr, dxx.ptr)
-    bias = device_randn(torch, K, 4096, f32, 11)
-    db = bias.similar()
-    for _ in range(3):
-        u = device_randn(torch, K, n5, f32, 12)
-        K.knet8("biasreludrop_32", 4096, 2048, ctypes.c_float(0.5), dyy.ptr, bias.ptr, u.ptr)
-        K.knet8("dropreluback_biasgrad_32", 4096, 2048, ctypes.c_float(0.5), dyy.ptr, u.ptr, dxx.ptr, db.ptr)
-    torch.cuda.synchronize()
+    for label, nbytes, nsets, make_launch in kernel_cases(torch, K):
+        launches = [make_launch(i) for i in (range(nsets) if mode == "cold" else range(1))]
+        for r in range(PROFILE_REPS):
+            launches[r % len(launches)]()
+        plan.append(["%s [%s]" % (label, mode), nbytes, PROFILE_REPS])
+        torch.cuda.synchronize()
     K.libknet8().check()
+    with open(plan_path, "w") as f:
+        json.dump(plan, f)
+
+
+def summarize_profile(root):
+    """Text summary of the rocprofv3 output of the profile passes under `root`: <mode>_trace/ (--kernel-trace --stats), <mode>_fetch/ and
+    <mode>_write/ (--pmc FETCH_SIZE / WRITE_SIZE), <mode>_plan.json, for mode in warm, cold.  Dispatches are grouped by kernel name and
+    grid; the groups with PROFILE_REPS dispatches are, in order of first appearance, the groups of the plan."""
+    import collections
+    import csv
+    import glob
+
+    def groups(path, value):
+        g = collections.OrderedDict()
+        for r in csv.DictReader(open(path)):
+            if "knet8" not in r["Kernel_Name"]:
+                continue
+            grid = r.get("Grid_Size_X") or r.get("Grid_Size")
+            wg = r.get("Workgroup_Size_X") or r.get("Workgroup_Size")
+            g.setdefault((r["Kernel_Name"], grid, wg), []).append(value(r))
+        return g
+
+    def short(name):
+        return name.replace("void knet8::", "").replace("knet8::", "").split("(")[0][:100]
+    print("HBM peak used for the fractions: %.0f GB/s.  Durations are rocprofv3 kernel-trace begin-to-end times per dispatch; GB/s = algorithmic bytes / average duration." % HBM_PEAK_GBS)
+    for mode in ("warm", "cold"):
+        tr = glob.glob(os.path.join(root, mode + "_trace", "*kernel_trace.csv"))
+        if not tr:
+            continue
+        plan = json.load(open(os.path.join(root, mode + "_plan.json")))
+        dur = groups(tr[0], lambda r: (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) * 1e-3)
+        cnt = {}
+        for which, cname in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
+            pc = glob.glob(os.path.join(root, "%s_%s" % (mode, which), "*counter_collection.csv"))
+            cnt[which] = groups(pc[0], lambda r: float(r["Counter_Value"])) if pc else {}
+        matched = [(k, v) for k, v in dur.items() if len(v) == PROFILE_REPS]
+        print()
+        print("== %s pass: %d launches per kernel (`python3 bench.py --profile-pass %s`) ==" % (mode, PROFILE_REPS, mode))
+        if len(matched) != len(plan):
+            print("!! %d groups of %d dispatches in the trace, %d in the plan: labels below may be off" % (len(matched), PROFILE_REPS, len(plan)))
+        scale = {}
+        for which in ("fetch", "write"):
+            ck = [k for k in cnt[which] if "Op_copy<float>" in k[0] or "copy" in short(k[0]).lower()]
+            if ck:
+                kib = float(np.mean(cnt[which][ck[0]]))
+                scale[which] = (1 << 20) / kib
+                print("byte-counter scale from copy_32 (1 GiB each way): %s_SIZE reads %.1f KiB per dispatch -> x %.4f" % (which.upper(), kib, scale[which]))
+        print("%-74s %-58s %7s %7s %7s %7s %8s %6s %10s %10s" % ("workload", "kernel", "avg_us", "med_us", "min_us", "max_us", "GB/s", "frac", "fetch_MiB", "write_MiB"))
+        for (key, v), (label, nbytes, _) in zip(matched, plan):
+            avg = float(np.mean(v))
+            fm = wm = float("nan")
+            if key in cnt.get("fetch", {}) and "fetch" in scale:
+                fm = float(np.mean(cnt["fetch"][key])) * scale["fetch"] / 1024
+            if key in cnt.get("write", {}) and "write" in scale:
+                wm = float(np.mean(cnt["write"][key])) * scale["write"] / 1024
+            print("%-74s %-58s %7.1f %7.1f %7.1f %7.1f %8.0f %6.3f %10.1f %10.1f" % (label[:74], short(key[0])[:58], avg, float(np.median(v)), min(v), max(v),
+                                                                                nbytes / avg * 1e-3, nbytes / avg * 1e-3 / HBM_PEAK_GBS, fm, wm))
+            if mode == "warm" and label.startswith("reluback_32_11") and fm == fm and wm == wm:
+                print("traffic reluback_32_11 %d   (bytes per launch: fetch + write above)" % int((fm + wm) * (1 << 20)))
 
 
 def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=False, head=False):
@@ -503,9 +572,15 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-extras", action="store_true", help="only the config-2 step, roofline and CPU baseline")
-    ap.add_argument("--profile-pass", action="store_true",
-                    help="launch each quoted kernel three times after a known-size copy kernel and exit (for rocprofv3 runs)")
+    ap.add_argument("--profile-pass", choices=["warm", "cold"], default=None,
+                    help="launch each quoted kernel %d times (config 2 after a known-size copy kernel; configs 3-5 on one buffer set or "
+                         "rotating over more than 1 GB) and exit: the workload of the rocprofv3 runs" % PROFILE_REPS)
+    ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default gpurun_out/prof/<mode>_plan.json)")
+    ap.add_argument("--summarize-profile", metavar="DIR", default=None, help="print the text summary of the rocprofv3 output under DIR and exit (no GPU needed)")
     args = ap.parse_args()
+    if args.summarize_profile:
+        summarize_profile(args.summarize_profile)
+        return
     if args.gpus != 1:
         print("bench.py measures one MI355X: the gradient kernels have no multi-GPU path (every GPU box here has one GPU); "
               "run with --gpus 1", file=sys.stderr)
@@ -516,8 +591,10 @@ def main():
     torch.cuda.set_device(0)
     torch.cuda.synchronize()
     if args.profile_pass:
-        profile_pass(torch, K)
-        print(json.dumps({"profile_pass": "done"}))
+        plan_path = args.plan_out or os.path.join(ROOT, "gpurun_out", "prof", args.profile_pass + "_plan.json")
+        os.makedirs(os.path.dirname(plan_path), exist_ok=True)
+        profile_pass(torch, K, args.profile_pass, plan_path)
+        print(json.dumps({"profile_pass": args.profile_pass, "plan": plan_path}))
         return
     elapsed, total_bytes, per_kernel = config2(torch, K, args.steps, args.warmup)
     value = total_bytes / elapsed * 1e-9
@@ -530,7 +607,9 @@ def main():
         "config": {"workload": "benchmark config 2: {relu,sigm,tanh,elu,selu}back on 2^28 fp32 and 2^27 fp64 vectors, "
                                "x,dy~N(0,1) seeded, y=f(x); 10 launches per step", "frac_of_hbm_peak": value / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "reluback_32_11 (ew_vec_kernel<float,2>)", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": RELUBACK_32_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": dom["bytes"],
+                     "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": profiled_traffic("reluback_32_11"),
+                     "traffic_source": "from_profile: profiles/libknet8_kernels_profile_pass.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --profile-pass`), not measured in this run",
+                     "algorithmic_bytes_per_launch": dom["bytes"],
                      "avg_launch_us": dom["us"]},
         "kernels_config2": {k: {"us": round(v["us"], 2), "GBps": round(v["GBps"], 1), "frac": round(v["GBps"] / HBM_PEAK_GBS, 4)} for k, v in per_kernel.items()},
     }
