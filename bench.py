@@ -641,6 +641,10 @@ def main():
             "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),
             "config5 same graph with fused bias+relu+dropout layers":
                 mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True, layers=True),
+            "config5 shapes without dropout, graph, product / bias add / relu as three launches per layer":
+                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.0, 20, True, graph=True),
+            "config5 shapes without dropout, graph, dense layers: bias and relu in the epilogue of the hipBLASLt product (z never written or re-read)":
+                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.0, 20, True, graph=True, layers=True),
         }
         ch = c_host_steps(K)
         if ch:

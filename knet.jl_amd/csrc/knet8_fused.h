@@ -43,6 +43,7 @@ __global__ __launch_bounds__(kEwBlock) void bias_act_kernel(long nitems, const T
 template <typename T, bool DROP, typename F>
 inline void launch_bias_act(hipStream_t stream, long m, long n, const T* z, const T* b, T* y, F f) {
   if (m <= 0 || n <= 0) return;
+  if (m * n >= (1L << 31)) { record_error("bias + activation: 2^31 or more elements; the kernel's 32-bit row arithmetic does not reach that far"); return; }
   constexpr int N = Vec16<T>::N;
   const bool vec = (m % N == 0) && aligned16(z) && aligned16(b) && aligned16(y);
   const long nitems = vec ? m * n / N : m * n;
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
 template <typename T, typename F>
 inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T* dy, const T* y, T* dz, T* db, F f) {
   if (m <= 0) return;
+  if (n > 0 && m * n >= (1L << 31)) { record_error("activation gradient + bias gradient: 2^31 or more elements are not supported"); return; }
   constexpr int N = Vec16<T>::N;
   const bool vec = (m % N == 0) && aligned16(dy) && aligned16(y) && aligned16(dz);
   const long tile = (long)kWave * N;

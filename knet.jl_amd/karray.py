@@ -204,6 +204,31 @@ class Graph:
             pass
 
 
+_CAPTURE_STREAM = None
+
+
+def capture_stream():
+    """The stream ``capture`` records on: created at first use, owned by the package, destroyed at interpreter exit."""
+    global _CAPTURE_STREAM
+    if _CAPTURE_STREAM is None:
+        import atexit
+        lib = libknet8()
+        _CAPTURE_STREAM = lib.fn["knet8_stream_create"]()
+
+        def _destroy():
+            global _CAPTURE_STREAM
+            if _CAPTURE_STREAM is not None:
+                try:
+                    if lib.stream == _CAPTURE_STREAM:
+                        lib.stream = None
+                    lib.fn["knet8_stream_destroy"](_CAPTURE_STREAM)
+                except Exception:
+                    pass
+                _CAPTURE_STREAM = None
+        atexit.register(_destroy)
+    return _CAPTURE_STREAM
+
+
 def capture(fn):
     """Run ``fn()`` once eagerly (so that pool blocks, reduction scratch and GEMM plans exist), then once more under
     stream capture, and return a ``Graph``.  ``fn`` must not synchronise with the host (no ``Array(x)``, no ``dims=:``
@@ -211,7 +236,12 @@ def capture(fn):
     global _PARKED
     lib = libknet8()
     if lib.stream is None:
-        lib.stream = lib.fn["knet8_stream_create"]()
+        # Capture needs a stream of its own.  Work already queued on the null stream (fills, copies and random draws that built the
+        # parameters) must have landed first: a non-blocking stream does not wait for the null stream.  The stream is created once,
+        # kept as the package's capture stream and destroyed when the interpreter exits; the caller restores `lib.stream` if it wants
+        # the null stream back.
+        lib.fn["knet8_synchronize"](None)
+        lib.stream = capture_stream()
     # Warm-up under the same parking rule as the capture itself, so that the pool ends up holding one block for every
     # allocation of the sequence (blocks freed while parked are not recycled within the run).
     warm = _PARKED = []
