@@ -137,8 +137,9 @@ def config2(torch, K, steps, warmup):
 def time_kernel(K, torch, make_launch, nbytes, footprints, reps=24):
     """Warm: `reps` back-to-back launches on one buffer set.  Cold: rotate over enough distinct buffer sets to exceed 1 GB, so that
     no launch finds its inputs in the Infinity Cache.  Two figures per mode, both from HIP events on the launch stream:
-      us_batch_mean    one event pair around `reps` back-to-back launches, divided by their number -- the average launch duration;
-                       `us`, GBps and frac_of_peak are computed from this one;
+      us_batch_mean    one event pair around `reps` back-to-back launches, divided by their number -- the average launch duration (median of
+                       three such batches); `us`, GBps and frac_of_peak are computed from this one.  (Replaying the same launches as one
+                       hipGraph, which takes the interpreter out of the timed region, measured the same to 0.2 us on every row.)
       us_event_median  median over event pairs around single launches (includes the gap the event records themselves add)."""
     out = {}
     for mode, sets in (("warm", footprints[:1]), ("cold", footprints)):
@@ -590,6 +591,10 @@ def main():
     K = ge.load_package()
     torch.cuda.set_device(0)
     torch.cuda.synchronize()
+    # Every launch goes to a stream of the library's own, as every @knet8 call of the reference goes to CUDA.stream()
+    # (src/libknet8/LibKnet8.jl:50-55), not to the legacy null stream (which has to order itself against every other stream of the process).
+    if not os.environ.get("KNET8_BENCH_NULL_STREAM"):
+        K.libknet8().stream = K.libknet8().fn["knet8_stream_create"]()
     if args.profile_pass:
         plan_path = args.plan_out or os.path.join(ROOT, "gpurun_out", "prof", args.profile_pass + "_plan.json")
         os.makedirs(os.path.dirname(plan_path), exist_ok=True)
