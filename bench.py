@@ -578,10 +578,22 @@ def main():
                          "rotating over more than 1 GB) and exit: the workload of the rocprofv3 runs" % PROFILE_REPS)
     ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default gpurun_out/prof/<mode>_plan.json)")
     ap.add_argument("--summarize-profile", metavar="DIR", default=None, help="print the text summary of the rocprofv3 output under DIR and exit (no GPU needed)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="compile tests/c_host/kernel_timeline.hip with hipcc and run it: per-workgroup start / loads-arrived / end stamps of the "
+                         "launch shapes behind the config 3-4 rows, next to a one-shot elementwise launch and an empty kernel")
     args = ap.parse_args()
     if args.summarize_profile:
         summarize_profile(args.summarize_profile)
         return
+    if args.timeline:
+        import subprocess
+        import tempfile
+        with tempfile.TemporaryDirectory() as tmp:
+            exe = os.path.join(tmp, "kernel_timeline")
+            subprocess.check_call([os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "-O3", "--offload-arch=gfx950", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
+                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result",
+                                   os.path.join(ROOT, "tests", "c_host", "kernel_timeline.hip"), "-o", exe], stderr=subprocess.DEVNULL)
+            sys.exit(subprocess.call([exe]))
     if args.gpus != 1:
         print("bench.py measures one MI355X: the gradient kernels have no multi-GPU path (every GPU box here has one GPU); "
               "run with --gpus 1", file=sys.stderr)
