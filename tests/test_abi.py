@@ -186,3 +186,22 @@ def test_header_is_plain_c_and_links(built_lib, tmp_path):
     subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
                            "-L", libdir, "-lknet8", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"])
     assert subprocess.call([str(exe)]) == 0
+
+
+def test_the_binary_carries_the_hash_of_the_sources_it_was_built_from(built_lib, monkeypatch):
+    """knet8_build_id() is the hash build.py computes over csrc/*.h, *.hip, gen_knet8.py and build.py: a library left over from other
+    sources cannot pass for the current ones, and the loader refuses it."""
+    build = _load("knet8_build_for_test", "knet.jl_amd/csrc/build.py")
+    lib = ctypes.CDLL(built_lib)
+    lib.knet8_build_id.restype = ctypes.c_char_p
+    have = lib.knet8_build_id().decode()
+    assert have == build.source_id(), "knet.jl_amd/lib/libknet8.so is stale: rebuild it (python __graft_entry__.py build)"
+    lk = _load("lk_for_build_id", "knet.jl_amd/libknet8.py")
+    assert lk.source_build_id() == have
+    assert lk.LibKnet8(built_lib).build_id == have                 # loads: ids agree
+    monkeypatch.setattr(lk, "source_build_id", lambda: "0" * 16)
+    monkeypatch.delenv("KNET8_ALLOW_STALE", raising=False)
+    with pytest.raises(OSError, match="built from other sources"):
+        lk.LibKnet8(built_lib)
+    monkeypatch.setenv("KNET8_ALLOW_STALE", "1")
+    assert lk.LibKnet8(built_lib).build_id == have                 # the override for development
