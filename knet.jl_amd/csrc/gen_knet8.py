@@ -620,7 +620,9 @@ typedef struct ihipStream_t* hipStream_t;
 
 HEADER_RUNTIME = """
 /* ---- runtime: device memory for KnetArray storage, copies, streams, GEMM ---- */
-/* replaces knetMalloc / the free-list pool of src/knetarrays/kptr.jl:105-142,186-194: size-class pool over hipMalloc */
+/* replaces knetMalloc / the free-list pool of src/knetarrays/kptr.jl:105-142,186-194: size-class pool over hipMalloc.
+ * The pool knows nothing of streams, as the reference's does not: a block handed back by knet8_free may be handed out again at once, so free a block
+ * only when the work that uses it was queued on the stream that its next user will queue on too (one stream per pool user), or after knet8_synchronize. */
 KNET8_API void* knet8_malloc(size_t nbytes);
 KNET8_API void knet8_free(void* ptr);
 /* replaces Knet.gc, src/knetarrays/kptr.jl:204-226: hipFree every cached block; returns the bytes released */
