@@ -111,8 +111,12 @@ __device__ __forceinline__ void cut_column(const T* p, int m, int& head, int& nb
   tail = m - head - nb * NV;
 }
 
-template <typename T, typename Algo, int TEAM, int E, bool VEC>
-__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
+// LV > 0 (single-input algorithms): the last LV of a lane's ITEMS vectors live in LDS (slot j of lane t at held[j*BT + t]: 16 bytes per lane,
+// neighbours adjacent) instead of registers, filled by loads that go from memory to LDS directly.  A 32000-row fp64 column is 256 KB: held in
+// registers alone it takes the whole register file of a compute unit -- one workgroup per CU, two rounds of workgroups for 512 columns; with 512
+// lanes holding 23 vectors in registers and 9 in LDS each (72 KB per workgroup), two columns are resident per CU.
+template <typename T, typename Algo, int TEAM, int E, bool VEC, int LV>
+__device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, const T* b, T* out) {
   // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
   // output pass, so the dependent chain is one memory round trip instead of two.
   constexpr bool kHold = Algo::kHoldA || (TEAM == kWave && E <= 16);
@@ -121,8 +125,12 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   constexpr int TEAMS = BT / TEAM;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
   constexpr int ITEMS = E / NV;
+  constexpr int RI = ITEMS - LV;   // vectors per lane in registers
+  static_assert(LV == 0 || (VEC && TEAMS == 1 && RI > 0 && kHold && !kTwo), "LDS slots: whole-workgroup teams of 16-byte vectors, one input");
   typedef typename Vec16<T>::type V;
   __shared__ T lds[BT / kWave];
+  __shared__ V held[LV > 0 ? LV * BT : 1];
+  V* const mine = held + threadIdx.x;
   const int tl = threadIdx.x % TEAM;
   const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
   const bool colok = col < n;  // only wave teams can be out of range
@@ -137,10 +145,16 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   const bool hv = NV > 1 && colok && tl < head, tv = NV > 1 && colok && tl < tail;  // this lane holds a head / a tail element
   const int tpos = head + nb * NV + tl;                                         // where its tail element sits
 
-  V ra[kHold ? ITEMS : 1], rb[kTwo ? ITEMS : 1];
+  // a slot beyond the lane's share stays unwritten and is never read
+#pragma unroll
+  for (int j = 0; j < LV; j++)
+    if (RI + j < cnt)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ac + head + (long)(tl + (RI + j) * TEAM) * NV),
+                                       (__attribute__((address_space(3))) void*)(held + j * BT + (threadIdx.x & ~(kWave - 1))), 16, 0, 2);
+  V ra[kHold ? RI : 1], rb[kTwo ? RI : 1];
   T ah = T(0), at = T(0), bh = T(0), bt = T(0);
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
+  for (int i = 0; i < RI; i++) {
     const long r = head + (long)(tl + i * TEAM) * NV;
     if (i < cnt) {
       if (VEC) {
@@ -160,10 +174,18 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   if (Algo::kNeedMax) {
     mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < ITEMS; i++)
+    for (int i = 0; i < RI; i++)
       if (i < cnt) {
 #pragma unroll
         for (int e = 0; e < NV; e++) mx = mx > ra[i][e] ? mx : ra[i][e];
+      }
+    if (LV > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the direct loads are invisible to the compiler's own bookkeeping
+#pragma unroll
+    for (int j = 0; j < LV; j++)
+      if (RI + j < cnt) {
+        const V v = mine[j * BT];
+#pragma unroll
+        for (int e = 0; e < NV; e++) mx = mx > v[e] ? mx : v[e];
       }
     if (hv) mx = mx > ah ? mx : ah;
     if (tv) mx = mx > at ? mx : at;
@@ -171,7 +193,7 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   }
   T s = T(0);
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++)
+  for (int i = 0; i < RI; i++)
     if (i < cnt) {
 #pragma unroll
       for (int e = 0; e < NV; e++) {
@@ -179,6 +201,19 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
         if constexpr (Algo::kKeepTerm && kHold) ra[i][e] = t;
         s = s + t;
       }
+    }
+  if (LV > 0 && !Algo::kNeedMax) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int j = 0; j < LV; j++)
+    if (RI + j < cnt) {
+      V v = mine[j * BT];
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        const T t = Algo::term(v[e], T(0), mx);
+        if constexpr (Algo::kKeepTerm && kHold) v[e] = t;
+        s = s + t;
+      }
+      if constexpr (Algo::kKeepTerm && kHold) mine[j * BT] = v;
     }
   if (hv) { const T t = Algo::term(ah, bh, mx); if constexpr (Algo::kKeepTerm) ah = t; s = s + t; }
   if (tv) { const T t = Algo::term(at, bt, mx); if constexpr (Algo::kKeepTerm) at = t; s = s + t; }
@@ -188,7 +223,13 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
   for (int i = 0; i < ITEMS; i++) {
     if (i >= cnt) continue;
     const long r = head + (long)(tl + i * TEAM) * NV;
-    V va = {};
+    V va = {}, vb = {};
+    if (i < RI) {
+      if (kHold) va = ra[kHold && i < RI ? i : 0];
+      if (kTwo) vb = rb[kTwo && i < RI ? i : 0];
+    } else {
+      va = mine[(i - RI) * BT];
+    }
     if (!kHold) {
       if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
       else va[0] = __builtin_nontemporal_load(ac + r);
@@ -196,8 +237,8 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
     V vo;
 #pragma unroll
     for (int e = 0; e < NV; e++) {
-      if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(ra[i][e], fin);
-      else vo[e] = Algo::out(kHold ? ra[i][e] : va[e], kTwo ? rb[i][e] : T(0), mx, fin);
+      if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(va[e], fin);
+      else vo[e] = Algo::out(va[e], kTwo ? vb[e] : T(0), mx, fin);
     }
     if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
     else __builtin_nontemporal_store(vo[0], oc + r);
@@ -207,6 +248,16 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax
     if (hv) { if constexpr (Algo::kKeepTerm) oc[tl] = Algo::out_kept(ah, fin); else oc[tl] = Algo::out(ah, bh, mx, fin); }
     if (tv) { if constexpr (Algo::kKeepTerm) oc[tpos] = Algo::out_kept(at, fin); else oc[tpos] = Algo::out(at, bt, mx, fin); }
   }
+}
+
+template <typename T, typename Algo, int TEAM, int E, bool VEC>
+__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
+  softmax_col_body<T, Algo, TEAM, E, VEC, 0>(m, n, a, b, out);
+}
+// four waves per SIMD (two 512-lane workgroups per compute unit): at most 128 registers per lane
+template <typename T, typename Algo, int TEAM, int E, int LV>
+__global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) void softmax_col_lds_kernel(int m, long n, const T* a, const T* b, T* out) {
+  softmax_col_body<T, Algo, TEAM, E, true, LV>(m, n, a, b, out);
 }
 
 // ---- fused nll + logsoftmax backward, register-resident, single reduction ---------------------------------
@@ -235,16 +286,20 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
 
 // The labelled logit is re-read by lane 0 of the team (one scalar load, issued with the others) instead of being
 // fished out of the register that happens to hold it.  Columns are cut into head / vectors / tail as in softmax_col_kernel.
-template <typename T, int TEAM, int E, bool VEC>
-__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
-                                                                            T scale, T* loss) {
+// LV > 0: the last LV vectors of each lane live in LDS, as in softmax_col_body.
+template <typename T, int TEAM, int E, bool VEC, int LV>
+__device__ __forceinline__ void nll_col_body(int m, long n, const T* a, T* out, const int* labels, T scale, T* loss) {
   constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NW = TEAM / kWave;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
   constexpr int ITEMS = E / NV;
+  constexpr int RI = ITEMS - LV;   // vectors per lane in registers
+  static_assert(LV == 0 || (VEC && TEAMS == 1 && RI > 0), "LDS slots: whole-workgroup teams of 16-byte vectors only");
   typedef typename Vec16<T>::type V;
   __shared__ T lds_m[BT / kWave], lds_s[BT / kWave];
+  __shared__ V held[LV > 0 ? LV * BT : 1];
+  V* const mine = held + threadIdx.x;
   const int tl = threadIdx.x % TEAM;
   const long col = (long)blockIdx.x * TEAMS + threadIdx.x / TEAM;
   const bool colok = col < n;
@@ -261,9 +316,16 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
   int lab = colok ? labels[col] : 0;
   if (lab < 0 || lab > m) lab = 0;  // callers check labels on the host; an out-of-range one is skipped, never dereferenced
   const T alab = (tl == 0 && lab > 0) ? ac[lab - 1] : T(0);
-  V rv[ITEMS];
+  V rv[RI];
+  // the LDS slots are filled by loads that go from memory to LDS directly (lane t's 16 bytes land at the wave's base + 16 t), no register in between;
+  // a slot beyond the lane's share stays unwritten and is never read
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
+  for (int j = 0; j < LV; j++)
+    if (RI + j < cnt)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ac + head + (long)(tl + (RI + j) * TEAM) * NV),
+                                       (__attribute__((address_space(3))) void*)(held + j * BT + (threadIdx.x & ~(kWave - 1))), 16, 0, 2);
+#pragma unroll
+  for (int i = 0; i < RI; i++) {
     if (i < cnt) {
       if (VEC) rv[i] = ld_stream(reinterpret_cast<const V*>(ac + head + (long)(tl + i * TEAM) * NV));
       else rv[i][0] = __builtin_nontemporal_load(ac + (tl + i * TEAM));
@@ -276,19 +338,39 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
 
   T mt = ninf;
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++)
+  for (int i = 0; i < RI; i++)
 #pragma unroll
     for (int e = 0; e < NV; e++) mt = mt > rv[i][e] ? mt : rv[i][e];
+  if (LV > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the direct loads are invisible to the compiler's own bookkeeping
+#pragma unroll
+  for (int j = 0; j < LV; j++)
+    if (RI + j < cnt) {
+      const V v = mine[j * BT];
+#pragma unroll
+      for (int e = 0; e < NV; e++) mt = mt > v[e] ? mt : v[e];
+    }
   if (NV > 1) { mt = mt > xh ? mt : xh; mt = mt > xt ? mt : xt; }
   T st = T(0);
   const T mref = mt == ninf ? T(0) : mt;  // a lane without elements holds only -inf padding: exp(-inf - 0) = 0
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++)
+  for (int i = 0; i < RI; i++)
 #pragma unroll
     for (int e = 0; e < NV; e++) {
       const T ex = dev_exp(rv[i][e] - mref);
       rv[i][e] = ex;
       st = st + ex;
+    }
+#pragma unroll
+  for (int j = 0; j < LV; j++)
+    if (RI + j < cnt) {
+      V v = mine[j * BT];
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        const T ex = dev_exp(v[e] - mref);
+        v[e] = ex;
+        st = st + ex;
+      }
+      mine[j * BT] = v;
     }
   if (NV > 1) {
     xh = dev_exp(xh - mref);
@@ -312,10 +394,13 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
   for (int i = 0; i < ITEMS; i++) {
     if (i >= cnt) continue;
     const int r = head + (tl + i * TEAM) * NV;
+    V ve;
+    if (i < RI) ve = rv[i < RI ? i : 0];
+    else ve = mine[(i - RI) * BT];
     V vo;
 #pragma unroll
     for (int e = 0; e < NV; e++) {
-      const T p = rv[i][e] * f;
+      const T p = ve[e] * f;
       const T dlp = (r + e + 1 == lab) ? -scale : T(0);
       vo[e] = lab == 0 ? T(0) : dlp + p;
     }
@@ -326,6 +411,18 @@ __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col
     if (hv) oc[tl] = lab == 0 ? T(0) : ((tl + 1 == lab) ? -scale : T(0)) + xh * f;
     if (tv) oc[tpos] = lab == 0 ? T(0) : ((tpos + 1 == lab) ? -scale : T(0)) + xt * f;
   }
+}
+
+template <typename T, int TEAM, int E, bool VEC>
+__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
+                                                                            T scale, T* loss) {
+  nll_col_body<T, TEAM, E, VEC, 0>(m, n, a, out, labels, scale, loss);
+}
+// four waves per SIMD (two 512-lane workgroups per compute unit): at most 128 registers per lane
+template <typename T, int TEAM, int E, int LV>
+__global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) void nll_col_lds_kernel(int m, long n, const T* a, T* out,
+                                                                                                      const int* labels, T scale, T* loss) {
+  nll_col_body<T, TEAM, E, true, LV>(m, n, a, out, labels, scale, loss);
 }
 
 // ---- streaming fallback for columns too long to hold in registers ----------------------------------------
@@ -716,6 +813,16 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
     if (vec_stream) hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, true>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     else hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, false>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     return;
+  }
+  // fp64 columns of 16 K to 32 K rows: two 512-lane workgroups per compute unit with part of the column in LDS (see nll_col_body)
+  // Measured on (32000,512) fp64, cold: logsoftmax 59.7 -> 44.5 us, softmax 59.8 -> 47.5, fused nll 52.2 -> 42.5; logsoftmaxback, whose output pass
+  // reads a second operand, gains nothing (70.8 -> 71.6) and keeps its registers-only kernel.
+  if constexpr (sizeof(T) == 8 && Algo::kInputs == 1) {
+    if (vec && m > 1024 * (kBig1024 / 2) && m <= 512 * 64 && tuning(kTuneSoftmaxNoLdsSlots) == 0) {
+      if constexpr (Algo::kNll) hipLaunchKernelGGL((nll_col_lds_kernel<T, 512, 64, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, out, labels, scale, loss);
+      else hipLaunchKernelGGL((softmax_col_lds_kernel<T, Algo, 512, 64, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, b, out);
+      return;
+    }
   }
   if (m <= 64 * 4) KNET8_SM(64, 4);
   else if (m <= 64 * 16) KNET8_SM(64, 16);

@@ -38,6 +38,37 @@ def test_forward_and_backward_over_column_lengths(knet, oracle, dt):
     knet.libknet8().check()
 
 
+def test_fp64_columns_held_partly_in_lds(knet, oracle):
+    """fp64 columns of 16385 to 32768 rows: the single-input kernels (logsoftmax, softmax, fused nll) keep 9 of each lane's 32 vectors in LDS.
+    Column lengths at both ends of the range, odd lengths (columns start on and off 16-byte boundaries in turn), a skipped instance; checked
+    against the oracle, and the registers-only kernels (knet8_tune key 6 = 1) must agree to the same tolerance."""
+    rng = np.random.default_rng(36)
+    fn = knet.libknet8().fn
+    rtol = 1e-12
+    for m, n in ((16385, 3), (20001, 7), (32000, 9), (32767, 4), (32768, 5)):
+        x = (rng.standard_normal((m, n)) * 2).astype(np.float64)
+        labels = rng.integers(1, m + 1, size=n)
+        labels[1] = 0
+        want_lsm, want_sm = oracle.logsoftmax(x, dims=1), oracle.softmax(x, dims=1)
+        want_grad, want_loss = oracle.nll_back(x, labels), oracle.nll(x, labels)
+        for knob in (0, 1):
+            old = fn["knet8_tune"](6, knob)
+            try:
+                xd = knet.KnetArray(x)
+                lsm = knet.Array(knet.logsoftmax(xd, dims=1))
+                assert np.abs(lsm - want_lsm).max() <= rtol * np.abs(want_lsm).max(), (m, knob)
+                assert close(knet.Array(knet.softmax(xd, dims=1)), want_sm, rtol), (m, knob)
+                p = knet.Param(knet.KnetArray(x))
+                J = knet.diff(lambda: knet.nll(p, labels, fused=True))
+                assert abs(float(knet.value(J)) - float(want_loss)) <= rtol * abs(float(want_loss)), (m, knob)
+                g = knet.Array(knet.grad(J, p))
+                assert close(g, want_grad, rtol), (m, knob)
+                assert np.all(g[:, 1] == 0)
+            finally:
+                fn["knet8_tune"](6, old)
+    knet.libknet8().check()
+
+
 def test_other_dims_and_misaligned_columns(knet, oracle):
     rng = np.random.default_rng(32)
     x = (rng.standard_normal((10, 100)) * 2).astype(np.float32)
