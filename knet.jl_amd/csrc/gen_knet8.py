@@ -674,7 +674,7 @@ KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hip
    every product of gemm_S / gemm_bias_act_S goes to hipBLASLt);
    key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270);
    key 5: non-zero makes the library behave as if the scratch memory of split launches could not be allocated (for tests of that error path);
-   key 6: non-zero keeps fp64 softmax columns of 16385 to 32768 rows in registers alone instead of registers + LDS (for comparisons) */
+   key 6: non-zero keeps softmax columns of 128 to 256 KB in registers alone instead of registers + LDS (for comparisons) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
    src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */

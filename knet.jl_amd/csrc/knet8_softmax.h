@@ -814,13 +814,16 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
     else hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, false>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     return;
   }
-  // fp64 columns of 16 K to 32 K rows: two 512-lane workgroups per compute unit with part of the column in LDS (see nll_col_body)
+  // Columns of 128 to 256 KB: two 512-lane workgroups per compute unit with part of the column in LDS (see softmax_col_body).
   // Measured on (32000,512) fp64, cold: logsoftmax 59.7 -> 44.5 us, softmax 59.8 -> 47.5, fused nll 52.2 -> 42.5; logsoftmaxback, whose output pass
   // reads a second operand, gains nothing (70.8 -> 71.6) and keeps its registers-only kernel.
-  if constexpr (sizeof(T) == 8 && Algo::kInputs == 1) {
-    if (vec && m > 1024 * (kBig1024 / 2) && m <= 512 * 64 && tuning(kTuneSoftmaxNoLdsSlots) == 0) {
-      if constexpr (Algo::kNll) hipLaunchKernelGGL((nll_col_lds_kernel<T, 512, 64, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, out, labels, scale, loss);
-      else hipLaunchKernelGGL((softmax_col_lds_kernel<T, Algo, 512, 64, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, b, out);
+  // The same 512-lane kernels serve fp32 columns of 32 769 to 65 536 rows (vocabularies of 50257 entries): forward kernels 44.5 -> 41.6 and 46.4 -> 40.7 us
+  // on (50257,512); the fused fp32 nll kernel is as fast from registers alone (42.4 against 45.8) and keeps them.
+  if constexpr (Algo::kInputs == 1 && (!Algo::kNll || sizeof(T) == 8)) {
+    constexpr int kLdsE = 32 * N;   // 32 vectors per lane, 512 lanes: columns of up to 256 KB (32768 fp64 or 65536 fp32 rows)
+    if (vec && m > 1024 * (kBig1024 / 2) && m <= 512 * kLdsE && tuning(kTuneSoftmaxNoLdsSlots) == 0) {
+      if constexpr (Algo::kNll) hipLaunchKernelGGL((nll_col_lds_kernel<T, 512, kLdsE, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, out, labels, scale, loss);
+      else hipLaunchKernelGGL((softmax_col_lds_kernel<T, Algo, 512, kLdsE, 9>), dim3((unsigned)n), dim3(512), 0, stream, (int)m, n, a, b, out);
       return;
     }
   }

@@ -38,7 +38,7 @@ def test_forward_and_backward_over_column_lengths(knet, oracle, dt):
     knet.libknet8().check()
 
 
-def test_fp64_columns_held_partly_in_lds(knet, oracle):
+def test_columns_held_partly_in_lds(knet, oracle):
     """fp64 columns of 16385 to 32768 rows: the single-input kernels (logsoftmax, softmax, fused nll) keep 9 of each lane's 32 vectors in LDS.
     Column lengths at both ends of the range, odd lengths (columns start on and off 16-byte boundaries in turn), a skipped instance; checked
     against the oracle, and the registers-only kernels (knet8_tune key 6 = 1) must agree to the same tolerance."""
@@ -64,6 +64,18 @@ def test_fp64_columns_held_partly_in_lds(knet, oracle):
                 g = knet.Array(knet.grad(J, p))
                 assert close(g, want_grad, rtol), (m, knob)
                 assert np.all(g[:, 1] == 0)
+            finally:
+                fn["knet8_tune"](6, old)
+    # the same kernels serve fp32 forward passes over columns of 32769 to 65536 rows
+    for m, n in ((32769, 3), (50257, 6), (65536, 2)):
+        x = (rng.standard_normal((m, n)) * 2).astype(np.float32)
+        want_lsm, want_sm = oracle.logsoftmax(x, dims=1), oracle.softmax(x, dims=1)
+        for knob in (0, 1):
+            old = fn["knet8_tune"](6, knob)
+            try:
+                xd = knet.KnetArray(x)
+                assert close(knet.Array(knet.logsoftmax(xd, dims=1)), want_lsm), (m, knob)
+                assert close(knet.Array(knet.softmax(xd, dims=1)), want_sm), (m, knob)
             finally:
                 fn["knet8_tune"](6, old)
     knet.libknet8().check()
