@@ -10,7 +10,7 @@ import math
 
 import numpy as np
 
-from .autograd import primitive
+from .autograd import primitive, selective
 from .karray import KnetArray
 from .libknet8 import knet8
 
@@ -61,24 +61,40 @@ def back111_op(name, x, y, dy):
     return dx
 
 
-def reluback(dy, y):
-    return back11_op("reluback", dy, y)
+def _second_order(name, wrt_y):
+    """``Fback(dy,y)`` as a tape primitive of its own, with the rules the reference declares for it, e.g.
+    ``@primitive sigmback(dy,y),ddx  ddx.*y.*(1 .- y)  ddx.*dy.*(1 .- 2 .* y)`` (src/ops20/activation.jl:15,29,42,58;
+    src/ops20_gpu/activation.jl:13 for tanhback), which test/unary.jl:73-77 checks with ``@gcheck``.  The rule for ``dy`` is in every
+    case the function itself applied to ``ddx`` -- ``ddx.*(y.>0)`` is ``reluback.(ddx,y)``, ``ddx.*y.*(1 .- y)`` is ``sigmback.(ddx,y)``
+    with the same operation order -- so it runs the same kernel; ``wrt_y(ddx, dy, y)`` is the rule for ``y`` (None: no gradient)."""
+    @primitive
+    def f(dy, y):
+        dx = back11_op(name, dy, y)
+
+        @selective
+        def back(ddx, need=(True, True)):
+            return (back11_op(name, ddx, y) if need[0] else None,
+                    wrt_y(ddx, dy, y) if need[1] and wrt_y is not None else None)
+        return dx, back
+
+    f.__name__ = name
+    return f
 
 
-def sigmback(dy, y):
-    return back11_op("sigmback", dy, y)
+def _bop(name, a, b):
+    from .binary import broadcast_op
+    return broadcast_op(name, a, b)
 
 
-def tanhback(dy, y):
-    return back11_op("tanhback", dy, y)
+def _negative_part(ddx, dy, y):
+    return _bop("mul", _bop("mul", ddx, dy), _bop("lt", y, 0))        # ddx.*dy.*(y.<0)
 
 
-def eluback(dy, y):
-    return back11_op("eluback", dy, y)
-
-
-def seluback(dy, y):
-    return back11_op("seluback", dy, y)
+reluback = _second_order("reluback", None)                                                                    # (ddx.*(y.>0))  nothing
+sigmback = _second_order("sigmback", lambda ddx, dy, y: _bop("mul", _bop("mul", ddx, dy), _bop("sub", 1, _bop("mul", 2, y))))   # ddx.*dy.*(1 .- 2 .* y)
+tanhback = _second_order("tanhback", lambda ddx, dy, y: _bop("mul", ddx, _bop("mul", _bop("mul", -2, dy), y)))                 # ddx.*(-2 .* dy.*y)
+eluback = _second_order("eluback", _negative_part)
+seluback = _second_order("seluback", _negative_part)
 
 
 def _activation(name, back):

@@ -8,7 +8,8 @@ restates that published behaviour for the primitives on the gradient path:
     J = diff(lambda: nll(predict(w, x), y))      # @diff nll(predict(w,x),y)
     grad(J, w[0]); value(J)
 
-Only what the MLP backward step needs is here (no higher-order gradients, no Sparse containers).
+Only what the MLP backward step needs is here: one level of recording (no nested ``diff``; the gradient functions
+``reluback`` ... ``softmaxback`` are primitives with the reference's rules, so they can be differentiated when called directly), no Sparse containers.
 """
 import numpy as np
 

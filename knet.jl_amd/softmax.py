@@ -7,7 +7,7 @@ through a transpose as in the reference (``:19-20``), batched over trailing dims
 permutation that brings the reduced dimensions to the front (the reference uses the broadcast/reduction chain of
 src/ops20/softmax.jl:42-74 there).
 """
-from .autograd import primitive
+from .autograd import primitive, selective
 from .karray import KnetArray
 from .libknet8 import knet8
 from . import reduction as R
@@ -141,16 +141,53 @@ softmax = _make("softmax", "softmaxback")
 logp = logsoftmax  # const logp = logsoftmax  (src/ops20/softmax.jl:40)
 
 
+def _colsum(a, m, n):
+    return R.sum(a.reshape(m, n), dims=1)    # (1, n)
+
+
+@primitive
 def logsoftmaxback(y, dy, dims=None):
-    """``∇logsoftmax``: ``dy - exp.(y).*sum(dy;dims)`` (src/ops20/softmax.jl:49-51)."""
+    """``∇logsoftmax``: ``dy - exp.(y).*sum(dy;dims)`` (src/ops20/softmax.jl:49-51).  Differentiable in both arguments with the rules the
+    reference gives its cuDNN call (``csb1``/``csb2``, LOG branch, src/ops20_gpu/softmax.jl:61-83):
+    wrt y ``-ddx .* exp.(y) .* sum(dy;dims)``, wrt dy ``ddx .- sum(ddx .* exp.(y);dims)``."""
+    from .activation import unary_op
+    from .binary import broadcast_op as bop
     m, n = _columns(y, dims)
-    return _bwd("logsoftmaxback", y, dy, m, n)
+    dx = _bwd("logsoftmaxback", y, dy, m, n)
+
+    @selective
+    def back(ddx, need=(True, True)):
+        ey = unary_op("exp", y).reshape(m, n)
+        d2 = ddx.reshape(m, n)
+        gy = gdy = None
+        if need[0]:
+            gy = bop("mul", bop("mul", bop("mul", -1, d2), ey), _colsum(dy, m, n)).reshape(y.dims)
+        if need[1]:
+            gdy = bop("sub", d2, _colsum(bop("mul", d2, ey), m, n)).reshape(y.dims)
+        return gy, gdy
+    return dx, back
 
 
+@primitive
 def softmaxback(y, dy, dims=None):
-    """``∇softmax``: ``y.*dy .- y.*sum(y.*dy;dims)`` (src/ops20/softmax.jl:61-63)."""
+    """``∇softmax``: ``y.*dy .- y.*sum(y.*dy;dims)`` (src/ops20/softmax.jl:61-63).  Differentiable in both arguments (``csb1``/``csb2``,
+    ACCURATE branch, src/ops20_gpu/softmax.jl:61-83): wrt y ``ddx.*dy - dy.*sum(y.*ddx) - ddx.*sum(y.*dy)``, wrt dy
+    ``y.*(ddx .- sum(y.*ddx))``, which is ``∇softmax(y, ddx)`` itself and runs the same kernel."""
+    from .binary import broadcast_op as bop
     m, n = _columns(y, dims)
-    return _bwd("softmaxback", y, dy, m, n)
+    dx = _bwd("softmaxback", y, dy, m, n)
+
+    @selective
+    def back(ddx, need=(True, True)):
+        gy = gdy = None
+        if need[0]:
+            y2, dy2, d2 = y.reshape(m, n), dy.reshape(m, n), ddx.reshape(m, n)
+            t = bop("sub", bop("mul", d2, dy2), bop("mul", dy2, _colsum(bop("mul", y2, d2), m, n)))
+            gy = bop("sub", t, bop("mul", d2, _colsum(bop("mul", y2, dy2), m, n))).reshape(y.dims)
+        if need[1]:
+            gdy = _bwd("softmaxback", y, ddx, m, n)
+        return gy, gdy
+    return dx, back
 
 
 @primitive
