@@ -22,6 +22,7 @@ import ctypes
 import json
 import os
 import sys
+import tempfile
 import time
 
 import numpy as np
@@ -576,7 +577,7 @@ def main():
     ap.add_argument("--profile-pass", choices=["warm", "cold"], default=None,
                     help="launch each quoted kernel %d times (config 2 after a known-size copy kernel; configs 3-5 on one buffer set or "
                          "rotating over more than 1 GB) and exit: the workload of the rocprofv3 runs" % PROFILE_REPS)
-    ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default gpurun_out/prof/<mode>_plan.json)")
+    ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default <tmp>/knet8_profile/<mode>_plan.json)")
     ap.add_argument("--summarize-profile", metavar="DIR", default=None, help="print the text summary of the rocprofv3 output under DIR and exit (no GPU needed)")
     ap.add_argument("--timeline", action="store_true",
                     help="compile tests/c_host/kernel_timeline.hip with hipcc and run it: per-workgroup start / loads-arrived / end stamps of the "
@@ -608,7 +609,7 @@ def main():
     if not os.environ.get("KNET8_BENCH_NULL_STREAM"):
         K.libknet8().stream = K.libknet8().fn["knet8_stream_create"]()
     if args.profile_pass:
-        plan_path = args.plan_out or os.path.join(ROOT, "gpurun_out", "prof", args.profile_pass + "_plan.json")
+        plan_path = args.plan_out or os.path.join(tempfile.gettempdir(), "knet8_profile", args.profile_pass + "_plan.json")
         os.makedirs(os.path.dirname(plan_path), exist_ok=True)
         profile_pass(torch, K, args.profile_pass, plan_path)
         print(json.dumps({"profile_pass": args.profile_pass, "plan": plan_path}))
