@@ -66,6 +66,14 @@ def test_columns_held_partly_in_lds(knet, oracle):
                 assert np.all(g[:, 1] == 0)
             finally:
                 fn["knet8_tune"](6, old)
+    # a base pointer inside an allocation, 8 bytes off the 16-byte grid: every operand of the call must be congruent for the vector path
+    from gpu_util import misaligned
+    m, n = 20002, 3
+    x = (rng.standard_normal((m, n)) * 2).astype(np.float64)
+    xd = misaligned(knet, x, 1).reshape(m, n)
+    yd = misaligned(knet, np.zeros_like(x), 1).reshape(m, n)
+    fn["logsoftmax_64_stream"](m, n, xd.ptr, yd.ptr, knet.libknet8().stream)
+    assert np.abs(knet.Array(yd) - oracle.logsoftmax(x, dims=1)).max() <= rtol * 30
     # the same kernels serve fp32 forward passes over columns of 32769 to 65536 rows
     for m, n in ((32769, 3), (50257, 6), (65536, 2)):
         x = (rng.standard_normal((m, n)) * 2).astype(np.float32)
