@@ -8,8 +8,8 @@
 // One "team" of lanes owns a column and keeps it in registers, so every operand is read from HBM exactly
 // once and the result written once: the column is loaded with 16-byte vectors, reduced (max, then sum)
 // with wave64 butterflies (+ LDS across waves), transformed and stored.  Team size follows the column
-// length: one wave (m <= 4096), a 256-thread workgroup (m <= 16384) or a 1024-thread workgroup
-// (m <= 65536 in fp32, half of each limit when two inputs are held or in fp64); longer columns fall back to a
+// length: one wave (m <= 1024), a 256-thread workgroup or a 1024-thread workgroup (up to 65536 rows in fp32, half
+// of that when two inputs are held or in fp64; the table is in launch_softmax); longer columns fall back to a
 // two-pass streaming kernel.
 //
 // HBM roofline: forward 2*sizeof(T)*m*n; backward 3*sizeof(T)*m*n; fused nll backward 2*sizeof(T)*m*n.
@@ -792,11 +792,9 @@ template <typename T, typename Algo>
 inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const T* b, T* out, const int* labels, T scale, T* loss) {
   if (m <= 0 || n <= 0) return;
   constexpr int N = Vec16<T>::N;
-  // Per-lane capacity: a lane of a wave or 256-lane team may hold 64 elements (32 when two inputs are held); the
-  // 1024-lane workgroup is limited to 128 registers per lane, i.e. 64 fp32 / 32 fp64 held elements (half with two held
+  // Per-lane capacity: the 1024-lane workgroup is limited to 128 registers per lane, i.e. 64 fp32 / 32 fp64 held elements (half with two held
   // inputs) -- more than that spills.  Longer columns stream.
   constexpr int kHeld = (Algo::kInputs == 2 && Algo::kHoldA) ? 2 : 1;
-  constexpr int kBig = 64 / kHeld;
   constexpr int kBig1024 = 256 / (int)(sizeof(T) * kHeld);
   // The fused nll kernel in fp32 holds up to 128 elements per lane in a 256-lane team (four waves, one per SIMD, two teams per compute
   // unit): on 32000-row columns 21.8-22.1 us against 22.0-22.3 us for the 1024-lane team (a barrier among four waves instead of sixteen).
@@ -827,10 +825,18 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
       return;
     }
   }
+  // Team and elements per lane by column length, from a sweep over m = 2000 ... 24000 in both widths (cold, 67-100 MB per launch; fractions of
+  // 8 TB/s): many lanes with few elements each beat few lanes with many -- one wave holding a 4000-row column (64 elements per lane) gave
+  // 0.63-0.64 where a 256-lane team gives 0.69-0.70; logsoftmaxback, which streams its second operand in the output pass, does best with 1024
+  // lanes from 2 K rows on (12000 rows fp32: 0.61 with 256 lanes x 64, 0.74 with 1024 x 16).  fp64 single-input kernels keep 256-lane teams up to
+  // 16 K rows (their exp needs the registers a 1024-lane workgroup cannot give: 0.68 against 0.61 at 6000 rows).
+  constexpr bool kStreamsA = Algo::kInputs == 2 && !Algo::kHoldA;
+  constexpr bool kWideSingle = sizeof(T) == 8 && Algo::kInputs == 1;
   if (m <= 64 * 4) KNET8_SM(64, 4);
   else if (m <= 64 * 16) KNET8_SM(64, 16);
-  else if (m <= 64 * kBig) KNET8_SM(64, kBig);
-  else if (m <= 256 * kBig) KNET8_SM(256, kBig);
+  else if (m <= 256 * 16) { if (kStreamsA && m > 2048) KNET8_SM(1024, 8); else KNET8_SM(256, 16); }
+  else if (m <= 1024 * 8) { if constexpr (kWideSingle) KNET8_SM(256, 32); else KNET8_SM(1024, 8); }
+  else if (m <= 1024 * 16) { if constexpr (kWideSingle) KNET8_SM(256, 64); else KNET8_SM(1024, 16); }
   else if (kWideNll && m <= 256 * 128) { if constexpr (kWideNll) KNET8_SM(256, 128); }
   else if (m <= 1024 * (kBig1024 / 2)) KNET8_SM(1024, kBig1024 / 2);
   else KNET8_SM(1024, kBig1024);
