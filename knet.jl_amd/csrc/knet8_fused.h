@@ -131,11 +131,11 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
       for (int w = 0; w < NW; w++) r = r + lds[w][threadIdx.x];
       st_coherent(partial + (at * P + p) * TILE + threadIdx.x, r);
     }
-    if (!last_block_ticket(counters + at, P, &flag)) return;
+    if (!last_block_ticket(counters + at * kTicketStride, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = T(0);
     strided_walk<T, RedSum<T>, NV, false, NW, U, SC>(partial + at * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
-    if (threadIdx.x == 0) st_coherent(counters + at, 0u);
+    if (threadIdx.x == 0) st_coherent(counters + at * kTicketStride, 0u);
   }
 #pragma unroll
   for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
@@ -163,7 +163,7 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
-    ws = workspace_for(stream, sizeof(T) * (size_t)atiles * P * tile, (size_t)atiles);
+    ws = workspace_for(stream, sizeof(T) * (size_t)atiles * P * tile, (size_t)atiles * kTicketStride);
     if (!scratch_ready(ws, "activation gradient + bias gradient: no scratch memory for a split launch")) return;
   }
   const dim3 grid((unsigned)(atiles * P));

@@ -9,7 +9,10 @@
 //   run view      x(sy, ny, no)  ->  y(ny)      reduce axes 1 and 3   (`_21` with sy>1, `_20`, `_22` with s1==1)
 //   strided view  x(s1, d, nb)   ->  y(s1, nb)  reduce axis 2         (`_21` with sy==1, `_22` with s1>1)
 //
-// Both split the reduced axis over P workgroups per output group when one group alone would leave the
+// Short runs and short contiguous axes (a (10, N) matrix summed over its columns, a (2, N) matrix over its rows) go to a third kernel that reads
+// stretches of neighbouring runs or of whole slabs (reduce_stretch_kernel).
+//
+// All split the reduced axis over P workgroups per output group when one group alone would leave the
 // machine idle or take too long; the P partials are combined, in fixed order, by whichever workgroup
 // draws the last ticket of its group, so one launch suffices and the result is deterministic (no float atomics).
 //
@@ -96,13 +99,13 @@ __global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x,
     return;
   }
   if (threadIdx.x == 0) st_coherent(partial + j * P + p, r);
-  if (!last_block_ticket(counters + j, P, &flag)) return;
+  if (!last_block_ticket(counters + j * kTicketStride, P, &flag)) return;
   T s = Op::init();
   for (unsigned q = threadIdx.x; q < P; q += BT) s = Op::merge(s, ld_coherent(partial + j * P + q));
   s = block_reduce<T, NW>(s, lds, MergeFn<Op, T>(), Op::init());
   if (threadIdx.x == 0) {
     y[j] = s;
-    st_coherent(counters + j, 0u);
+    st_coherent(counters + j * kTicketStride, 0u);
   }
 }
 
@@ -190,11 +193,11 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
       for (int w = 0; w < NW; w++) r = Op::merge(r, lds[w][threadIdx.x]);
       st_coherent(partial + (group * P + p) * TILE + threadIdx.x, r);
     }
-    if (!last_block_ticket(counters + group, P, &flag)) return;
+    if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
     strided_walk<T, Op, NV, false, NW, U, SC>(partial + group * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
-    if (threadIdx.x == 0) st_coherent(counters + group, 0u);
+    if (threadIdx.x == 0) st_coherent(counters + group * kTicketStride, 0u);
   }
 #pragma unroll
   for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
@@ -208,56 +211,124 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
   }
 }
 
-// Strided view with a short contiguous axis (s1 < 64): lanes along `a` alone would idle most of a wave,
-// so the (s1 x d) slab of batch b is walked as one contiguous range, L = s1*floor(256/s1) lanes at a
-// time; lane t always meets a == t % s1.  Workgroup (b,p) covers elements [p*chunk, (p+1)*chunk) of the
-// slab (chunk is a multiple of L).
-template <typename T, typename Op>
-__global__ __launch_bounds__(kRedBlock) void reduce_strided_small_kernel(const T* __restrict__ x, int s1, long d, long chunk,
-                                                                         unsigned P, T* __restrict__ y, T* partial,
-                                                                         unsigned* counters) {
-  __shared__ T lds[kRedBlock];
+// ---- stretches of short runs ------------------------------------------------------------------------
+// Run view whose runs are short (sy of at most a few hundred elements), and the strided view with a short contiguous axis.  One wave per output
+// would read a few bytes per lane and leave most lanes idle (run view), or have lanes read `s1` elements apart; instead a workgroup takes a
+// STRETCH of E contiguous elements -- the runs of g neighbouring outputs (R = 1), or, when all ny outputs of a slab fit several times, R whole
+// slabs (g = ny) -- so that wave instructions read whole cache lines whatever sy is.  Lane t holds elements (t + 256 q) NV .. +NV-1 of the stretch,
+// q < U, and sums them over the stretches of its part, `iter_stride` elements apart; which output an element belongs to depends on its place in
+// the stretch only: (i / sy) % g.  At the end the accumulators go to LDS and a team of TL lanes reduces the R*sy entries of each output.
+// P workgroups split the iterations of a group; the last to finish combines their g-vectors in fixed order.
+template <typename T, typename Op, int NV, int U>
+__global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __restrict__ x, int sy, int g_full, long nout, int R, int TL, long group_stride,
+                                                                  long iter_stride, long iters, long iters_per_part, long limit, unsigned P,
+                                                                  T* __restrict__ y, T* partial, unsigned* counters) {
+  constexpr int CAP = kRedBlock * U * NV;
+  constexpr int O = 4;   // stretches in flight per lane
+  __shared__ T lds[CAP + CAP / 32];
   __shared__ unsigned flag;
-  const long b = blockIdx.x / P;
+  const long group = blockIdx.x / P;
   const unsigned p = blockIdx.x % P;
-  const int reps = kRedBlock / s1, L = reps * s1;
-  const long total = (long)s1 * d;
-  const long i0 = (long)p * chunk;
-  long i1 = i0 + chunk;
-  if (i1 > total) i1 = total;
-  const T* xb = x + b * total;
-  T acc = Op::init();
-  if ((int)threadIdx.x < L) {
-    constexpr int U = 4;
-    for (long i = i0 + threadIdx.x; i < i1; i += (long)L * U) {
-      T v[U];
+  const long j0 = group * g_full;
+  const int g = (int)(nout - j0 < g_full ? nout - j0 : g_full);   // outputs of this group (nout: outputs of the whole launch)
+  const int E = R * g * sy;                                   // elements of one stretch
+  const T* base = x + group * group_stride;
+  const long t0 = (long)p * iters_per_part;
+  long t1 = t0 + iters_per_part;
+  if (t1 > iters) t1 = iters;
+  T acc[U][NV];
+#pragma unroll
+  for (int q = 0; q < U; q++)
+#pragma unroll
+    for (int e = 0; e < NV; e++) acc[q][e] = Op::init();
+  for (long t = t0; t < t1; t += O) {
+    T v[O][U][NV];
+#pragma unroll
+    for (int o = 0; o < O; o++) {
+      const long at = (t + o) * iter_stride;
 #pragma unroll
       for (int q = 0; q < U; q++) {
-        const long ii = i + (long)q * L;
-        v[q] = ii < i1 ? Op::item(__builtin_nontemporal_load(xb + ii)) : Op::init();
-      }
+        const int i = ((int)threadIdx.x + q * kRedBlock) * NV;
+        if (t + o < t1 && i < E && at + i < limit) {
+          if (NV > 1) {
+            typedef typename Vec16<T>::type V;
+            const V w = ld_stream(reinterpret_cast<const V*>(base + at + i));
 #pragma unroll
-      for (int q = 0; q < U; q++) acc = Op::merge(acc, v[q]);
+            for (int e = 0; e < NV; e++) v[o][q][e] = (i + e < E && at + i + e < limit) ? Op::item(w[e]) : Op::init();
+          } else {
+            v[o][q][0] = Op::item(__builtin_nontemporal_load(base + at + i));
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < NV; e++) v[o][q][e] = Op::init();
+        }
+      }
+    }
+#pragma unroll
+    for (int o = 0; o < O; o++)
+#pragma unroll
+      for (int q = 0; q < U; q++)
+#pragma unroll
+        for (int e = 0; e < NV; e++) acc[q][e] = Op::merge(acc[q][e], v[o][q][e]);
+  }
+  // one padding word per 32 entries: a team walks entries TL apart, neighbouring teams start sy apart
+#pragma unroll
+  for (int q = 0; q < U; q++)
+#pragma unroll
+    for (int e = 0; e < NV; e++) {
+      const int i = ((int)threadIdx.x + q * kRedBlock) * NV + e;
+      lds[i + (i >> 5)] = acc[q][e];
+    }
+  __syncthreads();
+  const int nteams = kRedBlock / TL, team = (int)threadIdx.x / TL, tl = (int)threadIdx.x % TL;
+  const int entries = R * sy;
+  T* mine = P > 1 ? partial + (group * P + p) * g_full : y + j0;
+  for (int jb = 0; jb < g; jb += nteams) {   // the same trip count for every lane of a wave: the shuffles below need all of them
+    const int jl = jb + team;
+    T r = Op::init();
+    if (jl < g)
+      for (int c = tl; c < entries; c += TL) {
+        const int i = ((c / sy) * g + jl) * sy + c % sy;
+        r = Op::merge(r, lds[i + (i >> 5)]);
+      }
+    for (int o = TL >> 1; o > 0; o >>= 1) r = Op::merge(r, __shfl_xor(r, o));
+    if (jl < g && tl == 0) {
+      if (P > 1) st_coherent(mine + jl, r);
+      else mine[jl] = r;
     }
   }
-  lds[threadIdx.x] = acc;
-  __syncthreads();
-  T r = Op::init();
-  const bool owner = (int)threadIdx.x < s1;
-  if (owner)
-    for (int q = 0; q < reps; q++) r = Op::merge(r, lds[threadIdx.x + q * s1]);
-  if (P == 1) {
-    if (owner) y[b * s1 + threadIdx.x] = r;
-    return;
+  if (P == 1) return;
+  if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) return;
+  // Combine: 256/gp lanes per output share the P partials (one lane alone would wait for P memory round trips in a row), eight loads in flight each;
+  // their sums meet in LDS in fixed order.
+  int gp = 1;
+  while (gp < g && gp < kRedBlock) gp <<= 1;
+  const int tlc = kRedBlock / gp;
+  for (int jb = 0; jb < g; jb += gp) {
+    const int jl = jb + (int)threadIdx.x % gp;
+    T r = Op::init();
+    if (jl < g) {
+      const T* pj = partial + group * P * g_full + jl;
+      unsigned q = threadIdx.x / gp;
+      for (; q + 7 * tlc < P; q += 8 * tlc) {
+        T v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) v[k] = ld_coherent(pj + (long)(q + k * tlc) * g_full);
+#pragma unroll
+        for (int k = 0; k < 8; k++) r = Op::merge(r, v[k]);
+      }
+      for (; q < P; q += tlc) r = Op::merge(r, ld_coherent(pj + (long)q * g_full));
+    }
+    __syncthreads();
+    lds[threadIdx.x] = r;
+    __syncthreads();
+    if ((int)threadIdx.x < gp && jl < g) {
+      T s = lds[threadIdx.x];
+      for (int k = 1; k < tlc; k++) s = Op::merge(s, lds[threadIdx.x + k * gp]);
+      y[j0 + jl] = s;
+    }
   }
-  if (owner) st_coherent(partial + (b * P + p) * s1 + threadIdx.x, r);
-  if (!last_block_ticket(counters + b, P, &flag)) return;
-  if (owner) {
-    T s = Op::init();
-    for (unsigned q = 0; q < P; q++) s = Op::merge(s, ld_coherent(partial + (b * P + q) * s1 + threadIdx.x));
-    y[b * s1 + threadIdx.x] = s;
-  }
-  if (threadIdx.x == 0) st_coherent(counters + b, 0u);
+  if (threadIdx.x == 0) st_coherent(counters + group * kTicketStride, 0u);
 }
 
 // ---- host-side planning ----------------------------------------------------------------------------
@@ -271,7 +342,7 @@ inline long ceil_div(long a, long b) { return (a + b - 1) / b; }
 inline unsigned plan_parts(long groups, long units_per_group, long min_units_per_wg) {
   const long ncu = tuning(kTuneNumCUs);
   long P = 1;
-  if (groups * 2 <= ncu) P = ceil_div(ncu, groups);
+  if (groups * 2 <= ncu) P = ncu / groups;   // rounded down: one workgroup more than there are CUs would double the time of the CU that gets it
   const long cap = units_per_group / min_units_per_wg;
   if (P > cap) P = cap;
   if (P > 65535) P = 65535;
@@ -279,9 +350,77 @@ inline unsigned plan_parts(long groups, long units_per_group, long min_units_per
   return (unsigned)P;
 }
 
+constexpr long kStretchMaxRun = 128;   // longest run the stretch kernel takes
+
+// Stretch kernel for x(sy, ny, no) -> y(ny) per batch (nb batches, `batch_stride` elements apart, outputs ny apart); sy*ny small enough for
+// whole slabs (R >= 1 of them per stretch) or sy <= kStretchMaxRun.  Returns false if the shape is not one for it.
+template <typename T, typename Op>
+inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long ny, long no, long nb, long batch_stride, T* y,
+                                  const ScratchSource* scratch) {
+  constexpr int N = Vec16<T>::N;
+  constexpr int U1 = 4, UV = 2;
+  const long slab = sy * ny;
+  if (sy > kStretchMaxRun || slab <= 0 || no <= 0) return false;
+  const bool whole = slab <= kRedBlock * U1 / 2;          // whole slabs, several per stretch (the scalar kernel's capacity decides: it must hold for both)
+  if (!whole && nb != 1) return false;
+  auto gcd = [](long a, long b) { while (b) { const long t = a % b; a = b; b = t; } return a; };
+  // 16-byte loads: every stretch must start on a 16-byte boundary and no vector may reach past the end of the array
+  bool vec = aligned16(x) && (nb == 1 || batch_stride % N == 0);
+  int g, R;
+  long groups, group_stride, iter_stride, iters, limit;
+  if (whole) {
+    vec = vec && (no * slab) % N == 0;
+    const int cap = kRedBlock * (vec ? UV * N : U1);
+    g = (int)ny;
+    R = (int)(cap / slab);
+    if (vec) { const long step = N / gcd(N, slab); R = (int)(R / step * step); }   // R*slab is a multiple of N
+    if (R > no) R = (int)no;                                                       // a single stretch, at offset 0
+    if (R < 1) return false;
+    groups = nb; group_stride = batch_stride; iter_stride = R * slab; iters = ceil_div(no, R); limit = no * slab;
+  } else {
+    vec = vec && slab % N == 0;
+    const int cap = kRedBlock * (vec ? UV * N : U1);
+    long G = cap / sy;
+    if (vec) { const long step = N / gcd(N, sy); G = G / step * step; }   // groups start on 16-byte boundaries
+    if (G < 1) return false;
+    if (G > ny) G = ny;
+    g = (int)G; R = 1;
+    groups = ceil_div(ny, G); group_stride = G * sy; iter_stride = slab; iters = no; limit = 0x7fffffffffffffffL;
+  }
+  if (groups > 0x7fffffffL / 2) return false;
+  const long entries = (long)R * sy;
+  int TL = 1;
+  while (TL < kWave && TL * 8 < entries) TL <<= 1;
+  // parts: about two workgroups per compute unit, at least eight stretches each, and the combining pass reads g*P partials
+  const long ncu = tuning(kTuneNumCUs);
+  long P = 1;
+  if (groups < 2 * ncu) P = 2 * ncu / groups;
+  if (P > iters / 8) P = iters / 8;
+  if (P * g > 65536) P = 65536 / g;
+  if (P < 1) P = 1;
+  long ipp = ceil_div(iters, P);
+  P = ceil_div(iters, ipp);
+  Workspace ws = {nullptr, nullptr};
+  if (P > 1) {
+    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * g, (size_t)groups * kTicketStride);
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return true;
+  }
+  const dim3 grid((unsigned)(groups * P));
+  if (vec)
+    hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, N, UV>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride,
+                       iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters);
+  else
+    hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, 1, U1>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride,
+                       iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters);
+  return true;
+}
+
 template <typename T, typename Op>
 inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y, const ScratchSource* scratch = nullptr) {
   if (ny <= 0) return;
+  // Short runs: one run per output and workgroup reads a few bytes per lane (a (2, 16M) matrix summed over its columns took 3.5 ms); stretches of
+  // neighbouring runs instead.  With many slabs the run kernel below is the faster one from 16-element runs on (measured: (64,1024,512) 23 against 44 us).
+  if (ny > 1 && (sy <= 8 || (no == 1 && sy <= 128)) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;
@@ -292,7 +431,7 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
-    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)ny * P, (size_t)ny);
+    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)ny * P, (size_t)ny * kTicketStride);
     if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
   }
   T* partial = static_cast<T*>(ws.partial);
@@ -315,22 +454,8 @@ template <typename T, typename Op>
 inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr) {
   if (s1 <= 0 || nb <= 0) return;
   constexpr int N = Vec16<T>::N;
-  if (s1 < kWave) {
-    const int reps = kRedBlock / (int)s1, L = reps * (int)s1;
-    const long total = s1 * d;
-    unsigned P = plan_parts(nb, ceil_div(total, L), 16);
-    long chunk = ceil_div(ceil_div(total, L), P) * L;
-    P = (unsigned)ceil_div(total, chunk > 0 ? chunk : 1);
-    if (P < 1) P = 1;
-    Workspace ws = {nullptr, nullptr};
-    if (P > 1) {
-      ws = take_scratch(scratch, stream, sizeof(T) * (size_t)nb * P * s1, (size_t)nb);
-      if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
-    }
-    hipLaunchKernelGGL((reduce_strided_small_kernel<T, Op>), dim3((unsigned)(nb * P)), dim3(kRedBlock), 0, stream, x, (int)s1, d,
-                       chunk, P, y, static_cast<T*>(ws.partial), ws.counters);
-    return;
-  }
+  // a short contiguous axis: lanes along `a` alone would idle most of a wave; whole (s1 x R) slabs per stretch instead
+  if (s1 < kWave && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch)) return;
   const bool vec = aligned16(x) && (s1 % N == 0);
   // rows that do not start on 16-byte boundaries: the same tile width from N interleaved 4- or 8-byte loads per lane
   const long tile = (long)kWave * N;
@@ -342,7 +467,7 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
-    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups);
+    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups * kTicketStride);
     if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
   }
   const dim3 grid((unsigned)(groups * P));

@@ -30,6 +30,10 @@ struct ScratchSource {
   Workspace (*get)(void* ctx, hipStream_t stream, size_t partial_bytes, size_t ncounters);
   void* ctx;
 };
+// Tickets of different output groups sit 256 bytes apart: atomics on one 64-byte line are carried out one after the other (11-12 ns each on MI355X,
+// measured: 256 workgroups drawing from 16 counters 4 bytes apart take 1.9 us longer than from counters 256 bytes apart).
+constexpr int kTicketStride = 64;   // in counters
+
 inline Workspace take_scratch(const ScratchSource* src, hipStream_t stream, size_t partial_bytes, size_t ncounters) {
   return src ? src->get(src->ctx, stream, partial_bytes, ncounters) : workspace_for(stream, partial_bytes, ncounters);
 }
