@@ -91,6 +91,45 @@ def test_raw_21_and_22_entry_points_on_odd_shapes_and_misaligned_views(knet, ora
     knet.libknet8().check()
 
 
+def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
+    """Shapes that go to the stretch kernel: runs of at most 128 elements with one slab, runs of at most 8 with many, a contiguous axis shorter than
+    a wave.  Groups with a tail, whole slabs with a last partial stretch, sizes that are and are not multiples of a 16-byte vector, batches, split
+    launches (enough stretches for several parts), base pointers off the 16-byte grid; every operator, exact on integer-valued data."""
+    from gpu_util import misaligned
+    rng = np.random.default_rng(26)
+    for dt, S in ((np.float32, "32"), (np.float64, "64")):
+        runs = [(2, 100001, 1), (8, 4096, 1), (10, 100000, 1), (128, 777, 1), (3, 5, 1), (100, 3355, 1), (127, 40, 1), (64, 2049, 1),
+                (4, 1000, 50), (8, 3, 1000), (2, 2, 100000), (7, 5, 333), (1, 3, 70000), (5, 600, 41), (8, 1, 5), (6, 100000, 3)]
+        for (sy, ny, no) in runs:
+            x = rng.integers(-4, 5, size=(sy, ny, no)).astype(dt)
+            x[x == 0] = 1 if x.size < 2000 else 0
+            for off in (0, 1):
+                xd = misaligned(knet, x, off)
+                # (prod only where no zero meets an overflowed partial product: inf*0 depends on the order)
+                for op in (OPS if x.size < 2000 else [o for o in OPS if o != "prod"] if (off == 0 and x.size < 300000) else ["sum", "maximum"]):
+                    y = knet.KnetArray(np.zeros(ny, dt))
+                    knet.knet8("%s_%s_21" % (op, S), x.size, xd.ptr, sy, ny, y.ptr)
+                    want = oracle.reduce(op, x, dims=(1, 3)).ravel()
+                    assert np.array_equal(knet.Array(y), want), (op, sy, ny, no, off)
+        for (s1, d, nb) in [(2, 1000001, 1), (32, 65536, 1), (63, 1000, 1), (5, 1000, 7), (3, 999, 4), (1, 100000, 3), (16, 3, 2), (7, 300000, 1)]:
+            x = rng.integers(-4, 5, size=(s1, d, nb)).astype(dt)
+            for off in (0, 1):
+                xd = misaligned(knet, x, off)
+                for op in ("sum", "minimum", "sumabs2"):
+                    y = knet.KnetArray(np.zeros((s1, nb), dt))
+                    knet.knet8("%s_%s_22" % (op, S), x.size, d - 1, xd.ptr, s1, s1 * d, s1 * nb, y.ptr)
+                    assert np.array_equal(knet.Array(y), oracle.reduce(op, x, dims=2).reshape(s1, nb)), (op, s1, d, nb, off)
+    # N(0,1) data: 1e-5 of the magnitude summed
+    x = rng.standard_normal((10, 200000)).astype(np.float32)
+    xd = knet.KnetArray(x)
+    check_sum(knet.Array(knet.sum(xd, dims=1)), oracle.reduce("sum", x, dims=1).astype(np.float64), x, 0)
+    check_sum(knet.Array(knet.sum(xd, dims=2)), oracle.reduce("sum", x, dims=2).astype(np.float64), x, 1)
+    # launches one after the other leave the tickets at zero
+    for _ in range(3):
+        assert np.allclose(knet.Array(knet.sum(xd, dims=2)), x.sum(axis=1, keepdims=True, dtype=np.float64), rtol=1e-4, atol=1e-2)
+    knet.libknet8().check()
+
+
 def test_repeated_launches_reuse_the_scratch_correctly(knet):
     # split reductions keep per-stream tickets that every launch must leave at zero
     rng = np.random.default_rng(24)
