@@ -27,15 +27,16 @@ constexpr int kRedBlock = 256;
 constexpr int kRedWaves = kRedBlock / kWave;
 
 // ---- operator table: (merge, item, init) triples of src/libknet8/ops.jl:144-156 ---------------------
-template <typename T> struct RedSum     { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a + x; } };
-template <typename T> struct RedProd    { __host__ __device__ static T init() { return T(1); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a * x; } };
-template <typename T> struct RedMaximum { __host__ __device__ static T init() { return -INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
-template <typename T> struct RedMinimum { __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
-template <typename T> struct RedSumabs  { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a + x; } };
-template <typename T> struct RedSumabs2 { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x * x; } __device__ static T merge(T a, T x) { return a + x; } };
-template <typename T> struct RedMaxabs  { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
-template <typename T> struct RedMinabs  { __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
-template <typename T> struct RedCountnz { __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x != 0 ? T(1) : T(0); } __device__ static T merge(T a, T x) { return a + x; } };
+// Merged: the operator that combines values to which item() has been applied already (partial results of a first pass).
+template <typename T> struct RedSum     { typedef RedSum<T> Merged; __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedProd    { typedef RedProd<T> Merged; __host__ __device__ static T init() { return T(1); } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a * x; } };
+template <typename T> struct RedMaximum { typedef RedMaximum<T> Merged; __host__ __device__ static T init() { return -INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
+template <typename T> struct RedMinimum { typedef RedMinimum<T> Merged; __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
+template <typename T> struct RedSumabs  { typedef RedSum<T> Merged; __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedSumabs2 { typedef RedSum<T> Merged; __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x * x; } __device__ static T merge(T a, T x) { return a + x; } };
+template <typename T> struct RedMaxabs  { typedef RedMaximum<T> Merged; __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a > x ? a : x; } };
+template <typename T> struct RedMinabs  { typedef RedMinimum<T> Merged; __host__ __device__ static T init() { return INFINITY; } __device__ static T item(T x) { return x < 0 ? -x : x; } __device__ static T merge(T a, T x) { return a < x ? a : x; } };
+template <typename T> struct RedCountnz { typedef RedSum<T> Merged; __host__ __device__ static T init() { return T(0); } __device__ static T item(T x) { return x != 0 ? T(1) : T(0); } __device__ static T merge(T a, T x) { return a + x; } };
 
 template <typename Op, typename T> struct MergeFn {
   __device__ __forceinline__ T operator()(T a, T b) const { return Op::merge(a, b); }
@@ -391,10 +392,10 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   const long entries = (long)R * sy;
   int TL = 1;
   while (TL < kWave && TL * 8 < entries) TL <<= 1;
-  // parts: about two workgroups per compute unit, at least eight stretches each, and the combining pass reads g*P partials
+  // parts: about four workgroups per compute unit (measured best of 2, 4, 8, 16), at least eight stretches each, and the combining pass reads g*P partials
   const long ncu = tuning(kTuneNumCUs);
   long P = 1;
-  if (groups < 2 * ncu) P = 2 * ncu / groups;
+  if (groups < 4 * ncu) P = 4 * ncu / groups;
   if (P > iters / 8) P = iters / 8;
   if (P * g > 65536) P = 65536 / g;
   if (P < 1) P = 1;
@@ -416,11 +417,25 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
 }
 
 template <typename T, typename Op>
+inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr, size_t front = 0);
+
+template <typename T, typename Op>
 inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y, const ScratchSource* scratch = nullptr) {
   if (ny <= 0) return;
-  // Short runs: one run per output and workgroup reads a few bytes per lane (a (2, 16M) matrix summed over its columns took 3.5 ms); stretches of
-  // neighbouring runs instead.  With many slabs the run kernel below is the faster one from 16-element runs on (measured: (64,1024,512) 23 against 44 us).
-  if (ny > 1 && (sy <= 8 || (no == 1 && sy <= 128)) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
+  // Short runs.  One slab (a (2, 16M) matrix summed over its columns): one run per workgroup would read a few bytes per lane (3.5 ms); stretches of
+  // neighbouring runs instead.  Many slabs (the bias gradient of a 7x7 feature map, x(49, 2048, N)): the slabs are first added onto each other as
+  // rows of sy*ny contiguous elements by the strided-view kernel, into scratch, then the sy*ny sums are reduced as one slab; the sy*ny extra
+  // elements written and read are nothing next to the no slabs.  (Measured, 134 MB fp32: (4,1000,8388) 158 -> 26.5 us, (49,2048,334) 43.7 -> 28.5 us, (16,16,131072) 35.9 -> 29.0 us.)
+  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave) {
+    const size_t front = (sizeof(T) * (size_t)(sy * ny) + 255) / 256 * 256;
+    Workspace tw = take_scratch(scratch, stream, front, 0);
+    if (tw.partial == nullptr) { record_error("reduction: no scratch memory for the slab sums"); return; }
+    T* tmp = static_cast<T*>(tw.partial);
+    launch_reduce_strided<T, Op>(stream, x, sy * ny, no, 1, tmp, scratch, front);
+    launch_reduce_run<T, typename Op::Merged>(stream, tmp, sy, ny, 1, y, scratch);
+    return;
+  }
+  if (ny > 1 && (sy <= 8 || (no == 1 && sy <= kStretchMaxRun)) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;
@@ -450,8 +465,9 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
 #undef KNET8_RUN
 }
 
+// `front`: bytes at the start of the scratch memory that belong to the caller (the partial results go behind them).
 template <typename T, typename Op>
-inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr) {
+inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch, size_t front) {
   if (s1 <= 0 || nb <= 0) return;
   constexpr int N = Vec16<T>::N;
   // a short contiguous axis: lanes along `a` alone would idle most of a wave; whole (s1 x R) slabs per stretch instead
@@ -467,11 +483,11 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   if (P < 1) P = 1;
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
-    ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * tile, (size_t)groups * kTicketStride);
+    ws = take_scratch(scratch, stream, front + sizeof(T) * (size_t)groups * P * tile, (size_t)groups * kTicketStride);
     if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
   }
   const dim3 grid((unsigned)(groups * P));
-  T* partial = static_cast<T*>(ws.partial);
+  T* partial = reinterpret_cast<T*>(static_cast<char*>(ws.partial) + (ws.partial ? front : 0));
   const bool big = kchunk >= 128;  // sixteen waves share a tile when each still gets >= 8 rows
 #define KNET8_STR(NV, BT, U, SC) \
   hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U, SC>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters)
