@@ -13,7 +13,7 @@ from gpu_util import bits_equal, ulp_diff
 pytestmark = pytest.mark.gpu
 
 ACTS = ["relu", "sigm", "tanh", "elu", "selu"]
-SHAPES = [(1, 1), (3, 5), (10, 100), (64, 100), (257, 33), (256, 1), (1000, 4096), (4096, 2048), (300, 5000), (4100, 130), (8, 70000)]
+SHAPES = [(1, 1), (3, 5), (10, 100), (64, 100), (257, 33), (256, 1), (1000, 4096), (4096, 2048), (300, 5000), (4100, 130), (8, 70000), (3, 100001), (63, 1000)]
 
 
 def sfx(dt):
