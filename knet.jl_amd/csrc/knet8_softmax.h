@@ -425,6 +425,130 @@ __global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
   nll_col_body<T, TEAM, E, true, LV>(m, n, a, out, labels, scale, loss);
 }
 
+// ---- many short columns -----------------------------------------------------------------------------------
+// Columns of at most 128 rows (ten classes, the 21 of a segmentation map): a wave per column would move 40 bytes per instruction.  A workgroup
+// takes a STRETCH of G whole columns instead -- G*m contiguous elements, read and written with full-width accesses whatever m is -- through LDS;
+// a team of TL lanes (a power of two, about m/8) owns a column there: it reads its at most 8 elements per lane from LDS, reduces with shuffles,
+// and puts the results back in place.  The same Algo table as the register-resident kernels; the fused nll variant uses the plain two-reduction
+// form (max, then sum of exp), one exp per element.
+constexpr int kShortRows = 128;
+// LDS layout: one padding word after every 32 entries, so that the teams of a wave, whose columns start m entries apart, do not meet in one bank
+// when m is a power of two.  (Four padding words, which would keep a 16-byte vector whole and aligned for the stretch's way in and out, measured
+// slower: 17 us against 12.4 us at m = 32: the column pass is the one that counts.)
+__device__ __forceinline__ int short_pad(int i) { return i + (i >> 5); }
+
+// R: elements of a column per lane (TL*R >= m).  Slots past the column's end are computed and thrown away, so the host picks, among R = 2, 3, 4, 6, 8,
+// the pair that wastes fewest: ten classes run as 4 lanes x 3, not 2 x 8.
+template <typename T, typename Algo, bool VEC, int R>
+__global__ __launch_bounds__(256) void softmax_short_kernel(int m, long n, int G, int TL, const T* a, const T* b, T* out, const int* labels, T scale,
+                                                            T* loss) {
+  constexpr bool kTwo = Algo::kInputs == 2;
+  constexpr int NV = VEC ? Vec16<T>::N : 1;
+  constexpr int Q = 4;
+  constexpr int CAP = 256 * Q * Vec16<T>::N;     // elements of a stretch: 16 KB
+  typedef typename Vec16<T>::type V;
+  __shared__ T la[CAP + CAP / 32];
+  __shared__ T lb[kTwo ? CAP + CAP / 32 : 1];
+  const long col0 = (long)blockIdx.x * G;
+  const int g = (int)(n - col0 < G ? n - col0 : G);
+  const int E = g * m;
+  const T* ab = a + col0 * m;
+  const T* bb = kTwo ? b + col0 * m : nullptr;
+  T* ob = out + col0 * m;
+  constexpr int PER = VEC ? Q : Q * Vec16<T>::N;   // accesses per lane: the scalar path makes up for its narrow ones
+#pragma unroll
+  for (int q = 0; q < PER; q++) {
+    const int i = ((int)threadIdx.x + q * 256) * NV;
+    if (VEC && i + NV <= E) {
+      const V va = ld_stream(reinterpret_cast<const V*>(ab + i));
+#pragma unroll
+      for (int e = 0; e < NV; e++) la[short_pad(i + e)] = va[e];
+      if (kTwo) {
+        const V vb = ld_stream(reinterpret_cast<const V*>(bb + i));
+#pragma unroll
+        for (int e = 0; e < NV; e++) lb[short_pad(i + e)] = vb[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < NV; e++)
+        if (i + e < E) {
+          la[short_pad(i + e)] = __builtin_nontemporal_load(ab + i + e);
+          if (kTwo) lb[short_pad(i + e)] = __builtin_nontemporal_load(bb + i + e);
+        }
+    }
+  }
+  __syncthreads();
+  const int nteams = 256 / TL, team = (int)threadIdx.x / TL, tl = (int)threadIdx.x % TL;
+  for (int cb = 0; cb < g; cb += nteams) {   // the same trip count for every lane of a wave: the shuffles need all of them
+    const int c = cb + team;
+    const bool live = c < g;
+    // (every slot is processed under a lane predicate: guarding the slots past the column's end with a branch of their own kept the LDS reads
+    //  from being issued back to back and measured 40 % slower at m = 32)
+    T av[R], bv[kTwo ? R : 1], tv[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const int k = tl + r * TL;
+      const int i = short_pad(c * m + k);
+      const bool ok = live && k < m;
+      av[r] = ok ? la[i] : T(0);
+      if (kTwo) bv[r] = ok ? lb[i] : T(0);
+    }
+    T mx = T(0);
+    if (Algo::kNeedMax) {
+      mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < R; r++)
+        if (live && tl + r * TL < m) mx = mx > av[r] ? mx : av[r];
+      for (int o = TL >> 1; o > 0; o >>= 1) { const T t = __shfl_xor(mx, o); mx = mx > t ? mx : t; }
+    }
+    T s = T(0);
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const bool ok = live && tl + r * TL < m;
+      tv[r] = ok ? Algo::term(av[r], kTwo ? bv[r] : T(0), mx) : T(0);
+      s = s + tv[r];
+    }
+    for (int o = TL >> 1; o > 0; o >>= 1) s = s + __shfl_xor(s, o);
+    const T fin = Algo::finish(s);
+    if constexpr (Algo::kNll) {
+      int lab = live ? labels[col0 + c] : 0;
+      if (lab < 0 || lab > m) lab = 0;   // callers check labels on the host; an out-of-range one is skipped, never dereferenced
+      const T f = scale / s;
+      if (live && tl == 0) loss[col0 + c] = lab > 0 ? -((la[short_pad(c * m + lab - 1)] - mx) - fin) : T(0);
+      // every lane of the team has read its elements and the labelled one before anything is overwritten: a team lies within one wave
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const int k = tl + r * TL;
+        if (live && k < m) la[short_pad(c * m + k)] = lab == 0 ? T(0) : ((k + 1 == lab) ? -scale : T(0)) + tv[r] * f;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const int k = tl + r * TL;
+        if (live && k < m) {
+          if constexpr (Algo::kKeepTerm) la[short_pad(c * m + k)] = Algo::out_kept(tv[r], fin);
+          else la[short_pad(c * m + k)] = Algo::out(av[r], kTwo ? bv[r] : T(0), mx, fin);
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < PER; q++) {
+    const int i = ((int)threadIdx.x + q * 256) * NV;
+    if (VEC && i + NV <= E) {
+      V vo;
+#pragma unroll
+      for (int e = 0; e < NV; e++) vo[e] = la[short_pad(i + e)];
+      st_stream(reinterpret_cast<V*>(ob + i), vo);
+    } else {
+#pragma unroll
+      for (int e = 0; e < NV; e++)
+        if (i + e < E) __builtin_nontemporal_store(la[short_pad(i + e)], ob + i + e);
+    }
+  }
+}
+
 // ---- streaming fallback for columns too long to hold in registers ----------------------------------------
 // One 1024-thread workgroup per column, two passes with 16-byte accesses and U of them in flight per lane.
 // Pass 1 reduces: for the max-based algorithms max and sum(exp(x - max)) are carried together as a pair that is
@@ -807,6 +931,44 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   const bool vec_stream = (m % N == 0) && ma == 0 && mo == 0 && mb == 0;
   const long resident_cap = tuning(kTuneSoftmaxResidentRows);  // 0: no limit below the register capacity (tests lower it to reach the streaming kernel with short columns)
 #define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
+  if (m <= kShortRows && n >= 64 && !(resident_cap > 0 && m > resident_cap)) {
+    // stretches of whole columns (see softmax_short_kernel): G columns per workgroup, starting on 16-byte boundaries on the vector path
+    constexpr int cap = 256 * 4 * N;
+    const bool v16 = ma == 0 && mo == 0 && mb == 0;
+    long G = cap / m;
+    if (v16) {
+      long step = N;
+      for (long t = 1; t <= N; t++)
+        if ((t * m) % N == 0) { step = t; break; }
+      G = G / step * step;
+    }
+    if (G >= 1) {
+      // lanes per column and elements per lane: cheapest passes over the workgroup's G columns, a pass costing its R slots plus about six slots' worth
+      // of reductions and bookkeeping (measured: ten classes are faster as 2 lanes x 8 in four passes than as 4 x 3 in seven)
+      int bestR = 8, bestTL = kWave;
+      long best = -1;
+      for (int R : {8, 6, 4, 3, 2}) {
+        int TL = 1;
+        while (TL < kWave && (long)TL * R < m) TL <<= 1;
+        if ((long)TL * R < m) continue;
+        const long slots = ((G + 256 / TL - 1) / (256 / TL)) * (R + 6);
+        if (best < 0 || slots < best) { best = slots; bestR = R; bestTL = TL; }
+      }
+      const dim3 grid((unsigned)((n + G - 1) / G));
+#define KNET8_SHORT(VEC, R) hipLaunchKernelGGL((softmax_short_kernel<T, Algo, VEC, R>), grid, dim3(256), 0, stream, (int)m, n, (int)G, bestTL, a, b, out, labels, scale, loss)
+      if (v16) {
+        switch (bestR) { case 2: KNET8_SHORT(true, 2); break; case 3: KNET8_SHORT(true, 3); break; case 4: KNET8_SHORT(true, 4); break;
+                         case 6: KNET8_SHORT(true, 6); break; default: KNET8_SHORT(true, 8); }
+      } else {
+        int TL = 1;   // operands that are not all on 16-byte boundaries: the one general variant
+        while (TL < kWave && TL * 8 < m) TL <<= 1;
+        bestTL = TL;
+        KNET8_SHORT(false, 8);
+      }
+#undef KNET8_SHORT
+      return;
+    }
+  }
   if ((resident_cap > 0 && m > resident_cap) || m > 1024L * kBig1024) {
     if (vec_stream) hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, true>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);
     else hipLaunchKernelGGL((softmax_col_stream_kernel<T, Algo, false>), dim3((unsigned)n), dim3(1024), 0, stream, m, n, a, b, out, labels, scale, loss);

@@ -89,6 +89,44 @@ def test_columns_held_partly_in_lds(knet, oracle):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_many_short_columns(knet, oracle, dt):
+    """Columns of at most 128 rows, 64 and more of them: workgroups take stretches of whole columns through LDS.  Column lengths around every
+    lanes-per-column choice, a last stretch that is not full, column counts that leave one column over, and operands off the 16-byte grid (the
+    general variant); every function of the family, the fused nll with a skipped instance."""
+    from gpu_util import misaligned
+    rng = np.random.default_rng(37)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    for m, n in ((1, 100), (2, 5001), (3, 4000), (5, 64), (8, 1025), (10, 2000), (16, 777), (21, 1000), (32, 300), (33, 300), (64, 129),
+                 (100, 500), (127, 65), (128, 200)):
+        x = (rng.standard_normal((m, n)) * 2).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        for off in (0, 1):
+            xd = misaligned(knet, x, off).reshape(m, n) if off else knet.KnetArray(x)
+            dyd = misaligned(knet, dy, off).reshape(m, n) if off else knet.KnetArray(dy)
+            want = oracle.logsoftmax(x, dims=1)
+            lsm = knet.Array(knet.logsoftmax(xd, dims=1))
+            assert np.abs(lsm - want).max() <= rtol * max(np.abs(want).max(), 1), (m, n, off)
+            sm = knet.Array(knet.softmax(xd, dims=1))
+            y = oracle.softmax(x, dims=1)
+            assert close(sm, y, rtol), (m, n, off)
+            assert np.allclose(sm.sum(axis=0), 1, atol=100 * rtol)
+            wd = misaligned(knet, want, off).reshape(m, n) if off else knet.KnetArray(want)
+            assert close(knet.Array(knet.logsoftmaxback(wd, dyd, dims=1)), oracle.logsoftmaxback(want, dy, dims=1), rtol), (m, n, off)
+            yd = misaligned(knet, y, off).reshape(m, n) if off else knet.KnetArray(y)
+            assert close(knet.Array(knet.softmaxback(yd, dyd, dims=1)), oracle.softmaxback(y, dy, dims=1), rtol), (m, n, off)
+        labels = rng.integers(1, m + 1, size=n)
+        labels[1] = 0
+        p = knet.Param(knet.KnetArray(x))
+        J = knet.diff(lambda: knet.nll(p, labels, fused=True))
+        want_loss = float(oracle.nll(x, labels))
+        assert abs(float(knet.value(J)) - want_loss) <= rtol * max(abs(want_loss), 1e-3), (m, n)
+        g = knet.Array(knet.grad(J, p))
+        assert close(g, oracle.nll_back(x, labels), rtol), (m, n)
+        assert np.all(g[:, 1] == 0)
+    knet.libknet8().check()
+
+
 def test_other_dims_and_misaligned_columns(knet, oracle):
     rng = np.random.default_rng(32)
     x = (rng.standard_normal((10, 100)) * 2).astype(np.float32)
