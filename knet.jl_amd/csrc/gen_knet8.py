@@ -661,8 +661,9 @@ KNET8_API int knet8_version(void);
    a loader compares it with the working tree and refuses a stale library */
 KNET8_API const char* knet8_build_id(void);
 /* No counterpart in the reference.  sum_32_21 for callers that cannot allocate device memory -- code under hipGraph capture, tight
-   serving loops, harnesses that forbid hipMalloc: the same kernels and the same result, bit for bit, with the partial results and
-   tickets of a split launch in a fixed array inside the library (1 MiB of partials + 4096 tickets per GPU, held until the process
+   serving loops, harnesses that forbid hipMalloc: the same kernels and the same result, bit for bit (except where a launch plan would not fit the fixed array and the planner takes another: then
+   to the 1e-5 of any reduction), with the partial results and
+   tickets of a split launch in a fixed array inside the library (1 MiB of partials + 64 KiB of tickets per GPU, held until the process
    ends) instead of the per-stream buffers that sum_32_21 grows through hipMalloc.  Calls no hipMalloc, hipFree or other allocating
    routine.  A shape whose split needs more than the array holds is refused: the error is recorded and y is left untouched.  All calls
    on one GPU share the array, so calls that overlap in time on one GPU (other streams, other threads) race; calls on one stream are

@@ -398,7 +398,7 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   if (groups < 4 * ncu) P = 4 * ncu / groups;
   if (P > iters / 8) P = iters / 8;
   if (P * g > 65536) P = 65536 / g;
-  if (P < 1) P = 1;
+  if (P < 1 || !scratch_fits(scratch, sizeof(T) * (size_t)groups * P * g, (size_t)groups * kTicketStride)) P = 1;   // a provider of fixed size: no split beyond it
   long ipp = ceil_div(iters, P);
   P = ceil_div(iters, ipp);
   Workspace ws = {nullptr, nullptr};
@@ -426,8 +426,8 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   // neighbouring runs instead.  Many slabs (the bias gradient of a 7x7 feature map, x(49, 2048, N)): the slabs are first added onto each other as
   // rows of sy*ny contiguous elements by the strided-view kernel, into scratch, then the sy*ny sums are reduced as one slab; the sy*ny extra
   // elements written and read are nothing next to the no slabs.  (Measured, 134 MB fp32: (4,1000,8388) 158 -> 26.5 us, (49,2048,334) 43.7 -> 28.5 us, (16,16,131072) 35.9 -> 29.0 us.)
-  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave) {
-    const size_t front = (sizeof(T) * (size_t)(sy * ny) + 255) / 256 * 256;
+  const size_t front = (sizeof(T) * (size_t)(sy * ny) + 255) / 256 * 256;
+  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave && scratch_fits(scratch, 2 * front, 0)) {
     Workspace tw = take_scratch(scratch, stream, front, 0);
     if (tw.partial == nullptr) { record_error("reduction: no scratch memory for the slab sums"); return; }
     T* tmp = static_cast<T*>(tw.partial);

@@ -29,7 +29,12 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
 struct ScratchSource {
   Workspace (*get)(void* ctx, hipStream_t stream, size_t partial_bytes, size_t ncounters);
   void* ctx;
+  size_t partial_capacity, counter_capacity;   // what the provider can serve at most (0: it grows as needed); launch planners that have a choice stay within it
 };
+inline bool scratch_fits(const ScratchSource* src, size_t partial_bytes, size_t ncounters) {
+  return src == nullptr || ((src->partial_capacity == 0 || partial_bytes <= src->partial_capacity) &&
+                            (src->counter_capacity == 0 || ncounters <= src->counter_capacity));
+}
 // Tickets of different output groups sit 256 bytes apart: atomics on one 64-byte line are carried out one after the other (11-12 ns each on MI355X,
 // measured: 256 workgroups drawing from 16 counters 4 bytes apart take 1.9 us longer than from counters 256 bytes apart).
 constexpr int kTicketStride = 64;   // in counters

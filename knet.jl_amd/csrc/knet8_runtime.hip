@@ -144,7 +144,7 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
 // own address, until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel
 // can use is asked from the runtime once per device and kept.
 constexpr size_t kStaticPartialBytes = size_t(1) << 20;
-constexpr size_t kStaticCounters = 4096;
+constexpr size_t kStaticCounters = 16384;   // tickets sit 64 apart: 256 output groups
 static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(unsigned)];
 
 constexpr int kMaxDevices = 64;
@@ -488,7 +488,7 @@ KNET8_API int knet8_version(void) { return 200; }
 KNET8_API const char* knet8_build_id(void) { return KNET8_BUILD_ID; }
 
 KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hipStream_t stream) {
-  const ScratchSource src = {static_scratch_get, nullptr};
+  const ScratchSource src = {static_scratch_get, nullptr, kStaticPartialBytes, kStaticCounters};
   reduce_21<float, RedSum<float>>(stream, nx, x, sy, ny, y, &src);
   check_launch("sum_32_21_noalloc");
 }

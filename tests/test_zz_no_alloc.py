@@ -34,6 +34,15 @@ def test_no_alloc_sum_matches_the_allocating_entry_point(knet):
     for x, sy, ny in ((big, big.size, 1), (small, small.size, 1), (big[:8, :].copy(), 1, 8)):
         got, want = _pair(knet, x, sy, ny)
         assert got.tobytes() == want.tobytes(), (x.shape, sy, ny)
+    # short runs and short contiguous axes (stretches of runs / whole slabs; many slabs of short runs in two passes, whose slab sums sit in the
+    # fixed array too; a matrix of few rows too wide for that goes the old single-launch way instead)
+    for shape, sy, ny in (((10, 30000), 10, 30000), ((2, 1000000), 1, 2), ((4, 1000, 50), 4, 1000), ((8, 3, 4000), 8, 3), ((4, 100000, 9), 4, 100000)):
+        x = rng.standard_normal(shape).astype(np.float32)
+        got, want = _pair(knet, x, sy, ny)
+        if x.size * 4 // shape[-1] * 2 <= (1 << 20) or len(shape) == 2:
+            assert got.tobytes() == want.tobytes(), (shape, sy, ny)      # the same launch plan on both sides
+        v = x.reshape(sy, ny, -1, order="F").astype(np.float64)
+        assert np.all(np.abs(got - v.sum(axis=(0, 2))) <= 1e-5 * np.abs(v).sum(axis=(0, 2)) + 1e-30), shape
     # shapes that need no scratch at all go through as well
     got, want = _pair(knet, big, 4096, 8192)
     assert got.tobytes() == want.tobytes()
