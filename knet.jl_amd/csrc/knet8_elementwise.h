@@ -152,6 +152,37 @@ __global__ __launch_bounds__(kEwBlock) void ew_bias_vec_kernel(long nvec, const 
   st_stream(reinterpret_cast<V*>(z + e), r);
 }
 
+// The same with a vector of any length and stride (1001 classes, a vocabulary of 50257): the full-size operand still moves in 16-byte accesses over
+// the flat array, the vector's entries are fetched one by one (they stay in cache) with the position in the vector carried along instead of divided
+// out per element.  The last n % N elements are done by workgroup 0.  (Measured on (1001, 8380) fp32: 18.0 -> 13.7 us.)
+template <typename T, typename F, bool XFULL>
+__global__ __launch_bounds__(kEwBlock) void ew_bias_gather_kernel(long nvec, long n, const T* full, const T* vec, unsigned s, unsigned nv, T* z, F f) {
+  typedef typename Vec16<T>::type V;
+  constexpr int N = Vec16<T>::N;
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i < nvec) {
+    const long e = i * N;
+    const V a = ld_stream(reinterpret_cast<const V*>(full + e));
+    const unsigned q = (unsigned)e / s;      // n is a 32-bit int at the ABI: 32-bit division
+    unsigned p = (unsigned)e - q * s, idx = q % nv;
+    V r;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+      const T bv = vec[idx];
+      r[k] = XFULL ? f(a[k], bv) : f(bv, a[k]);
+      if (++p == s) { p = 0; if (++idx == nv) idx = 0; }
+    }
+    st_stream(reinterpret_cast<V*>(z + e), r);
+  }
+  if (blockIdx.x == 0) {
+    const long e = nvec * N + threadIdx.x;
+    if (e < n) {
+      const T bv = vec[((unsigned)e / s) % nv];
+      z[e] = XFULL ? f(full[e], bv) : f(bv, full[e]);
+    }
+  }
+}
+
 template <typename T, typename F>
 inline void launch_bcast12(hipStream_t stream, long n, const T* x, int sx, int nx, const T* y, int sy, int ny, T* z, F f) {
   if (n <= 0) return;
@@ -166,6 +197,19 @@ inline void launch_bcast12(hipStream_t stream, long n, const T* x, int sx, int n
         hipLaunchKernelGGL((ew_bias_vec_kernel<T, F, true>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, x, y, s, nv, z, f);
       else
         hipLaunchKernelGGL((ew_bias_vec_kernel<T, F, false>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, y, x, s, nv, z, f);
+      return;
+    }
+  }
+  if (xfull != yfull && n >= 4 * N && n < (1L << 32)) {
+    const T* full = xfull ? x : y;
+    const T* vec = xfull ? y : x;
+    const int s = xfull ? sy : sx, nv = xfull ? ny : nx;
+    if (aligned16(full) && aligned16(z) && s >= 1 && nv >= 1) {
+      const long nvec = n / N, grid = (nvec + kEwBlock - 1) / kEwBlock;
+      if (xfull)
+        hipLaunchKernelGGL((ew_bias_gather_kernel<T, F, true>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, n, full, vec, (unsigned)s, (unsigned)nv, z, f);
+      else
+        hipLaunchKernelGGL((ew_bias_gather_kernel<T, F, false>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, n, full, vec, (unsigned)s, (unsigned)nv, z, f);
       return;
     }
   }

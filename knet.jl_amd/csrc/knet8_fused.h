@@ -40,12 +40,47 @@ __global__ __launch_bounds__(kEwBlock) void bias_act_kernel(long nitems, const T
   }
 }
 
+// Any number of units (1001, 50257): z and y still move in 16-byte accesses over the flat array, the bias entries are fetched one by one with the row
+// carried along; the last m*n % NV elements are done by workgroup 0.
+template <typename T, typename F, bool DROP>
+__global__ __launch_bounds__(kEwBlock) void bias_act_wrap_kernel(long nvec, long count, const T* z, const T* b, unsigned m, T* y, F f) {
+  typedef typename Vec16<T>::type V;
+  constexpr int NV = Vec16<T>::N;
+  const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
+  if (i < nvec) {
+    const long e = i * NV;
+    unsigned r = (unsigned)e % m;
+    const V a = ld_stream(reinterpret_cast<const V*>(z + e));
+    V u, o;
+    if (DROP) u = ld_stream(reinterpret_cast<const V*>(y + e));
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      const T zb = a[k] + b[r];
+      o[k] = f(zb, DROP ? u[k] : T(0));
+      if (++r == m) r = 0;
+    }
+    st_stream(reinterpret_cast<V*>(y + e), o);
+  }
+  if (blockIdx.x == 0) {
+    const long e = nvec * NV + threadIdx.x;
+    if (e < count) {
+      const T zb = z[e] + b[(unsigned)e % m];
+      y[e] = f(zb, DROP ? y[e] : T(0));
+    }
+  }
+}
+
 template <typename T, bool DROP, typename F>
 inline void launch_bias_act(hipStream_t stream, long m, long n, const T* z, const T* b, T* y, F f) {
   if (m <= 0 || n <= 0) return;
   if (m * n >= (1L << 31)) { record_error("bias + activation: 2^31 or more elements; the kernel's 32-bit row arithmetic does not reach that far"); return; }
   constexpr int N = Vec16<T>::N;
   const bool vec = (m % N == 0) && aligned16(z) && aligned16(b) && aligned16(y);
+  if (!vec && aligned16(z) && aligned16(y) && m * n >= 4 * N) {
+    const long nvec = m * n / N, grid = (nvec + kEwBlock - 1) / kEwBlock;
+    hipLaunchKernelGGL((bias_act_wrap_kernel<T, F, DROP>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, m * n, z, b, (unsigned)m, y, f);
+    return;
+  }
   const long nitems = vec ? m * n / N : m * n;
   const long grid = (nitems + kEwBlock - 1) / kEwBlock;
   if (vec)
@@ -171,12 +206,14 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   if (m <= 0) return;
   if (n > 0 && m * n >= (1L << 31)) { record_error("activation gradient + bias gradient: 2^31 or more elements are not supported"); return; }
   constexpr int N = Vec16<T>::N;
-  if (m < kWave && n > 0) {
+  const bool flat16 = (m * n) % N == 0 && aligned16(dy) && aligned16(y) && aligned16(dz);
+  if ((m < kWave || (m % N != 0 && flat16)) && n > 0) {
     // A layer of few units (ten classes): a 256-row tile would idle nearly all its lanes ((2, 4M): 531 us, (10, 839K): 132 us for 100 MB).
-    // Two launches instead: the element gradient over the flat array, then the row sums of dz by the reduction family's kernel for a short
-    // contiguous axis -- one more read of dz, 4/3 of the bytes, same bits for dz and the same kind of fixed-order sum for db.
+    // Two launches instead: the element gradient over the flat array, then the row sums of dz by the reduction family -- one more read of dz,
+    // 4/3 of the bytes, same bits for dz and the same kind of fixed-order sum for db.  Also for a number of units that is not a multiple of the
+    // vector width (1001) when the flat array can still move in 16-byte accesses: the tiled kernel falls back on 4-byte ones there.
     const long count = m * n;
-    const bool v = count % N == 0 && aligned16(dy) && aligned16(y) && aligned16(dz);
+    const bool v = flat16;
     if (v) hipLaunchKernelGGL((actback_flat_kernel<T, F, N>), dim3((unsigned)ceil_div(count / N, 256)), dim3(256), 0, stream, dy, y, count, dz, f);
     else hipLaunchKernelGGL((actback_flat_kernel<T, F, 1>), dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, stream, dy, y, count, dz, f);
     launch_reduce_strided<T, RedSum<T>>(stream, dz, m, n, 1, db);
