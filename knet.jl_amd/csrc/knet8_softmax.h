@@ -945,15 +945,22 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
     if (G >= 1) {
       // lanes per column and elements per lane: cheapest passes over the workgroup's G columns, a pass costing its R slots plus about six slots' worth
       // of reductions and bookkeeping (measured: ten classes are faster as 2 lanes x 8 in four passes than as 4 x 3 in seven)
+      // The stretch is cut to a whole number of passes when that costs less per column than a last pass with idle teams.
       int bestR = 8, bestTL = kWave;
-      long best = -1;
+      long bestG = G;
+      double best = -1;
       for (int R : {8, 6, 4, 3, 2}) {
         int TL = 1;
         while (TL < kWave && (long)TL * R < m) TL <<= 1;
         if ((long)TL * R < m) continue;
-        const long slots = ((G + 256 / TL - 1) / (256 / TL)) * (R + 6);
-        if (best < 0 || slots < best) { best = slots; bestR = R; bestTL = TL; }
+        const long nteams = 256 / TL;
+        for (long Gc : {G, G / nteams * nteams}) {     // nteams is a power of two of at least 4: Gc stays a multiple of `step`
+          if (Gc < 1) continue;
+          const double cost = (double)(((Gc + nteams - 1) / nteams) * (R + 6)) / (double)Gc;
+          if (best < 0 || cost < best) { best = cost; bestR = R; bestTL = TL; bestG = Gc; }
+        }
       }
+      G = bestG;
       const dim3 grid((unsigned)((n + G - 1) / G));
 #define KNET8_SHORT(VEC, R) hipLaunchKernelGGL((softmax_short_kernel<T, Algo, VEC, R>), grid, dim3(256), 0, stream, (int)m, n, (int)G, bestTL, a, b, out, labels, scale, loss)
       if (v16) {
