@@ -377,6 +377,65 @@ def summarize_profile(root):
                 print("traffic reluback_32_11 %d   (bytes per launch: fetch + write above)" % int((fm + wm) * (1 << 20)))
 
 
+def shape_scan(torch, K):
+    """Kernels of the gradient path on shapes away from the benchmark's: reductions over every kind of (rows, columns) split of a 134 MB array,
+    the softmax family on short and medium columns, the bias kernels on odd and small unit counts.  Cold figures (rotating buffers), same method as
+    the config-3/4 table; prints one text line per shape: microseconds / fraction of the 8 TB/s HBM peak for the algorithmic bytes."""
+    f32 = torch.float32
+
+    def line(label, cells):
+        print(label + "  " + "  ".join("%s %.1f/%.3f" % (n, r["cold"]["us"], r["cold"]["frac_of_peak"]) for n, r in cells), flush=True)
+
+    total = 32 << 20
+    nsets = 10
+    xs = [device_randn(torch, K, total, f32, 50 + i) for i in range(nsets)]
+    out = xs[0].similar((total,))
+    sets = list(range(nsets))
+    time_kernel(K, torch, lambda i: (lambda: K.knet8("sum_32_21", total, xs[i].ptr, 4096, total // 4096, out.ptr)), 4 * total, sets, reps=16)  # the first figures of a process read low
+    print("== sum_32_21 over a (rows, columns) fp32 matrix of 2^25 elements: dims=1 (runs of `rows`), dims=2 (contiguous axis of `rows`)")
+    for rows in (2, 8, 10, 32, 100, 256, 1000, 4096, 10000, 32768, 100000, 1 << 20):
+        cols = total // rows
+        n = rows * cols
+        cells = []
+        for dims, sy, ny in ((1, rows, cols), (2, 1, rows)):
+            cells.append(("dims=%d" % dims, time_kernel(K, torch, lambda i: (lambda: K.knet8("sum_32_21", n, xs[i].ptr, sy, ny, out.ptr)), 4 * (n + ny), sets, reps=16)))
+        line("(%8d,%8d)" % (rows, cols), cells)
+    print("== sum_32_21 over dims (1,3) of x(a, b, c), 2^25 elements")
+    for a, b in ((56 * 56, 256), (64, 1024), (7 * 7, 2048), (16, 16), (4, 1000)):
+        c = total // (a * b)
+        n = a * b * c
+        line("(%d,%d,%d)" % (a, b, c), [("", time_kernel(K, torch, lambda i: (lambda: K.knet8("sum_32_21", n, xs[i].ptr, a, b, out.ptr)), 4 * (n + b), sets, reps=16))])
+    del xs, out
+    total = 8 << 20
+    nsets = 12
+    sets = list(range(nsets))
+    xs = [device_randn(torch, K, total, f32, 50 + i, scale=2.0) for i in range(nsets)]
+    dys = [device_randn(torch, K, total, f32, 90 + i) for i in range(nsets)]
+    ys = [x.similar() for x in xs[:4]]
+    print("== softmax family down the columns of a (rows, columns) fp32 matrix of 2^23 elements")
+    for C in (2, 10, 21, 32, 100, 128, 256, 1000, 2000, 4000, 8000, 16000):
+        N = total // C
+        n = C * N
+        labels = K.KnetArray(np.random.default_rng(0).integers(1, C + 1, size=N).astype(np.int32))
+        loss = xs[0].similar((N,))
+        scale = ctypes.c_float(1.0 / N)
+        cells = [("logsoftmax", time_kernel(K, torch, lambda i: (lambda: K.knet8("logsoftmax_32", C, N, xs[i].ptr, ys[i % 4].ptr)), 8 * n, sets, reps=16)),
+                 ("logsoftmaxback", time_kernel(K, torch, lambda i: (lambda: K.knet8("logsoftmaxback_32", C, N, xs[i].ptr, dys[i].ptr, ys[i % 4].ptr)), 12 * n, sets, reps=16)),
+                 ("nll", time_kernel(K, torch, lambda i: (lambda: K.knet8("nll_logsoftmax_back_32", C, N, xs[i].ptr, labels.ptr, scale, ys[i % 4].ptr, loss.ptr)), 8 * n + 8 * N, sets, reps=16))]
+        line("(%6d,%8d)" % (C, N), cells)
+    print("== bias kernels on an (m, n) fp32 matrix of 2^23 elements: z .+ b, relu.(z .+ b), reluback + bias gradient")
+    bias = device_randn(torch, K, total, f32, 229)
+    db = bias.similar()
+    for m in (2, 10, 64, 1000, 1001, 4096, 100000):
+        n = total // m
+        t = m * n
+        cells = [("add_32_12", time_kernel(K, torch, lambda i: (lambda: K.knet8("add_32_12", t, dys[i].ptr, 1, t, bias.ptr, 1, m, ys[i % 4].ptr)), 8 * t + 4 * m, sets, reps=16)),
+                 ("biasrelu_32", time_kernel(K, torch, lambda i: (lambda: K.knet8("biasrelu_32", m, n, dys[i].ptr, bias.ptr, ys[i % 4].ptr)), 8 * t + 4 * m, sets, reps=16)),
+                 ("reluback_biasgrad_32", time_kernel(K, torch, lambda i: (lambda: K.knet8("reluback_biasgrad_32", m, n, dys[i].ptr, xs[i].ptr, ys[i % 4].ptr, db.ptr)), 12 * t + 4 * m, sets, reps=16))]
+        line("(%7d,%7d)" % (m, n), cells)
+    K.libknet8().check()
+
+
 def mlp_steps(torch, K, sizes, batch, pdrop, steps, fused, graph=False, layers=False, head=False):
     """Forward + backward of an MLP through KnetArray and the tape.  graph=True: the step is captured once into a hipGraph
     (labels resident on the device, loss kept on the device) and `steps` replays are timed.  layers=True: each hidden layer's
@@ -579,6 +638,7 @@ def main():
                          "rotating over more than 1 GB) and exit: the workload of the rocprofv3 runs" % PROFILE_REPS)
     ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default <tmp>/knet8_profile/<mode>_plan.json)")
     ap.add_argument("--summarize-profile", metavar="DIR", default=None, help="print the text summary of the rocprofv3 output under DIR and exit (no GPU needed)")
+    ap.add_argument("--scan", action="store_true", help="time the gradient-path kernels on shapes away from the benchmark's (text table) and exit")
     ap.add_argument("--timeline", action="store_true",
                     help="compile tests/c_host/kernel_timeline.hip with hipcc and run it: per-workgroup start / loads-arrived / end stamps of the "
                          "launch shapes behind the config 3-4 rows, next to a one-shot elementwise launch and an empty kernel")
@@ -608,6 +668,9 @@ def main():
     # (src/libknet8/LibKnet8.jl:50-55), not to the legacy null stream (which has to order itself against every other stream of the process).
     if not os.environ.get("KNET8_BENCH_NULL_STREAM"):
         K.libknet8().stream = K.libknet8().fn["knet8_stream_create"]()
+    if args.scan:
+        shape_scan(torch, K)
+        return
     if args.profile_pass:
         plan_path = args.plan_out or os.path.join(tempfile.gettempdir(), "knet8_profile", args.profile_pass + "_plan.json")
         os.makedirs(os.path.dirname(plan_path), exist_ok=True)
