@@ -169,7 +169,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
     if (!last_block_ticket(counters + at * kTicketStride, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = T(0);
-    strided_walk<T, RedSum<T>, NV, false, NW, U, SC>(partial + at * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
+    strided_walk<T, RedSum<T>, NV, false, NW, kCombineU, SC>(partial + at * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
     if (threadIdx.x == 0) st_coherent(counters + at * kTicketStride, 0u);
   }
 #pragma unroll

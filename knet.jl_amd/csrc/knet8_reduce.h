@@ -157,6 +157,10 @@ __device__ __forceinline__ void strided_walk(const T* base, long stride, long k0
   }
 }
 
+// Rows of partial results a wave of the combining workgroup has in flight at once: with many parts (a tile split 256 ways is 16 rows per wave) two
+// rows at a time are eight memory round trips in a row.
+constexpr int kCombineU = 8;
+
 template <typename T, typename Op, int NV, int BT, int U, bool SC = false>
 __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
                                                                    unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
     if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) return;
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
-    strided_walk<T, Op, NV, false, NW, U, SC>(partial + group * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
+    strided_walk<T, Op, NV, false, NW, kCombineU, SC>(partial + group * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
     if (threadIdx.x == 0) st_coherent(counters + group * kTicketStride, 0u);
   }
 #pragma unroll
