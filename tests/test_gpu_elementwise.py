@@ -169,6 +169,24 @@ def test_bias_add_broadcast_and_unbroadcast(knet, oracle):
         knet.add(knet.KnetArray(np.zeros((3, 4), np.float32)), knet.KnetArray(np.zeros((4, 3), np.float32)))
 
 
+def test_vector_broadcasts_of_any_length_and_stride(knet):
+    """`F_S_12` with a vector whose length or stride is not a multiple of the 16-byte vector width, and totals that are not either: the full-size
+    operand moves in 16-byte accesses over the flat array, the vector entries are gathered.  Both operand orders of the non-commutative operators,
+    both widths; one rounded operation per element, so the bits are numpy's."""
+    rng = np.random.default_rng(19)
+    ops = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "div": np.divide}
+    for dt in (np.float32, np.float64):
+        for shape, bshape in [((1001, 37), (1001, 1)), ((1001, 37), (1, 37)), ((10, 333), (10, 1)), ((3, 5, 7), (1, 5, 1)), ((7, 3, 11), (1, 1, 11)),
+                              ((2, 50001), (2, 1)), ((50257, 3), (50257, 1)), ((17, 19), (1, 19)), ((5, 4), (5, 1))]:
+            x = (rng.standard_normal(shape) + 3).astype(dt)
+            b = (rng.standard_normal(bshape) + 3).astype(dt)
+            xd, bd = knet.KnetArray(x), knet.KnetArray(b)
+            for name, f in ops.items():
+                assert bits_equal(knet.Array(knet.broadcast_op(name, xd, bd)), f(x, b)), (name, shape, bshape, "x.b")
+                assert bits_equal(knet.Array(knet.broadcast_op(name, bd, xd)), f(b, x)), (name, shape, bshape, "b.x")
+    knet.libknet8().check()
+
+
 def test_error_behaviour(knet):
     a = knet.KnetArray(np.zeros(4, np.float32))
     b = knet.KnetArray(np.zeros(5, np.float32))
