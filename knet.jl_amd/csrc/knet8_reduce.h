@@ -224,12 +224,12 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
 // q < U, and sums them over the stretches of its part, `iter_stride` elements apart; which output an element belongs to depends on its place in
 // the stretch only: (i / sy) % g.  At the end the accumulators go to LDS and a team of TL lanes reduces the R*sy entries of each output.
 // P workgroups split the iterations of a group; the last to finish combines their g-vectors in fixed order.
-template <typename T, typename Op, int NV, int U>
+// O: stretches in flight per lane (1 for a launch whose workgroups have a single stretch each: the registers go to a longer stretch, U, instead).
+template <typename T, typename Op, int NV, int U, int O>
 __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __restrict__ x, int sy, int g_full, long nout, int R, int TL, long group_stride,
                                                                   long iter_stride, long iters, long iters_per_part, long limit, unsigned P,
                                                                   T* __restrict__ y, T* partial, unsigned* counters) {
   constexpr int CAP = kRedBlock * U * NV;
-  constexpr int O = 4;   // stretches in flight per lane
   __shared__ T lds[CAP + CAP / 32];
   __shared__ unsigned flag;
   const long group = blockIdx.x / P;
@@ -255,11 +255,14 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
       for (int q = 0; q < U; q++) {
         const int i = ((int)threadIdx.x + q * kRedBlock) * NV;
         if (t + o < t1 && i < E && at + i < limit) {
-          if (NV > 1) {
+          if (NV > 1 && i + NV <= E && at + i + NV <= limit) {
             typedef typename Vec16<T>::type V;
             const V w = ld_stream(reinterpret_cast<const V*>(base + at + i));
 #pragma unroll
-            for (int e = 0; e < NV; e++) v[o][q][e] = (i + e < E && at + i + e < limit) ? Op::item(w[e]) : Op::init();
+            for (int e = 0; e < NV; e++) v[o][q][e] = Op::item(w[e]);
+          } else if (NV > 1) {   // the last vector of a stretch that does not end on a vector boundary: element by element, nothing past the end is touched
+#pragma unroll
+            for (int e = 0; e < NV; e++) v[o][q][e] = (i + e < E && at + i + e < limit) ? Op::item(__builtin_nontemporal_load(base + at + i + e)) : Op::init();
           } else {
             v[o][q][0] = Op::item(__builtin_nontemporal_load(base + at + i));
           }
@@ -293,7 +296,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
     T r = Op::init();
     if (jl < g)
       for (int c = tl; c < entries; c += TL) {
-        const int i = ((c / sy) * g + jl) * sy + c % sy;
+        const int i = R == 1 ? jl * sy + c : ((c / sy) * g + jl) * sy + c % sy;   // (one slab per stretch: no division per entry)
         r = Op::merge(r, lds[i + (i >> 5)]);
       }
     for (int o = TL >> 1; o > 0; o >>= 1) r = Op::merge(r, __shfl_xor(r, o));
@@ -355,7 +358,7 @@ inline unsigned plan_parts(long groups, long units_per_group, long min_units_per
   return (unsigned)P;
 }
 
-constexpr long kStretchMaxRun = 128;   // longest run the stretch kernel takes
+constexpr long kStretchMaxRun = 1024;   // longest run the stretch kernel takes
 
 // Stretch kernel for x(sy, ny, no) -> y(ny) per batch (nb batches, `batch_stride` elements apart, outputs ny apart); sy*ny small enough for
 // whole slabs (R >= 1 of them per stretch) or sy <= kStretchMaxRun.  Returns false if the shape is not one for it.
@@ -363,7 +366,8 @@ template <typename T, typename Op>
 inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long ny, long no, long nb, long batch_stride, T* y,
                                   const ScratchSource* scratch) {
   constexpr int N = Vec16<T>::N;
-  constexpr int U1 = 4, UV = 2;
+  constexpr int U1 = 4, UV = 2;      // accesses per lane and stretch, scalar and vector kernels
+  constexpr int S1 = 16, SV = 4;     // the same for launches of one stretch per workgroup (one slab of short runs)
   const long slab = sy * ny;
   if (sy > kStretchMaxRun || slab <= 0 || no <= 0) return false;
   const bool whole = slab <= kRedBlock * U1 / 2;          // whole slabs, several per stretch (the scalar kernel's capacity decides: it must hold for both)
@@ -372,6 +376,7 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   // 16-byte loads: every stretch must start on a 16-byte boundary and no vector may reach past the end of the array
   bool vec = aligned16(x) && (nb == 1 || batch_stride % N == 0);
   int g, R;
+  bool single = false;
   long groups, group_stride, iter_stride, iters, limit;
   if (whole) {
     vec = vec && (no * slab) % N == 0;
@@ -383,8 +388,9 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
     if (R < 1) return false;
     groups = nb; group_stride = batch_stride; iter_stride = R * slab; iters = ceil_div(no, R); limit = no * slab;
   } else {
-    vec = vec && slab % N == 0;
-    const int cap = kRedBlock * (vec ? UV * N : U1);
+    single = no == 1;
+    vec = vec && (single || slab % N == 0);   // one slab: only the groups have to start on 16-byte boundaries (a last vector that would reach past the group is read element by element)
+    const int cap = single ? kRedBlock * (vec ? SV * N : S1) : kRedBlock * (vec ? UV * N : U1);
     long G = cap / sy;
     if (vec) { const long step = N / gcd(N, sy); G = G / step * step; }   // groups start on 16-byte boundaries
     if (G < 1) return false;
@@ -411,12 +417,12 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
     if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return true;
   }
   const dim3 grid((unsigned)(groups * P));
-  if (vec)
-    hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, N, UV>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride,
-                       iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters);
-  else
-    hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, 1, U1>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride,
-                       iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters);
+#define KNET8_STRETCH(NV, U, O) \
+  hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, NV, U, O>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride, \
+                     iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters)
+  if (single) { if (vec) KNET8_STRETCH(N, SV, 1); else KNET8_STRETCH(1, S1, 1); }
+  else        { if (vec) KNET8_STRETCH(N, UV, 4); else KNET8_STRETCH(1, U1, 4); }
+#undef KNET8_STRETCH
   return true;
 }
 
@@ -439,7 +445,11 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
     launch_reduce_run<T, typename Op::Merged>(stream, tmp, sy, ny, 1, y, scratch);
     return;
   }
-  if (ny > 1 && (sy <= 8 || (no == 1 && sy <= kStretchMaxRun)) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
+  // (one slab: up to 256-element runs, measured against the run kernel below -- 129: 39 against 195 us, 256: 29.6 / 30.8, 384: 34 / 21.6 --, and up to
+  //  1024 when the runs do not start on 16-byte boundaries, where the run kernel is down to 4-byte loads: 513: 39 against 56 us)
+  constexpr int NR = Vec16<T>::N;
+  const bool short_one_slab = no == 1 && (sy <= 256 || (sy <= kStretchMaxRun && (sy % NR != 0 || !aligned16(x))));
+  if (ny > 1 && (sy <= 8 || short_one_slab) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;

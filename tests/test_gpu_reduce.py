@@ -92,14 +92,15 @@ def test_raw_21_and_22_entry_points_on_odd_shapes_and_misaligned_views(knet, ora
 
 
 def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
-    """Shapes that go to the stretch kernel: runs of at most 128 elements with one slab, runs of at most 8 with many, a contiguous axis shorter than
+    """Shapes that go to the stretch kernel: runs of at most 256 elements with one slab (1024 when they do not start on 16-byte boundaries), runs of at most 8 with many, a contiguous axis shorter than
     a wave.  Groups with a tail, whole slabs with a last partial stretch, sizes that are and are not multiples of a 16-byte vector, batches, split
     launches (enough stretches for several parts), base pointers off the 16-byte grid; every operator, exact on integer-valued data."""
     from gpu_util import misaligned
     rng = np.random.default_rng(26)
     for dt, S in ((np.float32, "32"), (np.float64, "64")):
         runs = [(2, 100001, 1), (8, 4096, 1), (10, 100000, 1), (128, 777, 1), (3, 5, 1), (100, 3355, 1), (127, 40, 1), (64, 2049, 1),
-                (4, 1000, 50), (8, 3, 1000), (2, 2, 100000), (7, 5, 333), (1, 3, 70000), (5, 600, 41), (8, 1, 5), (6, 100000, 3)]
+                (4, 1000, 50), (8, 3, 1000), (2, 2, 100000), (7, 5, 333), (1, 3, 70000), (5, 600, 41), (8, 1, 5), (6, 100000, 3),
+                (129, 300, 1), (256, 100, 1), (257, 101, 1), (513, 50, 1), (1001, 21, 1), (1023, 9, 1), (1024, 9, 1)]
         for (sy, ny, no) in runs:
             x = rng.integers(-4, 5, size=(sy, ny, no)).astype(dt)
             x[x == 0] = 1 if x.size < 2000 else 0
