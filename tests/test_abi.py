@@ -57,6 +57,32 @@ def test_every_symbol_of_the_reference_library_is_exported(built_lib):
     assert not [n for n in names if not hasattr(lib, n)]
 
 
+def test_every_signature_matches_the_reference_generators():
+    """tests/golden/libknet8_signatures.txt holds, for each of the reference's entry points, the return type and parameter types its generator
+    script prints (src/libknet8/cuda01.jl:20-25, cuda1.jl:28-33,63-68,95-100,127-132,157-162,188-200,371-442,482-493,519-524, cuda11.jl:22-27,
+    cuda111.jl:23-28, cuda12.jl:28-33, cuda13.jl:99-111,172-184, cuda16.jl:60-83, cuda17.jl:58-63, cuda20.jl:83-104, cuda21.jl:70-76,
+    cuda22.jl:61-66, relu.jl:27-38; read as text by tests/golden/make_libknet8_symbols.py).  The header must declare each with the same types in
+    the same order, `cudaStream_t` read as `hipStream_t`: a swapped, missing or extra parameter anywhere in the boundary fails here."""
+    lk = _load("lk_for_sig", "knet.jl_amd/libknet8.py")
+    decls = lk.parse_header()
+    names = open(os.path.join(ROOT, "tests", "golden", "libknet8_symbols.txt")).read().split()
+    rows = [l.rstrip("\n").split("\t") for l in open(os.path.join(ROOT, "tests", "golden", "libknet8_signatures.txt"))]
+    assert [r[0] for r in rows] == names          # one signature per exported symbol
+    bad = []
+    for name, ret, params in rows:
+        want = [p.replace("cudaStream_t", "hipStream_t") for p in params.split(",")] if params else []
+        have_ret, have = decls[name]
+        if have_ret != ret or have != want:
+            bad.append((name, ret, want, have_ret, have))
+    assert not bad, bad[:5]
+    # the fixture itself distinguishes the shapes an order slip would confuse
+    sig = {r[0]: r[2].split(",") for r in rows}
+    assert sig["sum_32_22"] == ["int", "int", "float*", "int", "int", "int", "float*"]
+    assert sig["setcol1_64_stream"] == ["int", "int", "int", "int*", "double*", "double", "cudaStream_t"]
+    assert sig["add_32_16_5"] == ["float*"] * 3 + ["int"] * 16
+    assert sig["xcopy_stream"] == ["int", "int", "const void*", "int", "void*", "int", "cudaStream_t"]
+
+
 def _split_top(text):
     """Split at top-level commas (parentheses, braces and brackets nest; string literals are skipped)."""
     parts, depth, cur, q = [], 0, "", False
