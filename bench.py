@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the backward-pass gradient kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--all]
 
 A "step" is one pass of the isolated unary gradients of benchmark config 2: reluback, sigmback, tanhback,
 eluback, seluback on 2^28-element fp32 vectors and on 2^27-element fp64 vectors (ten launches, 3.22 GB of
@@ -12,10 +12,13 @@ a fixed seed, y = f(x) from the library's forward kernels) and resident in HBM b
 The same JSON line carries
   roofline      -- reluback_32_11, the kernel every config-2 launch shares its template with: algorithmic bytes per
                    launch / mean launch duration measured with HIP events around each launch inside the timed region;
+                   roofline.rows: every kernel of configs 3-5 at its full shape as [cold fraction of 8 TB/s, warm fraction,
+                   fraction of the one-shot yardstick, cold us, yardstick us] (warm = back-to-back on the same buffers,
+                   cold = rotating over > 1 GB of distinct buffers so the 256 MB Infinity Cache cannot serve the reads);
   cpu_baseline  -- the C restatement of Knet's CPU Array path (oracle/) timed on one host core on a bounded sample;
-  kernels       -- per-kernel GB/s for configs 2-4 (warm = back-to-back on the same buffers, cold = rotating over
-                   > 1 GB of distinct buffers so the 256 MB Infinity Cache cannot serve the reads);
-  mlp           -- backward steps/sec of configs 1 and 5 through KnetArray and the tape.
+  kernels_config2, mlp_steps_per_sec (configs 1 and 5 through KnetArray and the tape, and from C hosts; the short
+                   keys are spelled out in MLP_LEGEND below and by --all), cpu_oracle_GBps_1_thread.
+Other modes print text for profiles/: --profile-pass / --summarize-profile (rocprofv3), --timeline, --two-streams, --scan.
 """
 import argparse
 import ctypes
@@ -203,26 +206,35 @@ def neighbours(torch, K):
 
 
 def kernel_cases(torch, K, widths=("32", "64")):
-    """The kernels of benchmark configs 3, 4 and 5 at their full shapes: yields (label, algorithmic bytes per launch, number of buffer sets,
-    make_launch) where make_launch(i) returns a function that launches the kernel on buffer set i.  Enough sets that one round over them
-    exceeds 1 GB.  fp32 is the configs' own width; the fp64 rows are the same kernels at the reference's other element type."""
+    """The kernels of benchmark configs 3, 4 and 5 at their full shapes: yields (key, label, algorithmic bytes per launch, number of buffer
+    sets, make_launch, yardstick key) where make_launch(i) returns a function that launches the kernel on buffer set i.  Enough sets that one
+    round over them exceeds 1 GB.  fp32 is the configs' own width; the fp64 rows are the same kernels at the reference's other element type.
+    A yardstick ("y_..." keys) is a plain one-shot elementwise kernel of the library moving the same number of bytes over the same buffers --
+    what this chip delivers to any kernel of that size, launch ramp and drain included: reluback_S_11 (2R+1W) for the three-stream kernels,
+    relu_S (1R+1W) for the two-stream ones and, over half as many elements (same bytes in total), for the reductions, which only read."""
     for S in widths:
         dt, sz = (torch.float32, 4) if S == "32" else (torch.float64, 8)
+        sfx = "" if S == "32" else "_f64"
         # config 3: unbroadcast reductions
         nsets = 10 if S == "32" else 5
-        mats = [device_randn(torch, K, 4096 * 8192, dt, 10 + i, dims=(4096, 8192)) for i in range(nsets)]
+        nmat = 4096 * 8192
+        mats = [device_randn(torch, K, nmat, dt, 10 + i, dims=(4096, 8192)) for i in range(nsets)]
         for d, ny in ((1, 8192), (2, 4096)):
             outs = [m.similar((ny,)) for m in mats]
             sy = 4096 if d == 1 else 1
-            yield ("sum_%s_21 (4096,8192) dims=%d" % (S, d), sz * (4096 * 8192 + ny), nsets,
-                   lambda i, sy=sy, ny=ny, outs=outs: (lambda: K.knet8("sum_%s_21" % S, 4096 * 8192, mats[i].ptr, sy, ny, outs[i].ptr)))
+            yield ("sum21_d%d%s" % (d, sfx), "sum_%s_21 (4096,8192) dims=%d" % (S, d), sz * (nmat + ny), nsets,
+                   lambda i, sy=sy, ny=ny, outs=outs: (lambda: K.knet8("sum_%s_21" % S, nmat, mats[i].ptr, sy, ny, outs[i].ptr)), "y_sum21_mat" + sfx)
+        yield ("y_sum21_mat" + sfx, "yardstick relu_%s n=%d (1R+1W inside one (4096,8192) matrix: the bytes of its sums)" % (S, nmat // 2), sz * nmat, nsets,
+               lambda i: (lambda: K.knet8("relu_%s" % S, nmat // 2, mats[i].ptr, mats[i].ptr + sz * (nmat // 2))), None)
         del mats, outs
         nn = 56 * 56 * 256 * 64
         nsets = 6 if S == "32" else 4
         mats = [device_randn(torch, K, nn, dt, 30 + i) for i in range(nsets)]
         outs = [m.similar((256,)) for m in mats]
-        yield ("sum_%s_21 NCHW (56,56,256,64)->(1,1,256,1)" % S, sz * (nn + 256), nsets,
-               lambda i: (lambda: K.knet8("sum_%s_21" % S, nn, mats[i].ptr, 3136, 256, outs[i].ptr)))
+        yield ("sum21_nchw" + sfx, "sum_%s_21 NCHW (56,56,256,64)->(1,1,256,1)" % S, sz * (nn + 256), nsets,
+               lambda i: (lambda: K.knet8("sum_%s_21" % S, nn, mats[i].ptr, 3136, 256, outs[i].ptr)), "y_sum21_nchw" + sfx)
+        yield ("y_sum21_nchw" + sfx, "yardstick relu_%s n=%d (1R+1W inside one NCHW array: the bytes of its sum)" % (S, nn // 2), sz * nn, nsets,
+               lambda i: (lambda: K.knet8("relu_%s" % S, nn // 2, mats[i].ptr, mats[i].ptr + sz * (nn // 2))), None)
         del mats, outs
         # config 4: logsoftmax backward and fused nll backward
         for C, N in ((32000, 512), (1000, 4096)):
@@ -233,17 +245,14 @@ def kernel_cases(torch, K, widths=("32", "64")):
             labels = K.KnetArray(np.random.default_rng(0).integers(1, C + 1, size=N).astype(np.int32))
             loss = ys[0].similar((N,))
             scale = (ctypes.c_float if S == "32" else ctypes.c_double)(1.0 / N)
-            yield ("logsoftmaxback_%s (%d,%d)" % (S, C, N), 3 * sz * C * N, nsets,
-                   lambda i: (lambda: K.knet8("logsoftmaxback_%s" % S, C, N, ys[i].ptr, dys[i].ptr, dxs[i].ptr)))
-            yield ("nll_logsoftmax_back_%s (%d,%d)" % (S, C, N), 2 * sz * C * N + sz * N, nsets,
-                   lambda i: (lambda: K.knet8("nll_logsoftmax_back_%s" % S, C, N, ys[i].ptr, labels.ptr, scale, dxs[i].ptr, loss.ptr)))
-            if S == "32":
-                # yardsticks: plain elementwise kernels moving the same bytes over the same buffers -- what this chip delivers to
-                # any kernel of this size, launch ramp and drain included
-                yield ("yardstick reluback_32_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (C * N, C, N), 12 * C * N, nsets,
-                       lambda i: (lambda: K.knet8("reluback_32_11", C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)))
-                yield ("yardstick relu_32 n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (C * N, C, N), 8 * C * N, nsets,
-                       lambda i: (lambda: K.knet8("relu_32", C * N, ys[i].ptr, dxs[i].ptr)))
+            yield ("lsmback_%d%s" % (C, sfx), "logsoftmaxback_%s (%d,%d)" % (S, C, N), 3 * sz * C * N, nsets,
+                   lambda i: (lambda: K.knet8("logsoftmaxback_%s" % S, C, N, ys[i].ptr, dys[i].ptr, dxs[i].ptr)), "y_3s_%d%s" % (C, sfx))
+            yield ("nll_%d%s" % (C, sfx), "nll_logsoftmax_back_%s (%d,%d)" % (S, C, N), 2 * sz * C * N + sz * N, nsets,
+                   lambda i: (lambda: K.knet8("nll_logsoftmax_back_%s" % S, C, N, ys[i].ptr, labels.ptr, scale, dxs[i].ptr, loss.ptr)), "y_2s_%d%s" % (C, sfx))
+            yield ("y_3s_%d%s" % (C, sfx), "yardstick reluback_%s_11 n=%d (2R+1W, the bytes of logsoftmaxback (%d,%d))" % (S, C * N, C, N), 3 * sz * C * N, nsets,
+                   lambda i: (lambda: K.knet8("reluback_%s_11" % S, C * N, dys[i].ptr, ys[i].ptr, dxs[i].ptr)), None)
+            yield ("y_2s_%d%s" % (C, sfx), "yardstick relu_%s n=%d (1R+1W, the bytes of nll_logsoftmax_back (%d,%d))" % (S, C * N, C, N), 2 * sz * C * N, nsets,
+                   lambda i: (lambda: K.knet8("relu_%s" % S, C * N, ys[i].ptr, dxs[i].ptr)), None)
             del ys, dys, dxs
     # config 5 per-layer kernels (fp32): dropback, then the fused layer passes: bias + relu + dropout forward (z, u -> y) and
     # dropback + reluback + bias gradient (dy, y -> dz, db)
@@ -253,23 +262,42 @@ def kernel_cases(torch, K, widths=("32", "64")):
     dys = [device_randn(torch, K, n5, f32, 180 + i) for i in range(40)]
     dxs = [y.similar() for y in ys[:4]]
     half = ctypes.c_float(0.5)
-    yield ("dropback_32 (4096,2048)", 12 * n5, 40,
-           lambda i: (lambda: K.knet8("dropback_32", n5, half, ys[i].ptr, ys[i].ptr, dys[i].ptr, dxs[i % 4].ptr)))
+    yield ("dropback", "dropback_32 (4096,2048)", 12 * n5, 40,
+           lambda i: (lambda: K.knet8("dropback_32", n5, half, ys[i].ptr, ys[i].ptr, dys[i].ptr, dxs[i % 4].ptr)), "y_3s_cfg5")
     us = [device_randn(torch, K, n5, f32, 230 + i) for i in range(4)]
     bias = device_randn(torch, K, 4096, f32, 229)
     db = bias.similar()
-    yield ("biasreludrop_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
-           lambda i: (lambda: K.knet8("biasreludrop_32", 4096, 2048, half, dys[i].ptr, bias.ptr, us[i % 4].ptr)))
-    yield ("dropreluback_biasgrad_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
-           lambda i: (lambda: K.knet8("dropreluback_biasgrad_32", 4096, 2048, half, dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr, db.ptr)))
+    yield ("biasreludrop", "biasreludrop_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
+           lambda i: (lambda: K.knet8("biasreludrop_32", 4096, 2048, half, dys[i].ptr, bias.ptr, us[i % 4].ptr)), "y_3s_cfg5")
+    yield ("dropreluback_biasgrad", "dropreluback_biasgrad_32 (4096,2048)", 12 * n5 + 4 * 4096, 40,
+           lambda i: (lambda: K.knet8("dropreluback_biasgrad_32", 4096, 2048, half, dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr, db.ptr)), "y_3s_cfg5")
+    yield ("y_3s_cfg5", "yardstick reluback_32_11 n=%d (2R+1W, the bytes of the config-5 layer passes)" % n5, 12 * n5, 40,
+           lambda i: (lambda: K.knet8("reluback_32_11", n5, dys[i].ptr, ys[i].ptr, dxs[i % 4].ptr)), None)
 
 
 def extras(torch, K):
+    """{key: (label, yardstick key, {"warm": ..., "cold": ...})} for every row of kernel_cases."""
     res = {}
-    for label, nbytes, nsets, make_launch in kernel_cases(torch, K):
-        res[label] = time_kernel(K, torch, make_launch, nbytes, list(range(nsets)))
+    for key, label, nbytes, nsets, make_launch, yard in kernel_cases(torch, K):
+        res[key] = (label, yard, time_kernel(K, torch, make_launch, nbytes, list(range(nsets))))
         K.libknet8().check()
     return res
+
+
+ROWS_LEGEND = ("per kernel of configs 3-5 at full shape: [cold fraction of 8 TB/s, warm fraction, cold time of the one-shot elementwise yardstick moving the "
+               "same bytes over the same buffers / cold time of the kernel, cold us per launch, yardstick cold us per launch]; cold = rotating over more "
+               "than 1 GB of buffers, warm = one buffer set; algorithmic bytes / mean of 24 back-to-back launches (HIP events on the launch stream)")
+
+
+def roofline_rows(ex):
+    rows = {}
+    for key, (label, yard, r) in ex.items():
+        if key.startswith("y_"):
+            continue
+        yu = ex[yard][2]["cold"]["us"] if yard in ex else None
+        rows[key] = [round(r["cold"]["frac_of_peak"], 3), round(r["warm"]["frac_of_peak"], 3), round(yu / r["cold"]["us"], 3) if yu else None,
+                     round(r["cold"]["us"], 2), round(yu, 2) if yu else None]
+    return rows
 
 
 PROFILE_REPS = 24
@@ -286,12 +314,14 @@ def profile_pass(torch, K, mode, plan_path):
     x = device_randn(torch, K, n, f32, 1)
     dy = device_randn(torch, K, n, f32, 2)
     dx = x.similar()
-    for _ in range(PROFILE_REPS):
+    # Every group is PROFILE_REPS + 1 launches: the first one (the kernel's first dispatch in the process, on operands no kernel of this
+    # shape has walked yet) is listed apart by the summary and left out of its averages, as the bench leaves its warm-up launches out.
+    for _ in range(PROFILE_REPS + 1):
         K.knet8("copy_32", n, x.ptr, dx.ptr)
     plan.append(["copy_32 n=2^28 (1 GiB read + 1 GiB written: the yardstick of the byte counters)", 8 * n, PROFILE_REPS])
     for back, fwd in OPS:
         y = K.unary_op(fwd, x)
-        for _ in range(PROFILE_REPS):
+        for _ in range(PROFILE_REPS + 1):
             K.knet8("%s_32_11" % back, n, dy.ptr, y.ptr, dx.ptr)
         plan.append(["%s_32_11 n=2^28" % back, 12 * n, PROFILE_REPS])
         del y
@@ -301,7 +331,7 @@ def profile_pass(torch, K, mode, plan_path):
     dxd = xd.similar()
     for back, fwd in OPS:
         yd = K.unary_op(fwd, xd)
-        for _ in range(PROFILE_REPS):
+        for _ in range(PROFILE_REPS + 1):
             K.knet8("%s_64_11" % back, 1 << 27, dyd.ptr, yd.ptr, dxd.ptr)
         plan.append(["%s_64_11 n=2^27" % back, 24 << 27, PROFILE_REPS])
         del yd
@@ -309,9 +339,9 @@ def profile_pass(torch, K, mode, plan_path):
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
     K.libknet8().fn["knet8_trim"]()
-    for label, nbytes, nsets, make_launch in kernel_cases(torch, K):
+    for key, label, nbytes, nsets, make_launch, yard in kernel_cases(torch, K):
         launches = [make_launch(i) for i in (range(nsets) if mode == "cold" else range(1))]
-        for r in range(PROFILE_REPS):
+        for r in range(PROFILE_REPS + 1):
             launches[r % len(launches)]()
         plan.append(["%s [%s]" % (label, mode), nbytes, PROFILE_REPS])
         torch.cuda.synchronize()
@@ -351,9 +381,13 @@ def summarize_profile(root):
         for which, cname in (("fetch", "FETCH_SIZE"), ("write", "WRITE_SIZE")):
             pc = glob.glob(os.path.join(root, "%s_%s" % (mode, which), "*counter_collection.csv"))
             cnt[which] = groups(pc[0], lambda r: float(r["Counter_Value"])) if pc else {}
+        first = {k: v[0] for k, v in dur.items() if len(v) == PROFILE_REPS + 1}
+        dur = collections.OrderedDict((k, v[1:] if len(v) == PROFILE_REPS + 1 else v) for k, v in dur.items())
+        for which in cnt:
+            cnt[which] = {k: (v[1:] if len(v) == PROFILE_REPS + 1 else v) for k, v in cnt[which].items()}
         matched = [(k, v) for k, v in dur.items() if len(v) == PROFILE_REPS]
         print()
-        print("== %s pass: %d launches per kernel (`python3 bench.py --profile-pass %s`) ==" % (mode, PROFILE_REPS, mode))
+        print("== %s pass: %d launches per kernel after one uncounted first launch, whose duration is the `first_us` column (`python3 bench.py --profile-pass %s`) ==" % (mode, PROFILE_REPS, mode))
         if len(matched) != len(plan):
             print("!! %d groups of %d dispatches in the trace, %d in the plan: labels below may be off" % (len(matched), PROFILE_REPS, len(plan)))
         scale = {}
@@ -363,7 +397,7 @@ def summarize_profile(root):
                 kib = float(np.mean(cnt[which][ck[0]]))
                 scale[which] = (1 << 20) / kib
                 print("byte-counter scale from copy_32 (1 GiB each way): %s_SIZE reads %.1f KiB per dispatch -> x %.4f" % (which.upper(), kib, scale[which]))
-        print("%-74s %-58s %7s %7s %7s %7s %8s %6s %10s %10s" % ("workload", "kernel", "avg_us", "med_us", "min_us", "max_us", "GB/s", "frac", "fetch_MiB", "write_MiB"))
+        print("%-74s %-58s %7s %7s %7s %7s %8s %8s %6s %10s %10s" % ("workload", "kernel", "avg_us", "med_us", "min_us", "max_us", "first_us", "GB/s", "frac", "fetch_MiB", "write_MiB"))
         for (key, v), (label, nbytes, _) in zip(matched, plan):
             avg = float(np.mean(v))
             fm = wm = float("nan")
@@ -371,10 +405,117 @@ def summarize_profile(root):
                 fm = float(np.mean(cnt["fetch"][key])) * scale["fetch"] / 1024
             if key in cnt.get("write", {}) and "write" in scale:
                 wm = float(np.mean(cnt["write"][key])) * scale["write"] / 1024
-            print("%-74s %-58s %7.1f %7.1f %7.1f %7.1f %8.0f %6.3f %10.1f %10.1f" % (label[:74], short(key[0])[:58], avg, float(np.median(v)), min(v), max(v),
-                                                                                nbytes / avg * 1e-3, nbytes / avg * 1e-3 / HBM_PEAK_GBS, fm, wm))
+            print("%-74s %-58s %7.1f %7.1f %7.1f %7.1f %8.1f %8.0f %6.3f %10.1f %10.1f" % (label[:74], short(key[0])[:58], avg, float(np.median(v)), min(v), max(v),
+                                                                                      first.get(key, float("nan")), nbytes / avg * 1e-3, nbytes / avg * 1e-3 / HBM_PEAK_GBS, fm, wm))
             if mode == "warm" and label.startswith("reluback_32_11") and fm == fm and wm == wm:
                 print("traffic reluback_32_11 %d   (bytes per launch: fetch + write above)" % int((fm + wm) * (1 << 20)))
+
+
+def timeline(torch, K):
+    """Per-workgroup stamps from the library's own kernels, compiled a second time with -DKNET8_TIMELINE (lib/libknet8_timeline.so: the same
+    headers, one more kernel argument, nothing restated).  For every fp32 row of configs 3-5 and its yardstick: eight stamped launches on cold
+    buffers (each after three unstamped launches on other buffer sets), medians of the percentiles over the eight; times in microseconds from the
+    first workgroup's start.  `inside` = first workgroup's start to last workgroup's end; the back-to-back figure is the same library with the stamps'
+    buffer switched off."""
+    lib = K.libknet8()
+    setbuf = lib.lib.knet8_timeline_set   # AttributeError unless KNET8_LIBRARY names the measurement build
+    setbuf.argtypes, setbuf.restype = [ctypes.c_void_p], None
+    slots = 16384
+    dev = lib.fn["knet8_malloc"](slots * 32)
+    host = np.zeros(slots * 4, np.uint64)
+    print("libknet8 on one MI355X: per-workgroup time stamps (100 MHz wall clock) written by the library's own kernels in its measurement build")
+    print("(`python3 bench.py --timeline`; -DKNET8_TIMELINE adds a stamp buffer argument to the kernels and nothing else).  Cold buffers; microseconds")
+    print("from the first workgroup's start; medians over 8 stamped launches.  mid = operands arrived and own share reduced (column kernels: the column's")
+    print("sum is known; split reductions: before the partial result is stored); end = last store acknowledged (after the ticket, and the combine for the")
+    print("last workgroup of a group).")
+    for key, label, nbytes, nsets, make_launch, yard in kernel_cases(torch, K, widths=("32",)):
+        launches = [make_launch(i) for i in range(nsets)]
+        setbuf(None)
+        for l in launches:
+            l()
+        K.synchronize()
+        stats = []
+        for r in range(8):
+            K.knet8("fill_32", slots * 8, ctypes.c_float(0.0), dev)
+            for q in range(1, 4):
+                launches[(r + q) % nsets]()
+            setbuf(dev)
+            launches[r % nsets]()
+            setbuf(None)
+            K.synchronize()
+            lib.fn["knet8_memcpy"](host.ctypes.data, dev, host.nbytes, 2, lib.stream)
+            st = host.reshape(slots, 4)
+            st = st[st[:, 2] != 0]
+            if len(st) == 0:
+                break
+            t0, t1, t2 = (st[:, c].astype(np.int64) for c in range(3))
+            xcc = (st[:, 3] & np.uint64(0xffffffff)).astype(np.int64)
+            origin = t0.min()
+            pct = lambda v: [float(np.percentile((v - origin) / 100.0, q)) for q in (0, 10, 50, 90, 100)]
+            stats.append({"n": len(st), "inside": (t2.max() - origin) / 100.0, "start": pct(t0), "mid": pct(t1), "end": pct(t2),
+                          "xcc": [float(np.mean((t2[xcc == x] - origin) / 100.0)) if np.any(xcc == x) else float("nan") for x in range(8)]})
+        if not stats:
+            print()
+            print("%s [%s]: this kernel carries no stamps (a one-shot kernel like its yardstick)" % (label, key))
+            continue
+        med = lambda f: np.median(np.array([f(s_) for s_ in stats]), axis=0)
+        inside = float(med(lambda s_: s_["inside"]))
+        ev = Events(K)
+        n = 24
+        b = ev.time(lambda: [launches[i % nsets]() for i in range(n)])
+        K.synchronize()
+        b2b = ev.ms(b) / n * 1e3
+        ev.close()
+        print()
+        print("%s [%s]: %d workgroups stamped" % (label, key, stats[0]["n"]))
+        print("  inside the launch: %6.2f us (%5.0f GB/s, %.3f of peak)   back to back, HIP events: %6.2f us per launch (%.3f of peak)   around the launch: %.2f us"
+              % (inside, nbytes / inside * 1e-3, nbytes / inside * 1e-3 / HBM_PEAK_GBS, b2b, nbytes / b2b * 1e-3 / HBM_PEAK_GBS, b2b - inside))
+        for name in ("start", "mid", "end"):
+            v = med(lambda s_: s_[name])
+            print("  %-5s min %6.2f  p10 %6.2f  p50 %6.2f  p90 %6.2f  max %6.2f" % (name, v[0], v[1], v[2], v[3], v[4]))
+        print("  mean end per XCD: " + " ".join("%d: %.1f" % (x, v) for x, v in enumerate(med(lambda s_: s_["xcc"])) if v == v))
+        sys.stdout.flush()
+    lib.check()
+
+
+def two_streams(torch, K):
+    """The diagnostic for where a 20-35 us launch loses its time: the same 24 independent cold launches issued to one stream, and alternated over
+    two streams of the same (default) priority, so that one launch's ramp and drain overlap its neighbour's.  If the aggregate per-launch time falls
+    toward the one-shot yardstick's, the loss is between launches; if it does not, it is inside the kernel."""
+    lib = K.libknet8()
+    fn = lib.fn
+    s1 = lib.stream
+    s2 = fn["knet8_stream_create"]()
+    print("libknet8 on one MI355X: 24 cold launches per kernel on one stream and alternated over two streams (`python3 bench.py --two-streams`).")
+    print("us per launch = elapsed time of the batch / 24 (HIP events; two streams: from the first record to the later of the two streams' ends); median of 5 batches.")
+    print("%-92s %10s %10s %8s %10s %10s" % ("kernel", "1 stream", "2 streams", "ratio", "frac 1s", "frac 2s"))
+    for key, label, nbytes, nsets, make_launch, yard in kernel_cases(torch, K, widths=("32",)):
+        launches = [make_launch(i) for i in range(nsets)]
+        n = max(24, 2 * nsets)
+        res = {}
+        for mode in (1, 2):
+            times = []
+            for rep in range(6):
+                for s_ in (s1, s2):
+                    fn["knet8_synchronize"](s_)
+                e0, e1, e2 = fn["knet8_event_create"](), fn["knet8_event_create"](), fn["knet8_event_create"]()
+                fn["knet8_event_record"](e0, s1)
+                for i in range(n):
+                    lib.stream = s2 if (mode == 2 and i % 2) else s1
+                    launches[i % nsets]()
+                lib.stream = s1
+                fn["knet8_event_record"](e1, s1)
+                fn["knet8_event_record"](e2, s2)
+                t = max(fn["knet8_event_elapsed"](e0, e1), fn["knet8_event_elapsed"](e0, e2))
+                for e in (e0, e1, e2):
+                    fn["knet8_event_destroy"](e)
+                if rep:
+                    times.append(t / n * 1e3)
+            res[mode] = float(np.median(times))
+        print("%-92s %10.2f %10.2f %8.3f %10.3f %10.3f" % (label[:92], res[1], res[2], res[2] / res[1], nbytes / res[1] * 1e-3 / HBM_PEAK_GBS,
+                                                         nbytes / res[2] * 1e-3 / HBM_PEAK_GBS), flush=True)
+    lib.check()
+    fn["knet8_stream_destroy"](s2)
 
 
 def shape_scan(torch, K):
@@ -542,15 +683,13 @@ def c_host_steps(K, steps=5000):
                 raise RuntimeError(name + " failed: " + r.stderr)
             rates = dict(line.split() for line in r.stdout.strip().splitlines())
             return rates, float(np.fromfile(fout, dtype=np.float32, count=1)[0])
-        for label, own in (("config1 reference launch sequence (C host): 18 launches of reference-named entry points, products on hipBLASLt (default routing)", 0),
-                           ("config1 reference launch sequence (C host), products on the library's own kernels (knet8_tune key 3 = 270)", 270)):
+        for label, own in (("cfg1_c_ref", 0), ("cfg1_c_ref_own", 270)):
             rates, loss = run("mlp_ref_sequence", [str(max(steps // 2, 1)), str(own)])
             rate = float(rates["steps_per_sec"])
             out[label] = {"steps_per_sec": rate, "ms_per_step": 1e3 / rate, "loss": loss}
         rates, loss = run("mlp_step", [str(steps)])
         rate = float(rates["steps_per_sec"])
-        out["config1 same step through the fused layer entry points (C host, eager, 3 launches: hidden layer forward, output layer forward + loss + backward, "
-            "hidden layer backward; opt-in API, own MFMA kernels in the two backward launches)"] = {
+        out["cfg1_c_fused"] = {
             "steps_per_sec": rate, "ms_per_step": 1e3 / rate, "graph_replay_steps_per_sec": float(rates["graph_steps_per_sec"]), "loss": loss}
     return out
 
@@ -566,22 +705,22 @@ def cpu_side_table():
         t0 = time.perf_counter()
         f()
         dt = time.perf_counter() - t0
-        out[name] = {"ms": round(dt * 1e3, 2), "GBps": round(nbytes / dt * 1e-9, 2)}
+        out[name] = round(nbytes / dt * 1e-9, 2)
     x = rng.standard_normal((4096, 8192), dtype=np.float32)
     xf = x.ravel(order="F")
-    t("sum (4096,8192) dims=1", x.nbytes, lambda: ko.sum_21(xf, 4096, 8192))
-    t("sum (4096,8192) dims=2", x.nbytes, lambda: ko.sum_21(xf, 1, 4096))
+    t("sum21_d1", x.nbytes, lambda: ko.sum_21(xf, 4096, 8192))
+    t("sum21_d2", x.nbytes, lambda: ko.sum_21(xf, 1, 4096))
     x = rng.standard_normal((56, 56, 256, 64), dtype=np.float32)
     xf = x.ravel(order="F")
-    t("sum NCHW (56,56,256,64)->(1,1,256,1)", x.nbytes, lambda: ko.sum_21(xf, 3136, 256))
+    t("sum21_nchw", x.nbytes, lambda: ko.sum_21(xf, 3136, 256))
     for C, N in ((32000, 512), (1000, 4096)):
         y = rng.standard_normal((C, N), dtype=np.float32)
         dy = rng.standard_normal((C, N), dtype=np.float32)
         labels = rng.integers(1, C + 1, size=N)
-        t("logsoftmaxback (%d,%d)" % (C, N), 12 * C * N, lambda: ko.logsoftmaxback(y, dy, dims=1))
-        t("nll backward chain (%d,%d)" % (C, N), 8 * C * N, lambda: ko.nll_back(y, labels))
+        t("lsmback_%d" % C, 12 * C * N, lambda: ko.logsoftmaxback(y, dy, dims=1))
+        t("nll_chain_%d" % C, 8 * C * N, lambda: ko.nll_back(y, labels))
     y = rng.standard_normal(4096 * 2048).astype(np.float32)
-    t("dropback (4096,2048)", 12 * y.size, lambda: ko.dropback(0.5, y, y, y))
+    t("dropback", 12 * y.size, lambda: ko.dropback(0.5, y, y, y))
     return out
 
 
@@ -627,38 +766,75 @@ def cpu_baseline():
                       "timed through ctypes, outputs written into touched memory; Knet's CPU Array path for these ops is single-threaded broadcast"}
 
 
+MLP_LEGEND = {
+    "cfg1_tape": "config 1 (MLP 784-64-10, batch 100) forward + backward, eager through the Python tape, step-by-step nll as in the reference",
+    "cfg1_tape_fnll": "same, fused nll kernel",
+    "cfg1_graph": "same step captured once into a hipGraph and replayed",
+    "cfg1_c_ref": "config 1 from a C99 host issuing the 18 launches an unchanged Knet model emits (reference-named entry points only, products on hipBLASLt: default routing)",
+    "cfg1_c_ref_own": "same C host with the library's own small-product kernels switched on (knet8_tune key 3 = 270)",
+    "cfg1_c_fused": "same step through the opt-in fused layer entry points (C host, eager, 3 launches; own MFMA kernels in the two backward launches)",
+    "cfg1_graph_dense": "config 1 graph with dense layers (product, bias and relu in one launch)",
+    "cfg1_graph_dense_nll": "config 1 graph, output layer forward + loss + gradients in one launch (3 launches per step)",
+    "cfg5_eager": "config 5 (7 x 4096 hidden + 1000 classes, batch 2048, relu + dropout 0.5) forward + backward, eager, fused nll",
+    "cfg5_graph": "same, captured into a hipGraph",
+    "cfg5_graph_fused": "same graph with fused bias+relu+dropout layers",
+    "cfg5_nodrop_graph": "config 5 shapes without dropout, graph, product / bias add / relu as three launches per layer",
+    "cfg5_nodrop_graph_dense": "config 5 shapes without dropout, graph, bias and relu in the epilogue of the hipBLASLt product",
+    "cfg1_eager_dense_nll": "(--all) config 1 eager with dense layers and dense_nll",
+    "beside_784_512_512_10": "(--all) MLP 784-512-512-10 batch 128, graph with dense layers and dense_nll (own MFMA kernels throughout): not a benchmark config",
+}
+
+
+def mlp_table(torch, K, everything):
+    c1, c5 = [784, 64, 10], [4096] * 8 + [1000]
+    runs = [("cfg1_tape", lambda: mlp_steps(torch, K, c1, 100, 0.0, 200, False)),
+            ("cfg1_tape_fnll", lambda: mlp_steps(torch, K, c1, 100, 0.0, 200, True)),
+            ("cfg1_graph", lambda: mlp_steps(torch, K, c1, 100, 0.0, 2000, True, graph=True)),
+            ("cfg1_graph_dense", lambda: mlp_steps(torch, K, c1, 100, 0.0, 2000, True, graph=True, layers=True)),
+            ("cfg1_graph_dense_nll", lambda: mlp_steps(torch, K, c1, 100, 0.0, 2000, True, graph=True, layers=True, head=True)),
+            ("cfg5_eager", lambda: mlp_steps(torch, K, c5, 2048, 0.5, 20, True)),
+            ("cfg5_graph", lambda: mlp_steps(torch, K, c5, 2048, 0.5, 20, True, graph=True)),
+            ("cfg5_graph_fused", lambda: mlp_steps(torch, K, c5, 2048, 0.5, 20, True, graph=True, layers=True)),
+            ("cfg5_nodrop_graph", lambda: mlp_steps(torch, K, c5, 2048, 0.0, 20, True, graph=True)),
+            ("cfg5_nodrop_graph_dense", lambda: mlp_steps(torch, K, c5, 2048, 0.0, 20, True, graph=True, layers=True))]
+    if everything:
+        runs += [("cfg1_eager_dense_nll", lambda: mlp_steps(torch, K, c1, 100, 0.0, 1000, True, layers=True, head=True)),
+                 ("beside_784_512_512_10", lambda: mlp_steps(torch, K, [784, 512, 512, 10], 128, 0.0, 1000, True, graph=True, layers=True, head=True))]
+    out = {k: f() for k, f in runs}
+    ch = c_host_steps(K)
+    if ch:
+        out.update(ch)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-extras", action="store_true", help="only the config-2 step, roofline and CPU baseline")
+    ap.add_argument("--all", action="store_true", help="also the per-row detail of configs 3-5 (both timing methods), the kernels next to the path "
+                    "(random numbers, permutations, strided softmax), two more MLP variants and the legend of the short keys")
     ap.add_argument("--profile-pass", choices=["warm", "cold"], default=None,
-                    help="launch each quoted kernel %d times (config 2 after a known-size copy kernel; configs 3-5 on one buffer set or "
+                    help="launch each quoted kernel 1 + %d times (config 2 after a known-size copy kernel; configs 3-5 on one buffer set or "
                          "rotating over more than 1 GB) and exit: the workload of the rocprofv3 runs" % PROFILE_REPS)
     ap.add_argument("--plan-out", default=None, help="with --profile-pass: where the launch plan goes (default <tmp>/knet8_profile/<mode>_plan.json)")
     ap.add_argument("--summarize-profile", metavar="DIR", default=None, help="print the text summary of the rocprofv3 output under DIR and exit (no GPU needed)")
     ap.add_argument("--scan", action="store_true", help="time the gradient-path kernels on shapes away from the benchmark's (text table) and exit")
     ap.add_argument("--timeline", action="store_true",
-                    help="compile tests/c_host/kernel_timeline.hip with hipcc and run it: per-workgroup start / loads-arrived / end stamps of the "
-                         "launch shapes behind the config 3-4 rows, next to a one-shot elementwise launch and an empty kernel")
+                    help="load the measurement build of the library (lib/libknet8_timeline.so: the same sources with -DKNET8_TIMELINE) and print per-workgroup "
+                         "start / mid / end stamps of the kernels behind the config 3-5 rows and of their one-shot yardsticks")
+    ap.add_argument("--two-streams", action="store_true", help="24 cold launches of every config 3-5 kernel on one stream and alternated over two (text table) and exit")
     args = ap.parse_args()
     if args.summarize_profile:
         summarize_profile(args.summarize_profile)
         return
-    if args.timeline:
-        import subprocess
-        import tempfile
-        with tempfile.TemporaryDirectory() as tmp:
-            exe = os.path.join(tmp, "kernel_timeline")
-            subprocess.check_call([os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "-O3", "--offload-arch=gfx950", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
-                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result",
-                                   os.path.join(ROOT, "tests", "c_host", "kernel_timeline.hip"), "-o", exe], stderr=subprocess.DEVNULL)
-            sys.exit(subprocess.call([exe]))
     if args.gpus != 1:
         print("bench.py measures one MI355X: the gradient kernels have no multi-GPU path (every GPU box here has one GPU); "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.timeline:
+        os.environ["KNET8_LIBRARY"] = os.path.join(ROOT, "knet.jl_amd", "lib", "libknet8_timeline.so")
     import torch  # device memory for the synthetic inputs, and the synchronisation the bench contract asks for
     import __graft_entry__ as ge
     K = ge.load_package()
@@ -670,6 +846,12 @@ def main():
         K.libknet8().stream = K.libknet8().fn["knet8_stream_create"]()
     if args.scan:
         shape_scan(torch, K)
+        return
+    if args.timeline:
+        timeline(torch, K)
+        return
+    if args.two_streams:
+        two_streams(torch, K)
         return
     if args.profile_pass:
         plan_path = args.plan_out or os.path.join(tempfile.gettempdir(), "knet8_profile", args.profile_pass + "_plan.json")
@@ -686,53 +868,41 @@ def main():
         "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32+f64", "data": "synthetic",
         "config": {"workload": "benchmark config 2: {relu,sigm,tanh,elu,selu}back on 2^28 fp32 and 2^27 fp64 vectors, "
-                               "x,dy~N(0,1) seeded, y=f(x); 10 launches per step", "frac_of_hbm_peak": value / HBM_PEAK_GBS},
+                               "x,dy~N(0,1) seeded, y=f(x); 10 launches per step", "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": {"bound": "hbm", "kernel": "reluback_32_11 (ew_vec_kernel<float,2>)", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": dom["GBps"] / HBM_PEAK_GBS, "traffic": profiled_traffic("reluback_32_11"),
-                     "traffic_source": "from_profile: profiles/libknet8_kernels_profile_pass.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --profile-pass`), not measured in this run",
+                     "traffic_source": "profiles/libknet8_kernels_profile_pass.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --profile-pass`), not measured in this run",
                      "algorithmic_bytes_per_launch": dom["bytes"],
                      "avg_launch_us": dom["us"]},
-        "kernels_config2": {k: {"us": round(v["us"], 2), "GBps": round(v["GBps"], 1), "frac": round(v["GBps"] / HBM_PEAK_GBS, 4)} for k, v in per_kernel.items()},
     }
     torch.cuda.empty_cache()
     K.libknet8().fn["knet8_trim"]()
+    detail = {}
     if not args.no_extras:
         ex = extras(torch, K)
-        line["kernels_config3_4_5"] = {k: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for k, v in ex.items()}
+        line["roofline"]["rows"] = roofline_rows(ex)
+        line["roofline"]["rows_legend"] = ROWS_LEGEND
+        if args.all:
+            detail["kernels_config3_4_5"] = {label: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for label, _, v in ex.values()}
+        del ex
         torch.cuda.empty_cache()
         K.libknet8().fn["knet8_trim"]()
-        nb = neighbours(torch, K)
-        line["kernels_next_to_the_path"] = {k: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for k, v in nb.items()}
-        K.libknet8().fn["knet8_trim"]()
-        line["mlp"] = {
-            "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager through the tape, step-by-step nll as in the reference)":
-                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, False),
-            "config1 MLP 784-64-10 batch 100 (fwd+bwd, eager, fused nll)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 200, True),
-            "config1 MLP 784-64-10 batch 100 (fwd+bwd captured once into a hipGraph, replayed)":
-                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True),
-            "config1 same graph with dense layers (product, bias and relu in one launch)": mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True),
-            "config1 eager with dense layers and dense_nll (3 launches per step, loss left on the device)":
-                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 1000, True, layers=True, head=True),
-            "config1 same graph, output layer forward + loss + gradients in one launch (dense_nll: 3 launches per step)":
-                mlp_steps(torch, K, [784, 64, 10], 100, 0.0, 2000, True, graph=True, layers=True, head=True),
-            "beside the configs: MLP 784-512-512-10 batch 128, graph with dense layers and dense_nll (own MFMA kernels throughout)":
-                mlp_steps(torch, K, [784, 512, 512, 10], 128, 0.0, 1000, True, graph=True, layers=True, head=True),
-            "config5 MLP 7x4096 hidden + 1000 classes, batch 2048, relu+dropout 0.5 (fwd+bwd, eager, fused nll)":
-                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True),
-            "config5 same, captured into a hipGraph": mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True),
-            "config5 same graph with fused bias+relu+dropout layers":
-                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.5, 20, True, graph=True, layers=True),
-            "config5 shapes without dropout, graph, product / bias add / relu as three launches per layer":
-                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.0, 20, True, graph=True),
-            "config5 shapes without dropout, graph, dense layers: bias and relu in the epilogue of the hipBLASLt product (z never written or re-read)":
-                mlp_steps(torch, K, [4096] * 8 + [1000], 2048, 0.0, 20, True, graph=True, layers=True),
-        }
-        ch = c_host_steps(K)
-        if ch:
-            line["mlp"].update(ch)
+        if args.all:
+            nb = neighbours(torch, K)
+            detail["kernels_next_to_the_path"] = {k: {m: {kk: round(vv, 4) for kk, vv in r.items()} for m, r in v.items()} for k, v in nb.items()}
+            K.libknet8().fn["knet8_trim"]()
     line["cpu_baseline"] = cpu_baseline()
+    # [microseconds per launch, fraction of 8 TB/s] of the ten config-2 kernels inside the timed region
+    line["kernels_config2"] = {k: [round(v["us"], 1), round(v["GBps"] / HBM_PEAK_GBS, 3)] for k, v in per_kernel.items()}
     if not args.no_extras:
-        line["cpu_oracle_config3_4_5 (1 thread, algorithmic GB/s)"] = cpu_side_table()
+        mlp = mlp_table(torch, K, args.all)
+        line["mlp_steps_per_sec"] = {k: round(v["steps_per_sec"], 1) for k, v in mlp.items()}
+        line["mlp_loss"] = {"cfg1": round(mlp["cfg1_tape"]["loss"], 5), "cfg5": round(mlp["cfg5_eager"]["loss"], 5)}
+        line["cpu_oracle_GBps_1_thread"] = cpu_side_table()
+        if args.all:
+            detail["mlp"] = mlp
+            detail["mlp_legend"] = MLP_LEGEND
+    line.update(detail)
     print(json.dumps(line))
 
 

@@ -14,6 +14,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(PKG, "lib", "libknet8.so")
+# The measurement build: the same sources with -DKNET8_TIMELINE, whose gradient kernels stamp the wall clock per workgroup
+# (`bench.py --timeline`).  Never loaded by the package unless KNET8_LIBRARY names it.
+LIB_TIMELINE = os.path.join(PKG, "lib", "libknet8_timeline.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off", "-fno-fast-math",
@@ -42,9 +45,10 @@ def sources():
     return srcs
 
 
-def compile_one(src):
-    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-DKNET8_BUILD_ID=\"%s\"" % source_id(), "-c", src, "-o", obj]
+def compile_one(job):
+    src, timeline = job
+    obj = os.path.join(OBJ, os.path.basename(src).replace(".hip", "_timeline.o" if timeline else ".o"))
+    cmd = [HIPCC] + FLAGS + (["-DKNET8_TIMELINE"] if timeline else []) + ["-DKNET8_BUILD_ID=\"%s\"" % source_id(), "-c", src, "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -52,21 +56,25 @@ def compile_one(src):
     return obj, out
 
 
-def build(verbose=False):
+def build(verbose=False, timeline=True):
+    """Compile and link libknet8.so and (timeline=True) the measurement build libknet8_timeline.so.  Returns the path of the former."""
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
     srcs = sources()
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        results = list(ex.map(compile_one, srcs))
-    objs = [o for o, _ in results]
+    jobs = [(s, False) for s in srcs] + ([(s, True) for s in srcs] if timeline else [])
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+        results = list(ex.map(compile_one, jobs))
     if verbose:
         for _, out in results:
             if out.strip():
                 print(out)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-L/opt/rocm/lib", "-lhipblaslt"]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n" + r.stdout)
+    for lib, objs in ((LIB, [o for o, _ in results[:len(srcs)]]), (LIB_TIMELINE, [o for o, _ in results[len(srcs):]])):
+        if not objs:
+            continue
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs + ["-L/opt/rocm/lib", "-lhipblaslt"]
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stdout)
     return LIB
 
 

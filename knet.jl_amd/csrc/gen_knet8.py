@@ -625,17 +625,24 @@ HEADER_RUNTIME = """
  * only when the work that uses it was queued on the stream that its next user will queue on too (one stream per pool user), or after knet8_synchronize. */
 KNET8_API void* knet8_malloc(size_t nbytes);
 KNET8_API void knet8_free(void* ptr);
-/* replaces Knet.gc, src/knetarrays/kptr.jl:204-226: hipFree every cached block; returns the bytes released */
+/* replaces Knet.gc, src/knetarrays/kptr.jl:204-226: waits for the device, then gives back every cached block of the pool, the scratch the
+   library keeps per stream for split reductions (current and outgrown buffers) and its hipBLASLt workspaces -- except scratch and workspaces that
+   were handed out while their stream was being captured, which a graph may still name; returns the bytes released */
 KNET8_API size_t knet8_trim(void);
 /* replaces meminfo/kmeminfo, src/knetarrays/kptr.jl:254-255: out[0]=bytes in use, out[1]=bytes cached, out[2]=hipMalloc calls, out[3]=pool hits */
 KNET8_API void knet8_meminfo(size_t* out4);
+/* no counterpart in the reference: out[0] = hipMalloc calls and out[1] = hipFree calls the library has made so far (pool, scratch, workspaces: every
+   one is counted), out[2] = bytes it currently holds outside the pool (per-stream reduction scratch, hipBLASLt workspaces, the 256-byte slots of
+   the _20 reductions), out[3] = plain products that ran on the library's own tiles because hipBLASLt reported no algorithm, out[4] = free and
+   out[5] = total device memory in bytes (hipMemGetInfo) */
+KNET8_API void knet8_stats(unsigned long long* out6);
 /* replaces the copyto!/unsafe_copyto! paths of src/knetarrays/copy.jl:6-11: kind 1 = host->device, 2 = device->host, 3 = device->device;
    host copies return when the data has landed */
 KNET8_API int knet8_memcpy(void* dst, const void* src, size_t nbytes, int kind, hipStream_t stream);
 KNET8_API int knet8_device_count(void);
 KNET8_API int knet8_set_device(int dev);
-/* non-blocking streams; destroying one waits for its work and frees the reduction scratch the library keeps for it (destroy graphs
-   captured on it first) */
+/* non-blocking streams; destroying one waits for its work and frees the reduction scratch and the hipBLASLt workspace the library keeps
+   for it (destroy graphs captured on it first) */
 KNET8_API hipStream_t knet8_stream_create(void);
 KNET8_API void knet8_stream_destroy(hipStream_t stream);
 KNET8_API int knet8_synchronize(hipStream_t stream);
@@ -675,7 +682,8 @@ KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hip
    every product of gemm_S / gemm_bias_act_S goes to hipBLASLt);
    key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270);
    key 5: non-zero makes the library behave as if the scratch memory of split launches could not be allocated (for tests of that error path);
-   key 6: non-zero keeps softmax columns of 128 to 256 KB in registers alone instead of registers + LDS (for comparisons) */
+   key 6: non-zero keeps softmax columns of 128 to 256 KB in registers alone instead of registers + LDS (for comparisons);
+   key 7: non-zero makes the hipBLASLt route of gemm_S do everything but the vendor call itself (for measuring the library's own share of a call's host time) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
    src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */
@@ -694,7 +702,9 @@ KNET8_API int bmm_64(char transa, char transb, int m, int n, int k, double alpha
 /* dense layer in one call: C = act(alpha*op(A)*op(B) + bias[i]) with bias of length m and act 0 (none) or 1 (relu).  No counterpart in
    the reference, which runs gemm!, the bias broadcast (src/knetarrays/binary.jl:61-95) and relu (src/ops20_gpu/activation.jl:17-29) as
    three launches.  Bias and relu run in the output stage of the hipBLASLt product (its BIAS / RELU_BIAS epilogues), so the result is
-   written once; where hipBLASLt has no such kernel the product is followed by one in-place pass. */
+   written once; where hipBLASLt has no such kernel the product is followed by one in-place pass.  The relu here is z > 0 ? z : 0 on every
+   route -- the vendor epilogue's and the reference's device relu (src/libknet8/ops.jl:63): a NaN in the product comes out as 0, +Inf stays,
+   -Inf becomes 0 -- whereas relu_S follows the CPU path and keeps a NaN. */
 KNET8_API int gemm_bias_act_32_stream(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc, hipStream_t stream);
 KNET8_API int gemm_bias_act_32(char transa, char transb, int m, int n, int k, float alpha, float* A, int lda, float* B, int ldb, float* bias, int act, float* C, int ldc);
 KNET8_API int gemm_bias_act_64_stream(char transa, char transb, int m, int n, int k, double alpha, double* A, int lda, double* B, int ldb, double* bias, int act, double* C, int ldc, hipStream_t stream);

@@ -136,6 +136,48 @@ template <typename T> __device__ __forceinline__ T ld_coherent(const T* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- per-workgroup time stamps (measurement build only) ------------------------------------------------------------
+// With -DKNET8_TIMELINE (a second library compiled from these same headers for measurements, never the one that ships) the kernels behind
+// the roofline tables take one more argument, a stamp buffer, and record for every `every`-th workgroup (all of them up to kTlSlots) the
+// 100 MHz wall clock at its start, at its phase boundary (operands arrived, own share reduced) and after its last store has been acknowledged,
+// with the XCD it ran on.  Without the macro the six macros below expand to nothing: the product's kernels carry no trace of them.
+#ifdef KNET8_TIMELINE
+struct TlStamp { unsigned long long t0, t1, t2; unsigned xcc, wg; };
+constexpr unsigned kTlSlots = 16384;
+struct TlClock {
+  TlStamp* buf;
+  unsigned long long t0, t1;
+  __device__ __forceinline__ explicit TlClock(TlStamp* b) : buf(b) { t0 = t1 = wall_clock64(); }
+  __device__ __forceinline__ void mid() { t1 = wall_clock64(); }
+  __device__ __forceinline__ void end() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned every = (gridDim.x + kTlSlots - 1) / kTlSlots;
+    if (buf != nullptr && threadIdx.x == 0 && blockIdx.x % every == 0) {
+      TlStamp q;
+      q.t0 = t0; q.t1 = t1; q.t2 = wall_clock64();
+      q.xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7;   // XCC_ID, bits 3:0
+      q.wg = blockIdx.x;
+      buf[blockIdx.x / every] = q;
+    }
+  }
+};
+#define KNET8_TL_PARAM , knet8::TlStamp* tl_buf
+#define KNET8_TL_PASS , tl_buf
+#define KNET8_TL_NONE , nullptr
+#define KNET8_TL_ARG , knet8::timeline_buffer()
+#define KNET8_TL_BEGIN knet8::TlClock tl_clock(tl_buf);
+#define KNET8_TL_MID tl_clock.mid();
+#define KNET8_TL_END tl_clock.end();
+#else
+#define KNET8_TL_PARAM
+#define KNET8_TL_PASS
+#define KNET8_TL_NONE
+#define KNET8_TL_ARG
+#define KNET8_TL_BEGIN
+#define KNET8_TL_MID
+#define KNET8_TL_END
+#endif
+
 }  // namespace knet8
 
 // ---- libm calls used by the operator tables (ocml, full precision: the library is built without fast-math)

@@ -33,7 +33,8 @@ template <typename T, typename F> struct EwApply<T, 3, F> {
 // trailing (n - tail0) elements are handled as scalars by the first lanes of workgroup 0.
 template <typename T, int NIN, typename F>
 __global__ __launch_bounds__(kEwBlock) void ew_vec_kernel(long nvec, int head, long tail0, long n, const T* a, const T* b,
-                                                          const T* c, T* out, F f) {
+                                                          const T* c, T* out, F f KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   typedef typename Vec16<T>::type V;
   constexpr int N = Vec16<T>::N;
   const long i = (long)blockIdx.x * kEwBlock + threadIdx.x;
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_vec_kernel(long nvec, int head, l
     if (e >= 0)
       out[e] = EwApply<T, NIN, F>::go(f, NIN >= 1 ? a[e] : T(0), NIN >= 2 ? b[e] : T(0), NIN >= 3 ? c[e] : T(0));
   }
+  KNET8_TL_END
 }
 
 // Scalar path for operands whose addresses differ modulo 16 bytes (sub-array views that start at
@@ -97,7 +99,7 @@ inline void launch_ew(hipStream_t stream, long n, const T* a, const T* b, const 
     long grid = (nvec + kEwBlock - 1) / kEwBlock;
     if (grid < 1) grid = 1;
     hipLaunchKernelGGL((ew_vec_kernel<T, NIN, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, nvec, (int)head, tail0, n,
-                       a, b, c, out, f);
+                       a, b, c, out, f KNET8_TL_ARG);
   } else {
     const long grid = (n + kEwBlock * 4 - 1) / (kEwBlock * 4);
     hipLaunchKernelGGL((ew_scalar_kernel<T, NIN, F>), dim3((unsigned)grid), dim3(kEwBlock), 0, stream, n, a, b, c, out, f);

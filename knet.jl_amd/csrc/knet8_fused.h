@@ -98,7 +98,8 @@ inline void launch_bias_act(hipStream_t stream, long m, long n, const T* z, cons
 // each moved with its own 4- or 8-byte access (see strided_walk).
 template <typename T, typename F, int NV, int BT, int U, bool SC>
 __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const T* yv, long m, long n, long jchunk, unsigned P, T* dz, T* __restrict__ db,
-                                                              T* partial, unsigned* counters, F f) {
+                                                              T* partial, unsigned* counters, F f KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   constexpr int TILE = kWave * NV;
   constexpr int NW = BT / kWave;
   __shared__ T lds[NW][TILE];
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
         for (int e = 0; e < NV; e++) acc[e] = acc[e] + g[q][e];
     }
   }
+  KNET8_TL_MID
   if (P > 1) {
 #pragma unroll
     for (int e = 0; e < NV; e++) lds[wave][SC ? e * kWave + lane : lane * NV + e] = acc[e];
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
       for (int w = 0; w < NW; w++) r = r + lds[w][threadIdx.x];
       st_coherent(partial + (at * P + p) * TILE + threadIdx.x, r);
     }
-    if (!last_block_ticket(counters + at * kTicketStride, P, &flag)) return;
+    if (!last_block_ticket(counters + at * kTicketStride, P, &flag)) { KNET8_TL_END return; }
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = T(0);
     strided_walk<T, RedSum<T>, NV, false, NW, kCombineU, SC>(partial + at * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
@@ -182,6 +184,7 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
     for (int w = 0; w < NW; w++) r = r + lds[w][threadIdx.x];
     db[a] = r;
   }
+  KNET8_TL_END
 }
 
 // The element gradient alone, over the flat array (few rows: see launch_actback_biasgrad).
@@ -235,7 +238,7 @@ inline void launch_actback_biasgrad(hipStream_t stream, long m, long n, const T*
   T* partial = static_cast<T*>(ws.partial);
   const bool big = jchunk >= 64;
 #define KNET8_ABG(BT, U, SC) \
-  hipLaunchKernelGGL((actback_biasgrad_kernel<T, F, N, BT, U, SC>), grid, dim3(BT), 0, stream, dy, y, m, n, jchunk, P, dz, db, partial, ws.counters, f)
+  hipLaunchKernelGGL((actback_biasgrad_kernel<T, F, N, BT, U, SC>), grid, dim3(BT), 0, stream, dy, y, m, n, jchunk, P, dz, db, partial, ws.counters, f KNET8_TL_ARG)
   if (vec) { if (big) KNET8_ABG(1024, 2, false); else KNET8_ABG(256, 4, false); }
   else     { if (big) KNET8_ABG(1024, 2, true); else KNET8_ABG(256, 4, true); }
 #undef KNET8_ABG

@@ -20,13 +20,14 @@ __device__ __forceinline__ float kfma(float a, float b, float c) { return __buil
 __device__ __forceinline__ double kfma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
 // Output stage shared by the kernels below: v = alpha*acc [+ beta*C] [+ bias[i]] [relu].  Each step is one rounded operation, so
-// a product with bias and relu folded in gives the bits of the product followed by the separate bias-add and relu launches.
+// a product with bias and relu folded in gives the bits of the product followed by the separate bias-add and relu launches (on data without
+// NaN: this relu is z > 0 ? z : 0 on every route of gemm_bias_act_S, the vendor epilogue included, where relu_S keeps a NaN).
 template <typename T>
 __device__ __forceinline__ void gemm_store(T* c, T acc, T alpha, T beta, const T* bias, int i, int act) {
   T v = alpha * acc;
   if (beta != T(0)) v = v + beta * *c;
   if (bias) v = v + bias[i];
-  if (act == 1) v = v != v ? v : (v > T(0) ? v : T(0));
+  if (act == 1) v = v > T(0) ? v : T(0);   // the device relu of the reference (src/libknet8/ops.jl:63) and of the vendor epilogue: NaN -> 0
   *c = v;
 }
 

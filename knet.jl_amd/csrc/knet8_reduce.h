@@ -49,7 +49,8 @@ template <typename Op, typename T> struct MergeFn {
 // of the K/NV units of output j.
 template <typename T, typename Op, int NV, bool SINGLE, int BT, int U>
 __global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x, long sy, long ny, long units, long chunk,
-                                                               unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
+                                                               unsigned P, T* __restrict__ y, T* partial, unsigned* counters KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   constexpr int NW = BT / kWave;
   __shared__ T lds[NW];
   __shared__ unsigned flag;
@@ -95,12 +96,14 @@ __global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x,
 #pragma unroll
   for (int e = 1; e < NV; e++) r = Op::merge(r, acc[e]);
   r = block_reduce<T, NW>(r, lds, MergeFn<Op, T>(), Op::init());
+  KNET8_TL_MID
   if (P == 1) {
     if (threadIdx.x == 0) y[j] = r;
+    KNET8_TL_END
     return;
   }
   if (threadIdx.x == 0) st_coherent(partial + j * P + p, r);
-  if (!last_block_ticket(counters + j * kTicketStride, P, &flag)) return;
+  if (!last_block_ticket(counters + j * kTicketStride, P, &flag)) { KNET8_TL_END return; }
   T s = Op::init();
   for (unsigned q = threadIdx.x; q < P; q += BT) s = Op::merge(s, ld_coherent(partial + j * P + q));
   s = block_reduce<T, NW>(s, lds, MergeFn<Op, T>(), Op::init());
@@ -108,6 +111,7 @@ __global__ __launch_bounds__(BT) void reduce_run_kernel(const T* __restrict__ x,
     y[j] = s;
     st_coherent(counters + j * kTicketStride, 0u);
   }
+  KNET8_TL_END
 }
 
 // ---- strided view --------------------------------------------------------------------------------
@@ -163,7 +167,8 @@ constexpr int kCombineU = 8;
 
 template <typename T, typename Op, int NV, int BT, int U, bool SC = false>
 __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict__ x, long s1, long d, long atiles, long kchunk,
-                                                                   unsigned P, T* __restrict__ y, T* partial, unsigned* counters) {
+                                                                   unsigned P, T* __restrict__ y, T* partial, unsigned* counters KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   constexpr int TILE = kWave * NV;
   constexpr int NW = BT / kWave;
   __shared__ T lds[NW][TILE];
@@ -187,6 +192,7 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
 #pragma unroll
   for (int e = 0; e < NV; e++) acc[e] = Op::init();
   if (livemask) strided_walk<T, Op, NV, true, NW, U, SC>(x + b * s1 * d + a0, s1, k0, k1, wave, acc, livemask);
+  KNET8_TL_MID
   if (P > 1) {
     // partial tile p of this group = this workgroup's reduction over its k range
 #pragma unroll
@@ -198,7 +204,7 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
       for (int w = 0; w < NW; w++) r = Op::merge(r, lds[w][threadIdx.x]);
       st_coherent(partial + (group * P + p) * TILE + threadIdx.x, r);
     }
-    if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) return;
+    if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) { KNET8_TL_END return; }
 #pragma unroll
     for (int e = 0; e < NV; e++) acc[e] = Op::init();
     strided_walk<T, Op, NV, false, NW, kCombineU, SC>(partial + group * P * TILE + (SC ? lane : lane * NV), TILE, 0, P, wave, acc);
@@ -214,6 +220,7 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
     for (int w = 0; w < NW; w++) r = Op::merge(r, lds[w][threadIdx.x]);
     y[b * s1 + a] = r;
   }
+  KNET8_TL_END
 }
 
 // ---- stretches of short runs ------------------------------------------------------------------------
@@ -362,9 +369,11 @@ constexpr long kStretchMaxRun = 1024;   // longest run the stretch kernel takes
 
 // Stretch kernel for x(sy, ny, no) -> y(ny) per batch (nb batches, `batch_stride` elements apart, outputs ny apart); sy*ny small enough for
 // whole slabs (R >= 1 of them per stretch) or sy <= kStretchMaxRun.  Returns false if the shape is not one for it.
+// `launched` (if given) is set to false when the shape was this kernel's but its split could not get scratch: nothing was written to y.
 template <typename T, typename Op>
 inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long ny, long no, long nb, long batch_stride, T* y,
-                                  const ScratchSource* scratch) {
+                                  const ScratchSource* scratch, bool* launched = nullptr) {
+  if (launched) *launched = true;
   constexpr int N = Vec16<T>::N;
   constexpr int U1 = 4, UV = 2;      // accesses per lane and stretch, scalar and vector kernels
   constexpr int S1 = 16, SV = 4;     // the same for launches of one stretch per workgroup (one slab of short runs)
@@ -414,7 +423,7 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
     ws = take_scratch(scratch, stream, sizeof(T) * (size_t)groups * P * g, (size_t)groups * kTicketStride);
-    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return true;
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) { if (launched) *launched = false; return true; }
   }
   const dim3 grid((unsigned)(groups * P));
 #define KNET8_STRETCH(NV, U, O) \
@@ -426,30 +435,37 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   return true;
 }
 
+// Both launchers return false when a launch that had to be split could not get its scratch memory: the error is recorded, nothing was
+// launched and y is untouched.
 template <typename T, typename Op>
-inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr, size_t front = 0);
+inline bool launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch = nullptr, size_t front = 0);
+
+// The slab sums of the two-pass route below live in scratch memory (sy*ny elements): beyond this size the route is not taken, so that one
+// odd call cannot pin hundreds of megabytes for as long as its stream lives.
+constexpr size_t kTwoPassMaxBytes = size_t(32) << 20;
 
 template <typename T, typename Op>
-inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y, const ScratchSource* scratch = nullptr) {
-  if (ny <= 0) return;
+inline bool launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, long no, T* y, const ScratchSource* scratch = nullptr) {
+  if (ny <= 0) return true;
   // Short runs.  One slab (a (2, 16M) matrix summed over its columns): one run per workgroup would read a few bytes per lane (3.5 ms); stretches of
   // neighbouring runs instead.  Many slabs (the bias gradient of a 7x7 feature map, x(49, 2048, N)): the slabs are first added onto each other as
   // rows of sy*ny contiguous elements by the strided-view kernel, into scratch, then the sy*ny sums are reduced as one slab; the sy*ny extra
   // elements written and read are nothing next to the no slabs.  (Measured, 134 MB fp32: (4,1000,8388) 158 -> 26.5 us, (49,2048,334) 43.7 -> 28.5 us, (16,16,131072) 35.9 -> 29.0 us.)
   const size_t front = (sizeof(T) * (size_t)(sy * ny) + 255) / 256 * 256;
-  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave && scratch_fits(scratch, 2 * front, 0)) {
+  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave && front <= kTwoPassMaxBytes && scratch_fits(scratch, 2 * front, 0)) {
     Workspace tw = take_scratch(scratch, stream, front, 0);
-    if (tw.partial == nullptr) { record_error("reduction: no scratch memory for the slab sums"); return; }
+    if (tw.partial == nullptr) { record_error("reduction: no scratch memory for the slab sums"); return false; }
     T* tmp = static_cast<T*>(tw.partial);
-    launch_reduce_strided<T, Op>(stream, x, sy * ny, no, 1, tmp, scratch, front);
-    launch_reduce_run<T, typename Op::Merged>(stream, tmp, sy, ny, 1, y, scratch);
-    return;
+    // the second pass reads what the first wrote: it must not run on scratch the first pass never filled
+    if (!launch_reduce_strided<T, Op>(stream, x, sy * ny, no, 1, tmp, scratch, front)) return false;
+    return launch_reduce_run<T, typename Op::Merged>(stream, tmp, sy, ny, 1, y, scratch);
   }
   // (one slab: up to 256-element runs, measured against the run kernel below -- 129: 39 against 195 us, 256: 29.6 / 30.8, 384: 34 / 21.6 --, and up to
   //  1024 when the runs do not start on 16-byte boundaries, where the run kernel is down to 4-byte loads: 513: 39 against 56 us)
   constexpr int NR = Vec16<T>::N;
   const bool short_one_slab = no == 1 && (sy <= 256 || (sy <= kStretchMaxRun && (sy % NR != 0 || !aligned16(x))));
-  if (ny > 1 && (sy <= 8 || short_one_slab) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch)) return;
+  bool launched = true;
+  if (ny > 1 && (sy <= 8 || short_one_slab) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch, &launched)) return launched;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;
@@ -461,14 +477,14 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
     ws = take_scratch(scratch, stream, sizeof(T) * (size_t)ny * P, (size_t)ny * kTicketStride);
-    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return false;
   }
   T* partial = static_cast<T*>(ws.partial);
   // workgroup size by the work of one part: a wave for short runs, 512 lanes when there is plenty
   const int bt = chunk <= 2 * kWave ? 64 : chunk <= 4096 ? 256 : 512;
   const dim3 grid((unsigned)(ny * P));
 #define KNET8_RUN(NV, SINGLE, BT, U) \
-  hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE, BT, U>), grid, dim3(BT), 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters)
+  hipLaunchKernelGGL((reduce_run_kernel<T, Op, NV, SINGLE, BT, U>), grid, dim3(BT), 0, stream, x, sy, ny, units, chunk, P, y, partial, ws.counters KNET8_TL_ARG)
   // (the scalar path, for runs that do not start on 16-byte boundaries, keeps four times as many loads in flight per lane to move the same bytes)
 #define KNET8_RUN_BT(NV, SINGLE) \
   do { if (bt == 64) KNET8_RUN(NV, SINGLE, 64, (NV == 1 ? 16 : 8)); else if (bt == 256) KNET8_RUN(NV, SINGLE, 256, (NV == 1 ? 16 : 4)); \
@@ -477,15 +493,17 @@ inline void launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   else     { if (no == 1) KNET8_RUN_BT(1, true); else KNET8_RUN_BT(1, false); }
 #undef KNET8_RUN_BT
 #undef KNET8_RUN
+  return true;
 }
 
 // `front`: bytes at the start of the scratch memory that belong to the caller (the partial results go behind them).
 template <typename T, typename Op>
-inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch, size_t front) {
-  if (s1 <= 0 || nb <= 0) return;
+inline bool launch_reduce_strided(hipStream_t stream, const T* x, long s1, long d, long nb, T* y, const ScratchSource* scratch, size_t front) {
+  if (s1 <= 0 || nb <= 0) return true;
   constexpr int N = Vec16<T>::N;
   // a short contiguous axis: lanes along `a` alone would idle most of a wave; whole (s1 x R) slabs per stretch instead
-  if (s1 < kWave && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch)) return;
+  bool launched = true;
+  if (s1 < kWave && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch, &launched)) return launched;
   const bool vec = aligned16(x) && (s1 % N == 0);
   // rows that do not start on 16-byte boundaries: the same tile width from N interleaved 4- or 8-byte loads per lane
   const long tile = (long)kWave * N;
@@ -498,16 +516,17 @@ inline void launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   Workspace ws = {nullptr, nullptr};
   if (P > 1) {
     ws = take_scratch(scratch, stream, front + sizeof(T) * (size_t)groups * P * tile, (size_t)groups * kTicketStride);
-    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return;
+    if (!scratch_ready(ws, "reduction: no scratch memory for a split launch")) return false;
   }
   const dim3 grid((unsigned)(groups * P));
   T* partial = reinterpret_cast<T*>(static_cast<char*>(ws.partial) + (ws.partial ? front : 0));
   const bool big = kchunk >= 128;  // sixteen waves share a tile when each still gets >= 8 rows
 #define KNET8_STR(NV, BT, U, SC) \
-  hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U, SC>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters)
+  hipLaunchKernelGGL((reduce_strided_kernel<T, Op, NV, BT, U, SC>), grid, dim3(BT), 0, stream, x, s1, d, atiles, kchunk, P, y, partial, ws.counters KNET8_TL_ARG)
   if (vec) { if (big) KNET8_STR(N, 1024, 2, false); else KNET8_STR(N, 256, 8, false); }
   else     { if (big) KNET8_STR(N, 1024, 2, true); else KNET8_STR(N, 256, 8, true); }
 #undef KNET8_STR
+  return true;
 }
 
 // `_21` contract: x[i] goes into y[(i/sy)%ny]  (src/libknet8/cuda21.jl:23).

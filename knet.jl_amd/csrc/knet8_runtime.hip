@@ -6,6 +6,7 @@
 
 #include <hipblaslt/hipblaslt.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <map>
@@ -41,6 +42,23 @@ static bool ok(hipError_t e, const char* what) {
   std::string msg = std::string(what) + ": " + hipGetErrorString(e);
   record_error(msg.c_str());
   return false;
+}
+
+// ---- every device allocation and release of the library goes through these two, which count the calls (knet8_stats): a test can
+// then assert that an entry point that promises not to allocate made none.
+static std::atomic<unsigned long long> g_malloc_calls{0}, g_free_calls{0};
+static std::atomic<unsigned long long> g_held_bytes{0};         // scratch, workspaces and scalar slots the library holds outside the pool
+static std::atomic<unsigned long long> g_gemm_left_vendor{0};   // plain products that ran on the library's own tiles because hipBLASLt had no algorithm
+static hipError_t dev_malloc(void** p, size_t n, bool held = false) {
+  g_malloc_calls.fetch_add(1, std::memory_order_relaxed);
+  const hipError_t e = hipMalloc(p, n);
+  if (held && e == hipSuccess) g_held_bytes.fetch_add(n, std::memory_order_relaxed);
+  return e;
+}
+static void dev_free(void* p, size_t held_bytes = 0) {
+  g_free_calls.fetch_add(1, std::memory_order_relaxed);
+  g_held_bytes.fetch_sub(held_bytes, std::memory_order_relaxed);
+  (void)hipFree(p);
 }
 
 // ---- launch-heuristic knobs ------------------------------------------------------------------------------
@@ -87,6 +105,8 @@ struct StreamScratch {
   unsigned* counters = nullptr;
   size_t ncounters = 0;
   std::vector<void*> retired;
+  std::vector<size_t> retired_bytes;
+  bool in_graph = false;   // handed out while the stream was being captured: a graph holds the addresses, so knet8_trim leaves them alone
   hipEvent_t t0 = nullptr, t1 = nullptr;
 };
 static std::mutex g_scratch_mutex;
@@ -96,6 +116,30 @@ static StreamScratch& scratch_of(hipStream_t stream) {
   int dev = 0;
   (void)hipGetDevice(&dev);
   return g_scratch[std::make_pair(dev, stream)];
+}
+
+static bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (stream == nullptr || hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return cap != hipStreamCaptureStatusNone;
+}
+
+// hipBLASLt workspaces, one per (device, stream), defined with the GEMM entry points below: release the one of a stream that is being
+// destroyed, or (every = true) all that no captured graph holds; returns the bytes released.
+static size_t gemm_release(int dev, hipStream_t stream, bool every);
+
+static size_t release_scratch(StreamScratch& s) {
+  size_t released = s.partial_bytes + s.ncounters * sizeof(unsigned);
+  if (s.partial) dev_free(s.partial, s.partial_bytes);
+  if (s.counters) dev_free(s.counters, s.ncounters * sizeof(unsigned));
+  for (size_t i = 0; i < s.retired.size(); i++) { dev_free(s.retired[i], s.retired_bytes[i]); released += s.retired_bytes[i]; }
+  s.partial = nullptr; s.partial_bytes = 0;
+  s.counters = nullptr; s.ncounters = 0;
+  s.retired.clear(); s.retired_bytes.clear();
+  return released;
 }
 
 __global__ __launch_bounds__(256) void zero_counters_kernel(unsigned* c, size_t n) {
@@ -109,19 +153,21 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
     Workspace none = {nullptr, nullptr};
     return none;
   }
+  const bool capturing = stream_is_capturing(stream);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   StreamScratch& s = scratch_of(stream);
+  if (capturing) s.in_graph = true;
   // Buffers that have become too small are retired, not freed: launches already queued on the stream, and graphs
   // captured on it, keep using their addresses.  Sizes grow geometrically, so the retired ones add up to less than
-  // the current one.
+  // the current one.  knet8_trim (after a device-wide wait) and knet8_stream_destroy release them.
   if (s.partial_bytes < partial_bytes) {
-    if (s.partial) s.retired.push_back(s.partial);
+    if (s.partial) { s.retired.push_back(s.partial); s.retired_bytes.push_back(s.partial_bytes); }
     size_t want = partial_bytes < (size_t(1) << 20) ? (size_t(1) << 20) : 2 * partial_bytes;
     s.partial = nullptr;
-    s.partial_bytes = ok(hipMalloc(&s.partial, want), "hipMalloc(reduction partials)") ? want : 0;
+    s.partial_bytes = ok(dev_malloc(&s.partial, want, true), "hipMalloc(reduction partials)") ? want : 0;
   }
   if (s.ncounters < ncounters) {
-    if (s.counters) s.retired.push_back(s.counters);
+    if (s.counters) { s.retired.push_back(s.counters); s.retired_bytes.push_back(s.ncounters * sizeof(unsigned)); }
     size_t want = ncounters < 4096 ? 4096 : 2 * ncounters;
     s.counters = nullptr;
     s.ncounters = 0;
@@ -129,7 +175,7 @@ Workspace workspace_for(hipStream_t stream, size_t partial_bytes, size_t ncounte
     // use the counters.  (A hipMemset goes to the null stream, which a non-blocking stream does not wait for: on recycled memory
     // the first split kernel on a new stream could then count on top of garbage and leave its tickets non-zero for good.  A fill
     // kernel is also what a stream capture can record safely.)
-    if (ok(hipMalloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned)), "hipMalloc(reduction counters)")) {
+    if (ok(dev_malloc(reinterpret_cast<void**>(&s.counters), want * sizeof(unsigned), true), "hipMalloc(reduction counters)")) {
       hipLaunchKernelGGL(zero_counters_kernel, dim3((unsigned)((want + 255) / 256)), dim3(256), 0, stream, s.counters, want);
       if (ok(hipGetLastError(), "zero_counters_kernel")) s.ncounters = want;
     }
@@ -196,7 +242,7 @@ void* scalar_slot(hipStream_t stream) {
   int dev = 0;
   (void)hipGetDevice(&dev);
   void*& p = slots[std::make_pair(dev, stream)];
-  if (!p && !ok(hipMalloc(&p, 256), "hipMalloc(scalar slot)")) p = nullptr;
+  if (!p && !ok(dev_malloc(&p, 256, true), "hipMalloc(scalar slot)")) p = nullptr;
   return p;
 }
 
@@ -231,9 +277,9 @@ static Pool g_pool;
 constexpr size_t kColorPeriod = 16384, kColorStep = 21 * 256, kColorMinBytes = size_t(1) << 20;
 
 static hipError_t pool_device_malloc(Pool& pool, void** out, size_t sz) {
-  if (sz < kColorMinBytes) return hipMalloc(out, sz);
+  if (sz < kColorMinBytes) return dev_malloc(out, sz);
   void* base = nullptr;
-  const hipError_t e = hipMalloc(&base, sz + kColorPeriod);
+  const hipError_t e = dev_malloc(&base, sz + kColorPeriod);
   if (e != hipSuccess) return e;
   const size_t want = (pool.next_color++ * kColorStep) % kColorPeriod;
   const size_t have = reinterpret_cast<uintptr_t>(base) % kColorPeriod;
@@ -246,10 +292,10 @@ static hipError_t pool_device_malloc(Pool& pool, void** out, size_t sz) {
 static void pool_device_free(Pool& pool, void* p) {
   auto it = pool.base_of.find(p);
   if (it != pool.base_of.end()) {
-    (void)hipFree(it->second);
+    dev_free(it->second);
     pool.base_of.erase(it);
   } else {
-    (void)hipFree(p);
+    dev_free(p);
   }
 }
 
@@ -328,8 +374,32 @@ KNET8_API void knet8_free(void* ptr) {
 
 KNET8_API size_t knet8_trim(void) {
   (void)hipDeviceSynchronize();
-  std::lock_guard<std::mutex> lock(g_pool.mutex);
-  return trim_locked(g_pool);
+  size_t released = 0;
+  {
+    std::lock_guard<std::mutex> lock(g_pool.mutex);
+    released += trim_locked(g_pool);
+  }
+  // Nothing is queued any more: the reduction scratch of every stream (current and retired buffers) and the hipBLASLt workspaces go back
+  // too, except those a captured graph may still name (handed out while their stream was being captured); the next launch that needs
+  // scratch allocates it afresh.
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    for (auto& kv : g_scratch)
+      if (!kv.second.in_graph) released += release_scratch(kv.second);
+  }
+  released += gemm_release(0, nullptr, true);
+  return released;
+}
+
+KNET8_API void knet8_stats(unsigned long long* out6) {
+  size_t free_b = 0, total_b = 0;
+  if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) { (void)hipGetLastError(); free_b = total_b = 0; }
+  out6[0] = g_malloc_calls.load();
+  out6[1] = g_free_calls.load();
+  out6[2] = g_held_bytes.load();
+  out6[3] = g_gemm_left_vendor.load();
+  out6[4] = free_b;
+  out6[5] = total_b;
 }
 
 KNET8_API void knet8_meminfo(size_t* out4) {
@@ -383,13 +453,12 @@ KNET8_API void knet8_stream_destroy(hipStream_t stream) {
     auto it = g_scratch.find(std::make_pair(dev, stream));
     if (it != g_scratch.end()) {
       StreamScratch& s = it->second;
-      if (s.partial) (void)hipFree(s.partial);
-      if (s.counters) (void)hipFree(s.counters);
-      for (void* p : s.retired) (void)hipFree(p);
+      release_scratch(s);
       if (s.t0) (void)hipEventDestroy(s.t0);
       if (s.t1) (void)hipEventDestroy(s.t1);
       g_scratch.erase(it);
     }
+    gemm_release(dev, stream, false);   // the stream's hipBLASLt workspace: a later stream with the same handle starts without one
   }
   ok(hipStreamDestroy(stream), "hipStreamDestroy");
 }
@@ -500,6 +569,12 @@ KNET8_API void knet8_seed(unsigned long long seed) {
   g_rng_seeded = true;
 }
 
+#ifdef KNET8_TIMELINE
+// Measurement build only: the device buffer (kTlSlots stamps of 32 bytes) the stamped kernels write to from now on; null switches the stamps off.
+static knet8::TlStamp* g_timeline = nullptr;
+KNET8_API void knet8_timeline_set(void* buffer) { g_timeline = static_cast<knet8::TlStamp*>(buffer); }
+#endif
+
 KNET8_API int knet8_tune(int key, int value) {
   if (key < 0 || key >= kTuneCount) return -1;
   const int old = g_tune[key];
@@ -511,6 +586,10 @@ KNET8_API int knet8_tune(int key, int value) {
 
 // ---- GEMM through hipBLASLt ----------------------------------------------------------------------------------
 namespace knet8 {
+
+#ifdef KNET8_TIMELINE
+TlStamp* timeline_buffer() { return g_timeline; }
+#endif
 
 struct GemmBatch {   // strided batch: product b uses A + b*sa, B + b*sb, C + b*sc (elements)
   int count = 1;
@@ -533,11 +612,52 @@ struct GemmPlan {
   bool timed = false;        // the algorithm was chosen by timing the candidates (not possible while the stream is being captured)
   bool unsupported = false;  // the vendor library has no kernel for this problem with this epilogue: callers take the separate bias pass
 };
+struct GemmWs {
+  void* p = nullptr;
+  bool in_graph = false;   // used by a product recorded into a graph: knet8_trim leaves it alone
+};
 static std::mutex g_gemm_mutex;
 static std::map<int, hipblasLtHandle_t> g_lt;
 static std::map<GemmKey, GemmPlan> g_plans;
-static std::map<std::pair<int, hipStream_t>, void*> g_gemm_ws;
+static std::map<std::pair<int, hipStream_t>, GemmWs> g_gemm_ws;
 static const size_t kGemmWorkspace = size_t(64) << 20;
+// Bumped whenever a workspace is released: the per-thread shortcut below then forgets what it remembered.
+static std::atomic<unsigned long long> g_gemm_generation{1};
+
+static size_t gemm_release(int dev, hipStream_t stream, bool every) {
+  std::lock_guard<std::mutex> lock(g_gemm_mutex);
+  size_t released = 0;
+  for (auto it = g_gemm_ws.begin(); it != g_gemm_ws.end();) {
+    const bool hit = every ? !it->second.in_graph : (it->first.first == dev && it->first.second == stream);
+    if (hit) {
+      if (it->second.p) { dev_free(it->second.p, kGemmWorkspace); released += kGemmWorkspace; }
+      it = g_gemm_ws.erase(it);
+    } else {
+      ++it;
+    }
+  }
+  if (released) g_gemm_generation.fetch_add(1);
+  return released;
+}
+
+// The last few plain products of this thread: problem, stream, and everything the vendor call needs.  A repeat (the same layer of the
+// same model in the next step) goes straight to hipblasLtMatmul: no map lookups, no capture query, the lock held for the vendor call only.  Only plans that are final
+// (algorithm chosen by timing) and carry no bias pointer are remembered; the plans themselves are never destroyed once valid.
+struct GemmRecent {
+  GemmKey key;
+  hipStream_t stream;
+  const GemmPlan* plan;
+  hipblasLtHandle_t handle;
+  void* ws;
+  unsigned long long generation = 0;   // 0: empty
+};
+constexpr int kGemmRecent = 8;
+static thread_local GemmRecent t_recent[kGemmRecent];
+static thread_local int t_recent_next = 0;
+static bool same_key(const GemmKey& a, const GemmKey& b) {
+  return a.m == b.m && a.n == b.n && a.k == b.k && a.ta == b.ta && a.tb == b.tb && a.lda == b.lda && a.ldb == b.ldb && a.ldc == b.ldc && a.dtype == b.dtype &&
+         a.dev == b.dev && a.batch == b.batch && a.epilogue == b.epilogue && a.sa == b.sa && a.sb == b.sb && a.sc == b.sc;
+}
 
 static bool lt_ok(hipblasStatus_t s, const char* what) {
   if (s == HIPBLAS_STATUS_SUCCESS) return true;
@@ -557,7 +677,9 @@ static void destroy_plan(GemmPlan& p) {
 
 // bias != nullptr / act != 0: the dense-layer form C = act(alpha*op(A)*op(B) + bias[i]) (beta must be 0).
 struct EpiNone { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb; } };
-struct EpiRelu { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb != zb ? zb : (zb > T(0) ? zb : T(0)); } };
+// relu of gemm_bias_act_S: z > 0 ? z : 0 -- what hipBLASLt's RELU_BIAS output stage computes and what the reference's device relu computes
+// (src/libknet8/ops.jl:63), so that a NaN comes out as 0 whichever route the product takes.
+struct EpiRelu { template <typename T> __device__ __forceinline__ T operator()(T zb, T) const { return zb > T(0) ? zb : T(0); } };
 
 enum { kEpiNone = 0, kEpiBias = 1, kEpiReluBias = 2 };
 constexpr int kGemmNoFusedForm = 2;   // gemm_lt: the vendor library has no kernel for this problem (with this epilogue); nothing was launched
@@ -571,17 +693,32 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
   const hipblasComputeType_t ct = sizeof(T) == 4 ? HIPBLAS_COMPUTE_32F : HIPBLAS_COMPUTE_64F;
   int dev = 0;
   (void)hipGetDevice(&dev);
+  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, epilogue, batch.sa, batch.sb, batch.sc};
+  const bool dry = g_tune[kTuneGemmDryRun] != 0;   // measurements of the library's own share of a call: everything but the vendor call
+  if (epilogue == kEpiNone) {
+    const unsigned long long gen = g_gemm_generation.load(std::memory_order_acquire);
+    for (int i = 0; i < kGemmRecent; i++) {
+      const GemmRecent& r = t_recent[i];
+      if (r.generation == gen && r.stream == stream && same_key(r.key, key)) {
+        if (dry) return 0;
+        // (the vendor call itself stays under the lock: concurrent hipblasLtMatmul calls on one handle from several host threads gave wrong
+        //  products in the library's own multi-thread test)
+        std::lock_guard<std::mutex> lock(g_gemm_mutex);
+        return lt_ok(hipblasLtMatmul(r.handle, r.plan->desc, &alpha, A, r.plan->la, B, r.plan->lb, &beta, C, r.plan->lc, C, r.plan->lc, &r.plan->algo, r.ws,
+                                     kGemmWorkspace, stream), "matmul") ? 0 : -1;
+      }
+    }
+  }
+  const bool capturing = stream_is_capturing(stream);
   std::lock_guard<std::mutex> lock(g_gemm_mutex);
   hipblasLtHandle_t& h = g_lt[dev];
   if (!h && !lt_ok(hipblasLtCreate(&h), "create")) return -1;
-  void*& ws = g_gemm_ws[std::make_pair(dev, stream)];
-  if (!ws && !ok(hipMalloc(&ws, kGemmWorkspace), "hipMalloc(gemm workspace)")) return -1;
-  const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, epilogue, batch.sa, batch.sb, batch.sc};
+  GemmWs& wsrec = g_gemm_ws[std::make_pair(dev, stream)];
+  if (!wsrec.p && !ok(dev_malloc(&wsrec.p, kGemmWorkspace, true), "hipMalloc(gemm workspace)")) return -1;
+  if (capturing) wsrec.in_graph = true;
+  void* const ws = wsrec.p;
   GemmPlan& p = g_plans[key];
   if (p.unsupported) return kGemmNoFusedForm;
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (stream) (void)hipStreamIsCapturing(stream, &cap);
-  const bool capturing = cap != hipStreamCaptureStatusNone;
   // A plan whose creation fails half way is taken out of the cache again: the next call must not find a descriptor without layouts.
   auto fail = [&]() { destroy_plan(p); g_plans.erase(key); return -1; };
   if (!p.desc) {
@@ -630,7 +767,11 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
     int found = 0;
     const hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(h, p.desc, p.la, p.lb, p.lc, p.lc, pref, kCand, res, &found);
     hipblasLtMatmulPreferenceDestroy(pref);
-    if (hs != HIPBLAS_STATUS_SUCCESS || found < 1) {
+    if (hs != HIPBLAS_STATUS_SUCCESS && hs != HIPBLAS_STATUS_NOT_SUPPORTED) {   // a failure of the query itself is an error, not "no kernel"
+      lt_ok(hs, "algorithm query");
+      return fail();
+    }
+    if (hs == HIPBLAS_STATUS_NOT_SUPPORTED || found < 1) {
       destroy_plan(p);   // not an error: the caller falls back on the library's own product kernels, and remembers it
       p.unsupported = true;
       return kGemmNoFusedForm;
@@ -666,6 +807,13 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
     p.valid = true;
     p.timed = can_time;
   }
+  if (epilogue == kEpiNone && p.timed && !capturing) {
+    GemmRecent& r = t_recent[t_recent_next];
+    t_recent_next = (t_recent_next + 1) % kGemmRecent;
+    r.key = key; r.stream = stream; r.plan = &p; r.handle = h; r.ws = ws;
+    r.generation = g_gemm_generation.load(std::memory_order_acquire);
+  }
+  if (dry) return 0;
   return lt_ok(hipblasLtMatmul(h, p.desc, &alpha, A, p.la, B, p.lb, &beta, C, p.lc, C, p.lc, &p.algo, ws, kGemmWorkspace, stream), "matmul") ? 0 : -1;
 }
 
@@ -676,11 +824,14 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
   const bool ta = (transa == 'T' || transa == 't' || transa == 'C' || transa == 'c');
   const bool tb = (transb == 'T' || transb == 't' || transb == 'C' || transb == 'c');
   if (batch.count > 1 && (bias || act)) { record_error("gemm: the bias/activation form takes no batch"); return -1; }
-  if ((long long)m * n >= (1LL << 31) || (long long)m * k >= (1LL << 31) || (long long)k * n >= (1LL << 31)) {
-    record_error("gemm: an operand has 2^31 or more elements; the 32-bit indices of the library's kernels do not reach that far");
-    return -1;
-  }
+  // The library's own kernels index their operands with 32 bits; the vendor route (64-bit layouts) has no such limit.
+  auto own_kernels_reach = [&]() {
+    if ((long long)m * n < (1LL << 31) && (long long)m * k < (1LL << 31) && (long long)k * n < (1LL << 31)) return true;
+    record_error("gemm: an operand has 2^31 or more elements; the 32-bit indices of the library's own kernels do not reach that far");
+    return false;
+  };
   if (batch.count == 1 && (k <= 0 || gemm_is_small(m, n, k))) {   // empty products (C = beta*C [+ bias]), and small ones when a caller has opted in (knet8_tune key 3)
+    if (!own_kernels_reach()) return -1;
     launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias, act);
     check_launch("gemm (small)");
     return 0;
@@ -690,6 +841,8 @@ static int gemm(char transa, char transb, int m, int n, int k, T alpha, const T*
     int rc = gemm_lt<T>(ta, tb, m, n, k, alpha, A, lda, B, ldb, bt, C, ldc, stream, kEpiNone, nullptr, batch);
     if (rc != kGemmNoFusedForm) return rc;
     if (batch.count > 1) { record_error("hipBLASLt: no algorithm for this batched product"); return -1; }
+    if (!own_kernels_reach()) return -1;
+    g_gemm_left_vendor.fetch_add(1, std::memory_order_relaxed);
     launch_gemm_small<T>(stream, ta, tb, m, n, k, alpha, A, lda, B, ldb, bt, C, ldc, nullptr, 0);
     check_launch("gemm (own kernel: no vendor algorithm)");
     return 0;

@@ -116,7 +116,8 @@ __device__ __forceinline__ void cut_column(const T* p, int m, int& head, int& nb
 // registers alone it takes the whole register file of a compute unit -- one workgroup per CU, two rounds of workgroups for 512 columns; with 512
 // lanes holding 23 vectors in registers and 9 in LDS each (72 KB per workgroup), two columns are resident per CU.
 template <typename T, typename Algo, int TEAM, int E, bool VEC, int LV>
-__device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, const T* b, T* out) {
+__device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, const T* b, T* out KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   // Short columns (one wave each, few registers): load every input up front even if it is only needed for the
   // output pass, so the dependent chain is one memory round trip instead of two.
   constexpr bool kHold = Algo::kHoldA || (TEAM == kWave && E <= 16);
@@ -219,6 +220,7 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
   if (tv) { const T t = Algo::term(at, bt, mx); if constexpr (Algo::kKeepTerm) at = t; s = s + t; }
   s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
   const T fin = Algo::finish(s);
+  KNET8_TL_MID
 #pragma unroll
   for (int i = 0; i < ITEMS; i++) {
     if (i >= cnt) continue;
@@ -248,16 +250,17 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
     if (hv) { if constexpr (Algo::kKeepTerm) oc[tl] = Algo::out_kept(ah, fin); else oc[tl] = Algo::out(ah, bh, mx, fin); }
     if (tv) { if constexpr (Algo::kKeepTerm) oc[tpos] = Algo::out_kept(at, fin); else oc[tpos] = Algo::out(at, bt, mx, fin); }
   }
+  KNET8_TL_END
 }
 
 template <typename T, typename Algo, int TEAM, int E, bool VEC>
-__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out) {
-  softmax_col_body<T, Algo, TEAM, E, VEC, 0>(m, n, a, b, out);
+__global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void softmax_col_kernel(int m, long n, const T* a, const T* b, T* out KNET8_TL_PARAM) {
+  softmax_col_body<T, Algo, TEAM, E, VEC, 0>(m, n, a, b, out KNET8_TL_PASS);
 }
 // four waves per SIMD (two 512-lane workgroups per compute unit): at most 128 registers per lane
 template <typename T, typename Algo, int TEAM, int E, int LV>
 __global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) void softmax_col_lds_kernel(int m, long n, const T* a, const T* b, T* out) {
-  softmax_col_body<T, Algo, TEAM, E, true, LV>(m, n, a, b, out);
+  softmax_col_body<T, Algo, TEAM, E, true, LV>(m, n, a, b, out KNET8_TL_NONE);
 }
 
 // ---- fused nll + logsoftmax backward, register-resident, single reduction ---------------------------------
@@ -288,7 +291,8 @@ template <typename T> __device__ __forceinline__ MaxSum<T> ms_wave_reduce(MaxSum
 // fished out of the register that happens to hold it.  Columns are cut into head / vectors / tail as in softmax_col_kernel.
 // LV > 0: the last LV vectors of each lane live in LDS, as in softmax_col_body.
 template <typename T, int TEAM, int E, bool VEC, int LV>
-__device__ __forceinline__ void nll_col_body(int m, long n, const T* a, T* out, const int* labels, T scale, T* loss) {
+__device__ __forceinline__ void nll_col_body(int m, long n, const T* a, T* out, const int* labels, T scale, T* loss KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   constexpr int BT = TEAM == kWave ? kWaveTeamBlock : TEAM;
   constexpr int TEAMS = BT / TEAM;
   constexpr int NW = TEAM / kWave;
@@ -390,6 +394,7 @@ __device__ __forceinline__ void nll_col_body(int m, long n, const T* a, T* out, 
   // softmax_i = e_i * exp(m_t - M) / S; fold the upstream scale in: one multiply per element
   const T f = (mt == ninf ? T(0) : dev_exp(mt - ms.m) / ms.s) * scale;
   if (colok && tl == 0) loss[col] = lab > 0 ? -((alab - ms.m) - logS) : T(0);
+  KNET8_TL_MID
 #pragma unroll
   for (int i = 0; i < ITEMS; i++) {
     if (i >= cnt) continue;
@@ -411,18 +416,19 @@ __device__ __forceinline__ void nll_col_body(int m, long n, const T* a, T* out, 
     if (hv) oc[tl] = lab == 0 ? T(0) : ((tl + 1 == lab) ? -scale : T(0)) + xh * f;
     if (tv) oc[tpos] = lab == 0 ? T(0) : ((tpos + 1 == lab) ? -scale : T(0)) + xt * f;
   }
+  KNET8_TL_END
 }
 
 template <typename T, int TEAM, int E, bool VEC>
 __global__ __launch_bounds__(TEAM == kWave ? kWaveTeamBlock : TEAM) void nll_col_kernel(int m, long n, const T* a, T* out, const int* labels,
-                                                                            T scale, T* loss) {
-  nll_col_body<T, TEAM, E, VEC, 0>(m, n, a, out, labels, scale, loss);
+                                                                            T scale, T* loss KNET8_TL_PARAM) {
+  nll_col_body<T, TEAM, E, VEC, 0>(m, n, a, out, labels, scale, loss KNET8_TL_PASS);
 }
 // four waves per SIMD (two 512-lane workgroups per compute unit): at most 128 registers per lane
 template <typename T, int TEAM, int E, int LV>
 __global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) void nll_col_lds_kernel(int m, long n, const T* a, T* out,
                                                                                                       const int* labels, T scale, T* loss) {
-  nll_col_body<T, TEAM, E, true, LV>(m, n, a, out, labels, scale, loss);
+  nll_col_body<T, TEAM, E, true, LV>(m, n, a, out, labels, scale, loss KNET8_TL_NONE);
 }
 
 // ---- many short columns -----------------------------------------------------------------------------------
@@ -904,11 +910,11 @@ inline void launch_softmax_cfg(hipStream_t stream, bool vec, int m, long n, cons
   // between them.)
   const dim3 grid((unsigned)((n + TEAMS - 1) / TEAMS));
   if constexpr (Algo::kNll) {
-    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
-    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false>), grid, block, 0, stream, m, n, a, out, labels, scale, loss);
+    if (vec) hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, true>), grid, block, 0, stream, m, n, a, out, labels, scale, loss KNET8_TL_ARG);
+    else hipLaunchKernelGGL((nll_col_kernel<T, TEAM, E, false>), grid, block, 0, stream, m, n, a, out, labels, scale, loss KNET8_TL_ARG);
   } else {
-    if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out);
-    else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out);
+    if (vec) hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, true>), grid, block, 0, stream, m, n, a, b, out KNET8_TL_ARG);
+    else hipLaunchKernelGGL((softmax_col_kernel<T, Algo, TEAM, E, false>), grid, block, 0, stream, m, n, a, b, out KNET8_TL_ARG);
   }
 }
 

@@ -347,7 +347,13 @@ def test_split_launch_without_scratch_is_refused_on_the_host(knet):
         dz = knet.KnetArray(dtype=np.float32, dims=(256, 4096))
         fn["reluback_biasgrad_32_stream"](256, 4096, dyd.ptr, yd.ptr, dz.ptr, out.ptr, lib.stream)
 
-    cases = [(sum_dims2, 256), (sum_all, 1), (sum_small_rows, 8), (bias_grad, 256)]
+    x3 = rng.integers(-3, 4, size=(4, 1000, 50)).astype(np.float32)      # many slabs of short runs: two passes, the slab sums in scratch
+    x3d = knet.KnetArray(x3)
+
+    def sum_two_pass(out):
+        fn["sum_32_21_stream"](x3.size, x3d.ptr, 4, 1000, out.ptr, lib.stream)
+
+    cases = [(sum_dims2, 256), (sum_all, 1), (sum_small_rows, 8), (sum_two_pass, 1000), (bias_grad, 256)]
     assert fn["knet8_tune"](5, 1) == 0
     try:
         for launch, ny in cases:
@@ -359,9 +365,128 @@ def test_split_launch_without_scratch_is_refused_on_the_host(knet):
             assert np.all(knet.Array(out) == sentinel), launch.__name__      # no kernel ran on it
     finally:
         fn["knet8_tune"](5, 0)
-    for launch, ny in cases[:3]:                                             # with the knob back the same calls work
+    for launch, ny in cases[:4]:                                             # with the knob back the same calls work
         out = knet.KnetArray(np.full(ny, sentinel, np.float32))
         launch(out)
-        want = x.sum(axis=1) if ny == 256 else (x.sum() if ny == 1 else x.reshape(-1, order="F").reshape(8, -1, order="F").sum(axis=1))
+        want = {256: lambda: x.sum(axis=1), 1: lambda: x.sum(), 8: lambda: x.reshape(-1, order="F").reshape(8, -1, order="F").sum(axis=1),
+                1000: lambda: x3.sum(axis=(0, 2))}[ny]()
         assert np.array_equal(knet.Array(out).ravel(), np.atleast_1d(want).astype(np.float32)), launch.__name__
     lib.check()
+
+
+def test_two_pass_reduction_whose_first_pass_is_refused_leaves_the_output_alone(knet):
+    """Many slabs of short runs go in two passes (slab sums into scratch, then one slab of short runs).  If the first pass's own split cannot get its
+    scratch after the slab sums got theirs, the second pass must not run on memory the first never filled.  The fixed array of sum_32_21_noalloc
+    makes that reachable: a planner told of 2^20 compute units asks for more partial results than the array holds."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    rng = np.random.default_rng(57)
+    x = rng.integers(-3, 4, size=(4, 2000, 4000)).astype(np.float32)     # first pass: 32 row tiles x 62 parts = 2 MB of partial results
+    xd = knet.KnetArray(x)
+    out = knet.KnetArray(np.full(2000, -777.0, np.float32))
+    old = fn["knet8_tune"](0, 1 << 20)
+    try:
+        fn["sum_32_21_noalloc"](x.size, xd.ptr, 4, 2000, out.ptr, lib.stream)
+        assert fn["knet8_synchronize"](lib.stream) == 0
+        msg = fn["knet8_last_error"]()
+    finally:
+        fn["knet8_tune"](0, old)
+    got = knet.Array(out)
+    want = x.sum(axis=(0, 2)).astype(np.float32)
+    assert msg is not None and b"scratch" in msg, msg
+    assert np.all(got == np.float32(-777.0))        # refused: untouched
+    fn["sum_32_21_noalloc"](x.size, xd.ptr, 4, 2000, out.ptr, lib.stream)
+    knet.synchronize()
+    lib.check()
+    assert np.array_equal(knet.Array(out), want)
+
+
+def test_streams_give_their_memory_back(knet):
+    """Eight streams in a row, each running one product (a 64 MiB hipBLASLt workspace per stream) and one split reduction (partial results and
+    tickets per stream), each destroyed afterwards: the device's free memory returns to where it was (to 8 MiB), and so it does after knet8_trim
+    for a stream that stays alive -- Knet.gc gives memory back (src/knetarrays/kptr.jl:204-226)."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    import ctypes
+
+    def stats():
+        out = (ctypes.c_ulonglong * 6)()
+        fn["knet8_stats"](ctypes.cast(out, ctypes.c_void_p))
+        return dict(zip(("mallocs", "frees", "held", "left_vendor", "free", "total"), out))
+    rng = np.random.default_rng(58)
+    A, B = rng.standard_normal((300, 200)).astype(np.float32), rng.standard_normal((200, 100)).astype(np.float32)
+    x = rng.integers(-3, 4, size=(256, 4096)).astype(np.float32)
+    Ad, Bd, Cd, xd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(np.zeros((300, 100), np.float32)), knet.KnetArray(x)
+    out = knet.KnetArray(np.zeros(256, np.float32))
+    want = A.astype(np.float64) @ B.astype(np.float64)
+
+    def work(stream):
+        assert fn["gemm_32_stream"](b"N", b"N", 300, 100, 200, 1.0, Ad.ptr, 300, Bd.ptr, 200, 0.0, Cd.ptr, 300, stream) == 0
+        fn["sum_32_21_stream"](x.size, xd.ptr, 1, 256, out.ptr, stream)
+        assert fn["knet8_synchronize"](stream) == 0
+        assert np.linalg.norm(knet.Array(Cd) - want) <= 1e-5 * np.linalg.norm(want)
+        assert np.array_equal(knet.Array(out), x.sum(axis=1))
+    s0 = fn["knet8_stream_create"]()
+    work(s0)                      # whatever is created once per process (library handles, code objects) exists from here on
+    fn["knet8_stream_destroy"](s0)
+    fn["knet8_trim"]()
+    st0 = stats()
+    for _ in range(8):
+        s = fn["knet8_stream_create"]()
+        work(s)
+        assert stats()["held"] >= st0["held"] + (64 << 20)       # workspace and scratch are there while the stream lives
+        fn["knet8_stream_destroy"](s)
+        assert stats()["held"] == st0["held"]                    # the library's own books: everything the stream held is released
+    fn["knet8_trim"]()                                           # (waits for the device, so that the driver's figure is settled)
+    st1 = stats()
+    assert st1["mallocs"] - st0["mallocs"] == st1["frees"] - st0["frees"] >= 24
+    # and the driver's books (hipMemGetInfo): eight leaked workspaces would be 512 MiB less.  One-sided: the driver shows some releases late, so the
+    # figure at the start may still count memory that was already given back
+    assert st1["free"] >= st0["free"] - (8 << 20), (st1["free"], st0["free"])
+    s = fn["knet8_stream_create"]()
+    work(s)
+    assert stats()["held"] >= st0["held"] + (64 << 20)
+    assert fn["knet8_trim"]() >= (64 << 20)                      # a live stream's workspace and scratch go back on a trim ...
+    assert stats()["held"] == st0["held"] and stats()["free"] >= st0["free"] - (8 << 20)
+    work(s)                                                      # ... and come back when needed
+    fn["knet8_stream_destroy"](s)
+    fn["knet8_trim"]()
+    assert stats()["held"] == st0["held"]
+    lib.check()
+
+
+def test_products_with_an_operand_of_more_than_2_to_the_31_elements_go_to_the_vendor_route(knet):
+    """A (65536 x 32770) fp32 operand has 2^31 + 131072 elements (8.6 GB): beyond the 32-bit indices of the library's own kernels, and no
+    obstacle for the hipBLASLt route every plain product takes.  A is zero except its last column, which lies wholly beyond element 2^31:
+    C = A*B is then that column times the last row of B."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    m, k, n = 65536, 32770, 4
+    assert m * k > (1 << 31)
+    rng = np.random.default_rng(59)
+    c = rng.standard_normal(m).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    A = fn["knet8_malloc"](m * k * 4)
+    assert A
+    try:
+        half = (m * k) // 2
+        fn["fill_32_stream"](half, 0.0, A, lib.stream)
+        fn["fill_32_stream"](m * k - half, 0.0, A + 4 * half, lib.stream)
+        fn["knet8_memcpy"](A + 4 * m * (k - 1), c.ctypes.data, c.nbytes, 1, lib.stream)
+        Bd, Cd = knet.KnetArray(B), knet.KnetArray(np.full((m, n), 7.0, np.float32))
+        assert fn["gemm_32_stream"](b"N", b"N", m, n, k, 1.0, A, m, Bd.ptr, k, 0.0, Cd.ptr, m, lib.stream) == 0
+        knet.synchronize()
+        lib.check()
+        want = np.outer(c.astype(np.float64), B[k - 1].astype(np.float64))
+        assert np.abs(knet.Array(Cd) - want).max() <= 1e-6 * np.abs(want).max()
+        # the library's own kernels refuse the same operand instead of wrapping their indices
+        old = fn["knet8_tune"](3, 1 << 30)
+        try:
+            assert fn["gemm_32_stream"](b"N", b"N", m, n, k, 1.0, A, m, Bd.ptr, k, 0.0, Cd.ptr, m, lib.stream) == -1
+        finally:
+            fn["knet8_tune"](3, old)
+        assert b"2^31" in fn["knet8_last_error"]()
+    finally:
+        knet.synchronize()
+        fn["knet8_free"](A)
+        fn["knet8_trim"]()

@@ -219,6 +219,45 @@ def test_gemm_bias_act_on_the_own_kernels_carries_the_bits_of_the_three_launch_c
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_gemm_bias_act_treats_nan_and_inf_alike_on_both_routes(knet, dt):
+    """A NaN, a +Inf and a -Inf in A: without activation the rows they touch come out NaN / +-Inf; with relu every route of the entry point --
+    the vendor epilogue (key 3 = 0) and the library's own kernels (key 3 = 270) -- computes z > 0 ? z : 0, the device relu of the reference
+    (src/libknet8/ops.jl:63): the NaN row becomes 0, +Inf stays, -Inf becomes 0.  (relu_S, which follows the CPU path, keeps a NaN.)"""
+    lib = knet.libknet8()
+    fn = lib.fn
+    S = sfx(dt)
+    m, n, k = 64, 48, 32
+    rng = np.random.default_rng(60)
+    A = rng.standard_normal((m, k)).astype(dt)
+    B = np.abs(rng.standard_normal((k, n))).astype(dt) + dt(0.5)      # positive: the sign of an infinite product is the sign of the entry of A
+    b = rng.standard_normal(m).astype(dt)
+    A[3, 5], A[7, 1], A[9, 2] = np.nan, np.inf, -np.inf
+    Ad, Bd, bd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(b)
+    clean = np.ones(m, bool)
+    clean[[3, 7, 9]] = False
+    want = A[clean].astype(np.float64) @ B.astype(np.float64) + b[clean, None]
+    old = fn["knet8_tune"](3, -1)
+    try:
+        for route in (0, 270):
+            fn["knet8_tune"](3, route)
+            for act in (0, 1):
+                C = knet.KnetArray(np.full((m, n), 5.0, dt))
+                assert fn["gemm_bias_act_%s_stream" % S](b"N", b"N", m, n, k, 1.0, Ad.ptr, m, Bd.ptr, k, bd.ptr, act, C.ptr, m, lib.stream) == 0
+                c = knet.Array(C)
+                ref = np.maximum(want, 0) if act else want
+                assert np.abs(c[clean] - ref).max() <= (1e-5 if dt == np.float32 else 1e-13) * np.abs(want).max(), (route, act)
+                if act == 0:
+                    assert np.all(np.isnan(c[3])) and np.all(c[7] == np.inf) and np.all(c[9] == -np.inf), (route, act)
+                else:
+                    assert np.all(c[3] == 0) and np.all(c[7] == np.inf) and np.all(c[9] == 0), (route, act, c[3, :4], c[7, :4], c[9, :4])
+    finally:
+        fn["knet8_tune"](3, old)
+    y = knet.Array(knet.relu(knet.KnetArray(np.array([np.nan, -1.0, 2.0], dt))))
+    assert np.isnan(y[0]) and y[1] == 0 and y[2] == 2
+    lib.check()
+
+
 def test_dense_primitive_in_the_mlp_matches_oracle(knet, oracle):
     rng = np.random.default_rng(56)
     ws = [(rng.standard_normal((64, 784)) * 0.01).astype(np.float32), (rng.standard_normal((64, 1)) * 0.1).astype(np.float32),

@@ -165,6 +165,28 @@ def test_config3_full_size(knet, oracle):
     knet.libknet8().check()
 
 
+def test_config3_full_size_fp64(knet, oracle):
+    """The same three reductions at the reference's other element type, at the launch geometry the bench times (`sum_64_21`): against the oracle's
+    wide-accumulator sums to 1e-12 of sum|x| per output, and exactly on integer-valued data."""
+    rng = np.random.default_rng(26)
+    x = rng.standard_normal((4096, 8192))
+    xd = knet.KnetArray(x)
+    for d in (1, 2):
+        got = knet.Array(knet.sum(xd, dims=d))
+        assert got.dtype == np.float64
+        check_sum(got, oracle.reduce("sum", x, dims=d).astype(np.float64), x, d - 1, rtol=1e-12)
+    xi = rng.integers(-5, 6, size=(4096, 8192)).astype(np.float64)
+    xid = knet.KnetArray(xi)
+    for d in (1, 2):
+        assert np.array_equal(knet.Array(knet.sum(xid, dims=d)), xi.sum(axis=d - 1, keepdims=True))
+    del xd, xid
+    x = rng.standard_normal((56, 56, 256, 64))
+    got = knet.Array(knet.sum(knet.KnetArray(x), dims=[1, 2, 4]))
+    assert got.shape == (1, 1, 256, 1)
+    check_sum(got, oracle.reduce("sum", x, dims=(1, 2, 4)).astype(np.float64), x, (0, 1, 3), rtol=1e-12)
+    knet.libknet8().check()
+
+
 def test_sum_gradient_through_the_tape(knet):
     x = np.arange(12, dtype=np.float32).reshape(3, 4)
     p = knet.Param(knet.KnetArray(x))

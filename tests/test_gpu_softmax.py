@@ -285,6 +285,39 @@ def test_config4_full_size(knet, oracle):
     knet.libknet8().check()
 
 
+def test_config4_full_size_fp64(knet, oracle):
+    """Config 4's two shapes in fp64, i.e. the kernels the bench's fp64 rows time at their own launch geometry: (32000,512) runs the fused nll
+    backward on 512-lane teams that hold part of each column in LDS and logsoftmaxback on 1024-lane register teams; (1000,4096) one wave per
+    column.  Against the oracle's fp64 loops: 1e-12 of the largest entry, loss to 1e-12, and the columns of the nll gradient sum to zero
+    (test/loss.jl:81-92 holds the GPU kernels to the CPU formulas in the same way)."""
+    rng = np.random.default_rng(36)
+    for C, N in [(32000, 512), (1000, 4096)]:
+        scores = rng.standard_normal((C, N)) * 2
+        labels = rng.integers(1, C + 1, size=N)
+        want_loss = oracle.nll(scores, labels)
+        want_grad = oracle.nll_back(scores, labels)
+        for fused in (False, True):
+            p = knet.Param(knet.KnetArray(scores))
+            J = knet.diff(lambda: knet.nll(p, labels, fused=fused))
+            assert abs(float(knet.value(J)) - float(want_loss)) <= 1e-12 * abs(float(want_loss)), (C, N, fused)
+            got = knet.Array(knet.grad(J, p))
+            assert got.dtype == np.float64 and close(got, want_grad, 1e-12), (C, N, fused)
+            big = np.abs(want_grad) >= 1e-3 * np.abs(want_grad).max()
+            relerr = np.abs(got[big] - want_grad[big]) / np.abs(want_grad[big])
+            assert relerr.max() <= 1e-11, (C, N, fused, relerr.max())
+            assert np.abs(got.sum(axis=0)).max() <= 1e-13
+        lsm = oracle.logsoftmax(scores, dims=1)
+        dy = rng.standard_normal((C, N))
+        got = knet.Array(knet.logsoftmaxback(knet.KnetArray(lsm), knet.KnetArray(dy), dims=1))
+        want = oracle.logsoftmaxback(lsm, dy, dims=1)
+        term = np.exp(lsm) * np.abs(dy).sum(axis=0, keepdims=True)
+        err = np.abs(got - want) / np.maximum(np.abs(dy), term)
+        assert err.max() <= 1e-12, (C, N, err.max())
+        got = knet.Array(knet.logsoftmax(knet.KnetArray(scores), dims=1))
+        assert close(got, lsm, 1e-13), (C, N)
+    knet.libknet8().check()
+
+
 def test_random_column_shapes(knet, oracle):
     """Seeded sweep over (m, n): every team size / capacity / vector-scalar combination of the column kernels, plus labels that are
     first, last and skipped."""

@@ -7,17 +7,52 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
+def _alloc_calls(knet):
+    """hipMalloc + hipFree calls the library has made so far (it counts every one)."""
+    import ctypes
+    out = (ctypes.c_ulonglong * 6)()
+    knet.libknet8().fn["knet8_stats"](ctypes.cast(out, ctypes.c_void_p))
+    return out[0] + out[1]
+
+
 def _pair(knet, x, sy, ny):
     lib = knet.libknet8()
     fn = lib.fn
     xd = knet.KnetArray(x.ravel(order="F"))
     a = knet.KnetArray(np.full(ny, -555.0, np.float32))
     b = knet.KnetArray(np.full(ny, -555.0, np.float32))
+    before = _alloc_calls(knet)
     fn["sum_32_21_noalloc"](x.size, xd.ptr, sy, ny, a.ptr, lib.stream)
+    assert _alloc_calls(knet) == before, "sum_32_21_noalloc allocated or freed device memory"   # what the entry point exists for
     fn["sum_32_21_stream"](x.size, xd.ptr, sy, ny, b.ptr, lib.stream)
     knet.synchronize()
     lib.check()
     return knet.Array(a), knet.Array(b)
+
+
+def test_no_alloc_sum_allocates_nothing_not_even_on_a_new_stream(knet):
+    """The very first call on a stream the library has never seen (no scratch, no tickets of its own yet) with a shape that splits: the
+    allocation counter of the library does not move, while the allocating entry point on the same fresh stream does allocate."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    rng = np.random.default_rng(76)
+    x = rng.integers(-3, 4, size=(512, 4096)).astype(np.float32)
+    xd = knet.KnetArray(x)
+    a, b = knet.KnetArray(np.zeros(512, np.float32)), knet.KnetArray(np.zeros(512, np.float32))
+    knet.synchronize()
+    s = fn["knet8_stream_create"]()
+    try:
+        before = _alloc_calls(knet)
+        fn["sum_32_21_noalloc"](x.size, xd.ptr, 1, 512, a.ptr, s)
+        fn["sum_32_21_noalloc"](x.size, xd.ptr, x.size, 1, b.ptr, s)
+        assert _alloc_calls(knet) == before
+        fn["sum_32_21_stream"](x.size, xd.ptr, 1, 512, b.ptr, s)
+        assert _alloc_calls(knet) > before          # the counter does see the per-stream scratch being made
+        assert fn["knet8_synchronize"](s) == 0
+    finally:
+        fn["knet8_stream_destroy"](s)
+    lib.check()
+    assert np.array_equal(knet.Array(a), x.sum(axis=1)) and np.array_equal(knet.Array(b), x.sum(axis=1))
 
 
 def test_no_alloc_sum_matches_the_allocating_entry_point(knet):
