@@ -314,15 +314,20 @@ def profile_pass(torch, K, mode, plan_path):
     x = device_randn(torch, K, n, f32, 1)
     dy = device_randn(torch, K, n, f32, 2)
     dx = x.similar()
+    # The host waits for each group before it prepares the next group's operands: launches are asynchronous, so without the wait the
+    # generation of the next inputs (torch's generator kernels and copies, on another stream) runs beside the launches still queued here and
+    # shares the memory system with one of them (seen as one dispatch of 24 at 922 us instead of 490).
     # Every group is PROFILE_REPS + 1 launches: the first one (the kernel's first dispatch in the process, on operands no kernel of this
     # shape has walked yet) is listed apart by the summary and left out of its averages, as the bench leaves its warm-up launches out.
     for _ in range(PROFILE_REPS + 1):
         K.knet8("copy_32", n, x.ptr, dx.ptr)
+    K.synchronize()
     plan.append(["copy_32 n=2^28 (1 GiB read + 1 GiB written: the yardstick of the byte counters)", 8 * n, PROFILE_REPS])
     for back, fwd in OPS:
         y = K.unary_op(fwd, x)
         for _ in range(PROFILE_REPS + 1):
             K.knet8("%s_32_11" % back, n, dy.ptr, y.ptr, dx.ptr)
+        K.synchronize()
         plan.append(["%s_32_11 n=2^28" % back, 12 * n, PROFILE_REPS])
         del y
     del x, dy, dx
@@ -333,6 +338,7 @@ def profile_pass(torch, K, mode, plan_path):
         yd = K.unary_op(fwd, xd)
         for _ in range(PROFILE_REPS + 1):
             K.knet8("%s_64_11" % back, 1 << 27, dyd.ptr, yd.ptr, dxd.ptr)
+        K.synchronize()
         plan.append(["%s_64_11 n=2^27" % back, 24 << 27, PROFILE_REPS])
         del yd
     del xd, dyd, dxd
@@ -392,7 +398,7 @@ def summarize_profile(root):
             print("!! %d groups of %d dispatches in the trace, %d in the plan: labels below may be off" % (len(matched), PROFILE_REPS, len(plan)))
         scale = {}
         for which in ("fetch", "write"):
-            ck = [k for k in cnt[which] if "Op_copy<float>" in k[0] or "copy" in short(k[0]).lower()]
+            ck = [k for k in cnt[which] if ("Op_copy<float>" in k[0] or "copy" in short(k[0]).lower()) and len(cnt[which][k]) == PROFILE_REPS]
             if ck:
                 kib = float(np.mean(cnt[which][ck[0]]))
                 scale[which] = (1 << 20) / kib
