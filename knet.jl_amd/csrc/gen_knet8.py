@@ -683,7 +683,8 @@ KNET8_API void sum_32_21_noalloc(int nx, float* x, int sy, int ny, float* y, hip
    key 4: dense_back_S / dense_nll_back_S accept layers whose products have up to this many MFLOP each (default 270);
    key 5: non-zero makes the library behave as if the scratch memory of split launches could not be allocated (for tests of that error path);
    key 6: non-zero keeps softmax columns of 128 to 256 KB in registers alone instead of registers + LDS (for comparisons);
-   key 7: non-zero makes the hipBLASLt route of gemm_S do everything but the vendor call itself (for measuring the library's own share of a call's host time) */
+   key 7: non-zero makes the hipBLASLt route of gemm_S do everything but the vendor call itself (for measuring the library's own share of a call's host time);
+   key 8: non-zero keeps repeated products on hipblasLtMatmul instead of the prepared calls of the vendor's extension interface (for comparisons) */
 KNET8_API int knet8_tune(int key, int value);
 /* Seed of the default random stream used by rand_S / randn_S (restarts it at counter 0): the device half of Knet.seed!,
    src/knetarrays/random.jl:14-18 (CUDA.seed!).  Unseeded, the stream starts from the operating system's entropy. */

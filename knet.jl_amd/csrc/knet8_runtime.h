@@ -56,7 +56,7 @@ void fetch_scalar(hipStream_t stream, const void* dev, void* host, size_t nbytes
 // State of the default random stream (knet8_seed): hands out `blocks` consecutive generator counters under the current seed.
 void rng_take(unsigned long long blocks, unsigned long long* seed, unsigned long long* offset);
 
-enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneGemmSmallMflop = 3, kTuneDenseBackMflop = 4, kTuneFailScratch = 5, kTuneSoftmaxNoLdsSlots = 6, kTuneGemmDryRun = 7, kTuneCount = 8 };
+enum { kTuneNumCUs = 0, kTuneSoftmaxResidentRows = 1, kTuneGemmSmallMflop = 3, kTuneDenseBackMflop = 4, kTuneFailScratch = 5, kTuneSoftmaxNoLdsSlots = 6, kTuneGemmDryRun = 7, kTuneGemmNoPrepared = 8, kTuneCount = 9 };
 int tuning(int key);
 
 #ifdef KNET8_TIMELINE

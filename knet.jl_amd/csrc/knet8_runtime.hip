@@ -5,6 +5,7 @@
 #include "knet8_fused.h"
 
 #include <hipblaslt/hipblaslt.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 
 #include <atomic>
 #include <cstdio>
@@ -80,7 +81,7 @@ void rng_take(unsigned long long blocks, unsigned long long* seed, unsigned long
   g_rng_offset += blocks;
 }
 
-static int g_tune[kTuneCount] = {0, 0, 0, 0, 0, 0, 0, 0};
+static int g_tune[kTuneCount] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 int tuning(int key) {
   if (key < 0 || key >= kTuneCount) return 0;
   if (key == kTuneNumCUs && g_tune[key] == 0) {  // compute units of the current device, asked once
@@ -640,18 +641,34 @@ static size_t gemm_release(int dev, hipStream_t stream, bool every) {
   return released;
 }
 
-// The last few plain products of this thread: problem, stream, and everything the vendor call needs.  A repeat (the same layer of the
-// same model in the next step) goes straight to hipblasLtMatmul: no map lookups, no capture query, the lock held for the vendor call only.  Only plans that are final
-// (algorithm chosen by timing) and carry no bias pointer are remembered; the plans themselves are never destroyed once valid.
+// The last plain products of this thread: problem, stream, operands, and everything the vendor call needs.  A repeat of the problem (the
+// same layer of the same model in the next step) goes straight to the vendor call: no map lookups, the lock held for the call only.  When
+// the operands repeat as well -- the pool hands a steady-state training step the same blocks every time -- the call is *prepared*: the
+// vendor library's extension interface builds the kernel's arguments once (hipblaslt_ext::Gemm::initialize) and every later call only
+// launches them (run), which costs a caller about what a plain kernel launch costs instead of a full hipblasLtMatmul.  Only plans that are
+// final (algorithm chosen by timing) and carry no bias pointer are remembered; plans are never destroyed once valid.
 struct GemmRecent {
   GemmKey key;
-  hipStream_t stream;
-  const GemmPlan* plan;
-  hipblasLtHandle_t handle;
-  void* ws;
+  hipStream_t stream = nullptr;
+  const GemmPlan* plan = nullptr;
+  hipblasLtHandle_t handle = nullptr;
+  void* ws = nullptr;
   unsigned long long generation = 0;   // 0: empty
+  const void *A = nullptr, *B = nullptr;
+  void* C = nullptr;
+  double alpha = 0, beta = 0;          // the scalars of the prepared call (a float is held exactly)
+  union { float f; double d; } alpha_t, beta_t;   // what the prepared arguments point to
+  int repeats = 0;                     // calls in a row with these operands and scalars
+  bool no_prepare = false;             // the extension interface refused this problem: stay with hipblasLtMatmul
+  hipblaslt_ext::Gemm* prepared = nullptr;
+  void reset() {
+    delete prepared;
+    prepared = nullptr;
+    generation = 0; repeats = 0; no_prepare = false;
+  }
+  ~GemmRecent() { delete prepared; }
 };
-constexpr int kGemmRecent = 8;
+constexpr int kGemmRecent = 32;
 static thread_local GemmRecent t_recent[kGemmRecent];
 static thread_local int t_recent_next = 0;
 static bool same_key(const GemmKey& a, const GemmKey& b) {
@@ -695,21 +712,40 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
   (void)hipGetDevice(&dev);
   const GemmKey key = {dev, (int)sizeof(T), ta, tb, m, n, k, lda, ldb, ldc, batch.count, epilogue, batch.sa, batch.sb, batch.sc};
   const bool dry = g_tune[kTuneGemmDryRun] != 0;   // measurements of the library's own share of a call: everything but the vendor call
-  if (epilogue == kEpiNone) {
+  const bool capturing = stream_is_capturing(stream);
+  if (epilogue == kEpiNone && !capturing) {   // (a product being recorded into a graph takes the full path, which notes that a graph now names the workspace)
     const unsigned long long gen = g_gemm_generation.load(std::memory_order_acquire);
     for (int i = 0; i < kGemmRecent; i++) {
-      const GemmRecent& r = t_recent[i];
-      if (r.generation == gen && r.stream == stream && same_key(r.key, key)) {
-        if (dry) return 0;
-        // (the vendor call itself stays under the lock: concurrent hipblasLtMatmul calls on one handle from several host threads gave wrong
-        //  products in the library's own multi-thread test)
-        std::lock_guard<std::mutex> lock(g_gemm_mutex);
-        return lt_ok(hipblasLtMatmul(r.handle, r.plan->desc, &alpha, A, r.plan->la, B, r.plan->lb, &beta, C, r.plan->lc, C, r.plan->lc, &r.plan->algo, r.ws,
-                                     kGemmWorkspace, stream), "matmul") ? 0 : -1;
+      GemmRecent& r = t_recent[i];
+      if (r.generation != gen || r.stream != stream || r.A != A || r.B != B || r.C != C || !same_key(r.key, key)) continue;
+      if (dry) return 0;
+      const bool same_scalars = r.alpha == (double)alpha && r.beta == (double)beta;
+      r.repeats = same_scalars ? r.repeats + 1 : 0;
+      r.alpha = (double)alpha; r.beta = (double)beta;
+      // (the vendor calls stay under the lock: concurrent calls on one handle from several host threads gave wrong products in the
+      //  library's own multi-thread test)
+      std::lock_guard<std::mutex> lock(g_gemm_mutex);
+      const bool allowed = g_tune[kTuneGemmNoPrepared] == 0;
+      if ((!same_scalars || !allowed) && r.prepared) { delete r.prepared; r.prepared = nullptr; }
+      if (!r.prepared && !r.no_prepare && r.repeats >= 1 && allowed) {
+        if (sizeof(T) == 4) { r.alpha_t.f = (float)alpha; r.beta_t.f = (float)beta; } else { r.alpha_t.d = (double)alpha; r.beta_t.d = (double)beta; }
+        auto* g = new hipblaslt_ext::Gemm(r.handle, r.plan->desc, &r.alpha_t, A, r.plan->la, B, r.plan->lb, &r.beta_t, C, r.plan->lc, C, r.plan->lc);
+        hipblasLtMatmulAlgo_t algo = r.plan->algo;
+        size_t need = 0;
+        g->setMaxWorkspaceBytes(kGemmWorkspace);
+        if (g->isAlgoSupported(algo, need) == HIPBLAS_STATUS_SUCCESS && need <= kGemmWorkspace &&
+            g->initialize(algo, r.ws, false, stream) == HIPBLAS_STATUS_SUCCESS) {
+          r.prepared = g;
+        } else {
+          delete g;
+          r.no_prepare = true;
+        }
       }
+      if (r.prepared) return lt_ok(r.prepared->run(stream), "prepared matmul") ? 0 : -1;
+      return lt_ok(hipblasLtMatmul(r.handle, r.plan->desc, &alpha, A, r.plan->la, B, r.plan->lb, &beta, C, r.plan->lc, C, r.plan->lc, &r.plan->algo, r.ws,
+                                   kGemmWorkspace, stream), "matmul") ? 0 : -1;
     }
   }
-  const bool capturing = stream_is_capturing(stream);
   std::lock_guard<std::mutex> lock(g_gemm_mutex);
   hipblasLtHandle_t& h = g_lt[dev];
   if (!h && !lt_ok(hipblasLtCreate(&h), "create")) return -1;
@@ -810,7 +846,9 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
   if (epilogue == kEpiNone && p.timed && !capturing) {
     GemmRecent& r = t_recent[t_recent_next];
     t_recent_next = (t_recent_next + 1) % kGemmRecent;
+    r.reset();
     r.key = key; r.stream = stream; r.plan = &p; r.handle = h; r.ws = ws;
+    r.A = A; r.B = B; r.C = C; r.alpha = (double)alpha; r.beta = (double)beta;
     r.generation = g_gemm_generation.load(std::memory_order_acquire);
   }
   if (dry) return 0;

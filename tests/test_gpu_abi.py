@@ -321,6 +321,36 @@ def test_product_routing_knob_both_routes_agree(knet, oracle):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt,S", [(np.float32, "32"), (np.float64, "64")])
+def test_repeated_products_on_the_same_operands_stay_correct(knet, dt, S):
+    """A product repeated on the same device operands (what a training step does through the pool) is served by a call the vendor library's
+    extension interface prepared once; the operands' CONTENTS and the scalars may change from call to call, and every call must give the product of
+    what is in memory then: new data in A, another alpha, beta = 1 accumulating, and the same through knet8_tune key 8 (prepared calls off)."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    rng = np.random.default_rng(61)
+    m, n, k = 192, 100, 300
+    tol = 1e-5 if dt == np.float32 else 1e-13
+    for off in (0, 1):
+        old = fn["knet8_tune"](8, off)
+        try:
+            B = rng.standard_normal((k, n)).astype(dt)
+            Ad, Bd, Cd = knet.KnetArray(np.zeros((m, k), dt)), knet.KnetArray(B), knet.KnetArray(np.zeros((m, n), dt))
+            acc = np.zeros((m, n))
+            for it, (alpha, beta) in enumerate([(1.0, 0.0), (1.0, 0.0), (1.0, 0.0), (1.0, 0.0), (0.5, 0.0), (0.5, 0.0), (0.5, 0.0), (2.0, 1.0), (2.0, 1.0), (2.0, 1.0), (1.0, 0.0)]):
+                A = rng.standard_normal((m, k)).astype(dt)
+                Af = np.asfortranarray(A)           # kept alive across the copy
+                fn["knet8_memcpy"](Ad.ptr, Af.ctypes.data, Af.nbytes, 1, lib.stream)
+                assert fn["gemm_%s_stream" % S](b"N", b"N", m, n, k, alpha, Ad.ptr, m, Bd.ptr, k, beta, Cd.ptr, m, lib.stream) == 0
+                acc = alpha * (A.astype(np.float64) @ B.astype(np.float64)) + beta * acc
+                got = knet.Array(Cd)
+                assert np.linalg.norm(got - acc) <= tol * np.linalg.norm(acc) * (it + 1), (off, it, alpha, beta)
+                acc = got.astype(np.float64)     # accumulate on what the device holds, so the tolerance does not compound
+        finally:
+            fn["knet8_tune"](8, old)
+    lib.check()
+
+
 def test_split_launch_without_scratch_is_refused_on_the_host(knet):
     """When the scratch memory of a split launch cannot be had (out of device memory; forced here through knet8_tune key 5) the
     launch must not happen at all: the failure is recorded, as "Out of gpu memory" is an error and not a crash in the reference
