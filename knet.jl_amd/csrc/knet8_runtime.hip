@@ -6,6 +6,7 @@
 
 #include <hipblaslt/hipblaslt.h>
 #include <hipblaslt/hipblaslt-ext.hpp>
+#include <hipblaslt/hipblaslt-version.h>
 
 #include <atomic>
 #include <cstdio>
@@ -668,6 +669,24 @@ struct GemmRecent {
   }
   ~GemmRecent() { delete prepared; }
 };
+// The extension interface is a C++ class whose layout belongs to one build of the vendor library.  A process may have resolved libhipblaslt.so.1 to
+// another build than the one whose headers this file was compiled against (a Python process that imported PyTorch first gets the copy PyTorch
+// bundles): prepared calls are used only when the loaded library reports the very revision of those headers, otherwise every product stays on the
+// C interface (hipblasLtMatmul), whose ABI is stable.
+#define KNET8_STR2(x) #x
+#define KNET8_STR(x) KNET8_STR2(x)
+static bool ext_interface_matches(hipblasLtHandle_t h) {
+  static int state = -1;   // (called under g_gemm_mutex)
+  if (state < 0) {
+    char rev[256] = {0};
+    int version = 0;
+    const bool ok = hipblasLtGetVersion(h, &version) == HIPBLAS_STATUS_SUCCESS && hipblasLtGetGitRevision(h, rev) == HIPBLAS_STATUS_SUCCESS &&
+                    version == HIPBLASLT_VERSION_MAJOR * 100000 + HIPBLASLT_VERSION_MINOR * 100 + HIPBLASLT_VERSION_PATCH &&
+                    std::string(rev) == KNET8_STR(HIPBLASLT_VERSION_TWEAK);
+    state = ok ? 1 : 0;
+  }
+  return state == 1;
+}
 constexpr int kGemmRecent = 32;
 static thread_local GemmRecent t_recent[kGemmRecent];
 static thread_local int t_recent_next = 0;
@@ -725,14 +744,13 @@ static int gemm_lt(bool ta, bool tb, int m, int n, int k, T alpha, const T* A, i
       // (the vendor calls stay under the lock: concurrent calls on one handle from several host threads gave wrong products in the
       //  library's own multi-thread test)
       std::lock_guard<std::mutex> lock(g_gemm_mutex);
-      const bool allowed = g_tune[kTuneGemmNoPrepared] == 0;
+      const bool allowed = g_tune[kTuneGemmNoPrepared] == 0 && ext_interface_matches(r.handle);
       if ((!same_scalars || !allowed) && r.prepared) { delete r.prepared; r.prepared = nullptr; }
       if (!r.prepared && !r.no_prepare && r.repeats >= 1 && allowed) {
         if (sizeof(T) == 4) { r.alpha_t.f = (float)alpha; r.beta_t.f = (float)beta; } else { r.alpha_t.d = (double)alpha; r.beta_t.d = (double)beta; }
         auto* g = new hipblaslt_ext::Gemm(r.handle, r.plan->desc, &r.alpha_t, A, r.plan->la, B, r.plan->lb, &r.beta_t, C, r.plan->lc, C, r.plan->lc);
         hipblasLtMatmulAlgo_t algo = r.plan->algo;
         size_t need = 0;
-        g->setMaxWorkspaceBytes(kGemmWorkspace);
         if (g->isAlgoSupported(algo, need) == HIPBLAS_STATUS_SUCCESS && need <= kGemmWorkspace &&
             g->initialize(algo, r.ws, false, stream) == HIPBLAS_STATUS_SUCCESS) {
           r.prepared = g;

@@ -173,6 +173,28 @@ def test_no_undefined_device_runtime_surprises(built_lib):
     assert any("amdhip64" in n for n in needed)
 
 
+def test_the_library_loads_beside_the_hipblaslt_that_pytorch_bundles(built_lib):
+    """A Python process that imported PyTorch first has libhipblaslt.so.1 resolved to PyTorch's bundled copy, an older build than the one under
+    /opt/rocm.  libknet8.so must still load there: every hipblaslt symbol it imports has to exist in both copies (the C++ extension interface is
+    then switched off at run time, because its class layout belongs to one build; that check is in the library)."""
+    import glob
+    import importlib.util
+    spec = importlib.util.find_spec("torch")
+    if spec is None or not spec.submodule_search_locations:
+        pytest.skip("PyTorch is not installed here")
+    bundled = glob.glob(os.path.join(list(spec.submodule_search_locations)[0], "lib", "libhipblaslt.so*"))
+    if not bundled:
+        pytest.skip("this PyTorch bundles no libhipblaslt")
+
+    def syms(path, flag):
+        out = subprocess.check_output(["nm", "-D", flag, path], text=True)
+        return {l.split()[-1] for l in out.splitlines() if l.strip()}
+    wanted = {s for s in syms(built_lib, "--undefined-only") if "hipblaslt" in s.lower()}
+    assert len(wanted) >= 10
+    have = syms(bundled[0], "--defined-only")
+    assert not sorted(wanted - have), sorted(wanted - have)
+
+
 def test_generated_files_match_the_operator_tables():
     gen = _load("gen_knet8_for_test", "knet.jl_amd/csrc/gen_knet8.py")
     for path, text in gen.generate(write=False).items():
