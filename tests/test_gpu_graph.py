@@ -58,6 +58,46 @@ def test_captured_mlp_step_matches_eager_on_every_replay(knet, oracle):
         lib.stream = old_stream
 
 
+def test_a_trim_leaves_what_a_captured_graph_names(knet):
+    """knet8_trim gives back the per-stream reduction scratch and hipBLASLt workspaces -- except those handed out while their stream was being
+    captured: a graph holds their addresses.  A graph of one product and one split reduction replays correctly after a trim, with eager work of the
+    same kinds (which allocates scratch afresh) in between."""
+    rng = np.random.default_rng(83)
+    lib = knet.libknet8()
+    fn = lib.fn
+    old_stream = lib.stream
+    try:
+        A, B = rng.integers(-2, 3, size=(200, 300)).astype(np.float32), rng.integers(-2, 3, size=(300, 150)).astype(np.float32)
+        x = rng.integers(-3, 4, size=(256, 4096)).astype(np.float32)
+        Ad, Bd, xd = knet.KnetArray(A), knet.KnetArray(B), knet.KnetArray(x)
+
+        def step():
+            return [knet.matmul(Ad, Bd), knet.sum(xd, dims=2)]
+        g = knet.capture(step)
+        for r in range(3):
+            if r == 1:
+                assert fn["knet8_trim"]() >= 0
+                # eager work on another stream after the trim: new scratch and a new workspace are made, the graph's stay where they were
+                s2 = fn["knet8_stream_create"]()
+                lib.stream = s2
+                assert np.array_equal(knet.Array(knet.sum(xd, dims=2)).ravel(), x.sum(axis=1))
+                assert np.array_equal(knet.Array(knet.matmul(Ad, Bd)), A @ B)
+                knet.synchronize()
+                lib.stream = old_stream
+                fn["knet8_stream_destroy"](s2)
+            fn["fill_32_stream"](200 * 150, 0.0, g.outputs[0].ptr, g.stream)
+            fn["fill_32_stream"](256, 0.0, g.outputs[1].ptr, g.stream)
+            g.replay()
+            knet.synchronize()
+            fn["knet8_synchronize"](g.stream)
+            assert np.array_equal(knet.Array(g.outputs[0]), A @ B), r
+            assert np.array_equal(knet.Array(g.outputs[1]).ravel(), x.sum(axis=1)), r
+        del g
+        lib.check()
+    finally:
+        lib.stream = old_stream
+
+
 def test_captured_step_with_fused_layers_dropout_and_split_reductions(knet, oracle):
     """A deeper net whose hidden layers are the fused bias+relu+dropout launches: the backward kernels split their bias-gradient sums
     over several workgroups (ticket counters and partial buffers live in the per-stream scratch), which a graph replays as is."""
