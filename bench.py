@@ -494,6 +494,8 @@ def two_streams(torch, K):
     s2 = fn["knet8_stream_create"]()
     print("libknet8 on one MI355X: 24 cold launches per kernel on one stream and alternated over two streams (`python3 bench.py --two-streams`).")
     print("us per launch = elapsed time of the batch / 24 (HIP events; two streams: from the first record to the later of the two streams' ends); median of 5 batches.")
+    print("Reading: where the second stream brings a kernel to the level of the one-shot yardsticks (0.79-0.82), its loss on one stream lies between launches -- the")
+    print("tail of one launch (slowest workgroups, partial results, ticket, combine) runs under the ramp of the next; where it does not, the loss is inside the kernel.")
     print("%-92s %10s %10s %8s %10s %10s" % ("kernel", "1 stream", "2 streams", "ratio", "frac 1s", "frac 2s"))
     for key, label, nbytes, nsets, make_launch, yard in kernel_cases(torch, K, widths=("32",)):
         launches = [make_launch(i) for i in range(nsets)]

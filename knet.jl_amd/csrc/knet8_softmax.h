@@ -154,6 +154,10 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
                                        (__attribute__((address_space(3))) void*)(held + j * BT + (threadIdx.x & ~(kWave - 1))), 16, 0, 2);
   V ra[kHold ? RI : 1], rb[kTwo ? RI : 1];
   T ah = T(0), at = T(0), bh = T(0), bt = T(0);
+#ifndef KNET8_LOAD_PACE
+#define KNET8_LOAD_PACE 1
+#endif
+  constexpr bool kPacedLoads = KNET8_LOAD_PACE != 0 && !kHold && TEAM == 1024 && RI >= 4 && sizeof(T) == 4;   // (an fp64 column of this length has its compute unit to itself)
 #pragma unroll
   for (int i = 0; i < RI; i++) {
     const long r = head + (long)(tl + i * TEAM) * NV;
@@ -166,6 +170,11 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
         if (kTwo) rb[i][0] = __builtin_nontemporal_load(bc + r);
       }
     }
+    // Long columns whose second operand is streamed later (logsoftmaxback): the held operand is requested two vectors at a time.  With all eight
+    // requested at once the two workgroups of a compute unit are served one after the other -- the first has its column after 5 us, the second
+    // after 13-22 -- and finish that far apart; in pairs their requests interleave and both have their sums by 10-11 us.  (32000 rows fp32, cold:
+    // 33.9 -> 33.6 us on top of the batched output pass, which took it from 35.2 to 33.9.)
+    if (kPacedLoads && (i + 1) % 2 == 0 && i + 1 < RI) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   if (NV > 1) {
     if (hv) { ah = ac[tl]; if (kTwo) bh = bc[tl]; }
@@ -221,29 +230,68 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
   s = team_reduce<T, TEAM>(s, lds, AddFn(), T(0));
   const T fin = Algo::finish(s);
   KNET8_TL_MID
+  // An operand that is only needed here (logsoftmaxback's y) is fetched kStreamBatch vectors at a time, all requested before the first of them is
+  // used.  Written as load / use / store per vector, every load waits for the store before it as well (loads and stores share one counter, and a
+  // wait on a mixed counter is a wait for all of it): eight dependent memory round trips per lane, during which a workgroup cannot take the
+  // bandwidth that workgroups which are already done have freed.  A batch is one branch and one wait: its loads are unconditional (a lane whose
+  // share ends inside the batch reads its last vector again instead) and only the stores are guarded.
+#ifndef KNET8_STREAM_BATCH
+#define KNET8_STREAM_BATCH 4
+#endif
+  constexpr int kStreamBatch = (!kHold && LV == 0 && ITEMS >= KNET8_STREAM_BATCH) ? KNET8_STREAM_BATCH : 1;
+  if constexpr (kStreamBatch > 1) {
 #pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    if (i >= cnt) continue;
-    const long r = head + (long)(tl + i * TEAM) * NV;
-    V va = {}, vb = {};
-    if (i < RI) {
-      if (kHold) va = ra[kHold && i < RI ? i : 0];
-      if (kTwo) vb = rb[kTwo && i < RI ? i : 0];
-    } else {
-      va = mine[(i - RI) * BT];
-    }
-    if (!kHold) {
-      if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
-      else va[0] = __builtin_nontemporal_load(ac + r);
-    }
-    V vo;
+    for (int i0 = 0; i0 < ITEMS; i0 += kStreamBatch) {
+      if (i0 < cnt) {
+        V sa[kStreamBatch];
 #pragma unroll
-    for (int e = 0; e < NV; e++) {
-      if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(va[e], fin);
-      else vo[e] = Algo::out(va[e], kTwo ? vb[e] : T(0), mx, fin);
+        for (int j = 0; j < kStreamBatch; j++) {
+          const int ii = i0 + j < cnt ? i0 + j : cnt - 1;
+          const long r = head + (long)(tl + ii * TEAM) * NV;
+          if (VEC) sa[j] = ld_stream(reinterpret_cast<const V*>(ac + r));
+          else sa[j][0] = __builtin_nontemporal_load(ac + r);
+        }
+#pragma unroll
+        for (int j = 0; j < kStreamBatch; j++) {
+          const int i = i0 + j;
+          if (i < ITEMS) {
+            const long r = head + (long)(tl + i * TEAM) * NV;
+            V vo;
+#pragma unroll
+            for (int e = 0; e < NV; e++) vo[e] = Algo::out(sa[j][e], kTwo ? rb[kTwo && i < RI ? i : 0][e] : T(0), mx, fin);
+            if (i < cnt) {
+              if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+              else __builtin_nontemporal_store(vo[0], oc + r);
+            }
+          }
+        }
+      }
     }
-    if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
-    else __builtin_nontemporal_store(vo[0], oc + r);
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      if (i >= cnt) continue;
+      const long r = head + (long)(tl + i * TEAM) * NV;
+      V va = {}, vb = {};
+      if (i < RI) {
+        if (kHold) va = ra[kHold && i < RI ? i : 0];
+        if (kTwo) vb = rb[kTwo && i < RI ? i : 0];
+      } else {
+        va = mine[(i - RI) * BT];
+      }
+      if (!kHold) {
+        if (VEC) va = ld_stream(reinterpret_cast<const V*>(ac + r));
+        else va[0] = __builtin_nontemporal_load(ac + r);
+      }
+      V vo;
+#pragma unroll
+      for (int e = 0; e < NV; e++) {
+        if constexpr (Algo::kKeepTerm && kHold) vo[e] = Algo::out_kept(va[e], fin);
+        else vo[e] = Algo::out(va[e], kTwo ? vb[e] : T(0), mx, fin);
+      }
+      if (VEC) st_stream(reinterpret_cast<V*>(oc + r), vo);
+      else __builtin_nontemporal_store(vo[0], oc + r);
+    }
   }
   if (NV > 1) {
     // a streamed (not held) first input was read above as ah/at all the same: the extras are always held
