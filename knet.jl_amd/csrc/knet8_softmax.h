@@ -238,7 +238,7 @@ __device__ __forceinline__ void softmax_col_body(int m, long n, const T* a, cons
 #ifndef KNET8_STREAM_BATCH
 #define KNET8_STREAM_BATCH 4
 #endif
-  constexpr int kStreamBatch = (!kHold && LV == 0 && ITEMS >= KNET8_STREAM_BATCH) ? KNET8_STREAM_BATCH : 1;
+  constexpr int kStreamBatch = (!kHold && LV == 0 && ITEMS >= KNET8_STREAM_BATCH) ? KNET8_STREAM_BATCH : 1;   // (columns of two vectors per lane measured slower batched: 4000 rows 18.5 -> 20.9 us)
   if constexpr (kStreamBatch > 1) {
 #pragma unroll
     for (int i0 = 0; i0 < ITEMS; i0 += kStreamBatch) {
