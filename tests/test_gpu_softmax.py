@@ -318,6 +318,42 @@ def test_config4_full_size_fp64(knet, oracle):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt,S", [(np.float32, "32"), (np.float64, "64")])
+def test_logsoftmaxback_batched_output_pass_every_share_pattern(knet, oracle, dt, S):
+    """logsoftmaxback on 1024-lane teams fetches y a batch of four vectors at a time with unconditional loads (a lane whose share ends inside a batch reads
+    its last vector again) and guarded stores.  Column lengths chosen so that lanes hold every count of vectors from one to the full eight (four in
+    the shorter configuration), with columns that start off the 16-byte grid; through the C ABI on views inside sentinel-filled arrays: the result
+    matches the oracle and nothing outside the m*n outputs is written."""
+    lib = knet.libknet8()
+    fn = lib.fn
+    rng = np.random.default_rng(62)
+    nv = 4 if dt == np.float32 else 2
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    # vectors per column = ceil-ish(m / nv); lanes 0..1023 take vectors lane, lane+1024, ...: m just above k*1024*nv gives counts k+1 and k
+    ms = [1024 * nv * k + d for k in (2, 3, 4, 5, 6, 7) for d in (nv, 1024 * nv // 2 + 3)] + [8192 * nv, 8192 * nv - 1, 2048 * nv + 1, 4096 * nv - 2 * nv]
+    ms = [m for m in ms if 2048 < m <= 8192 * nv]
+    pad = 64
+    for m in ms:
+        for off in (0, 1, 3):
+            n = 3
+            y = oracle.logsoftmax((rng.standard_normal((m, n)) * 2).astype(dt), dims=1)
+            dy = rng.standard_normal((m, n)).astype(dt)
+            want = oracle.logsoftmaxback(y, dy, dims=1)
+            bufs = []
+            for a in (y, dy, np.full((m, n), -777.0, dt)):
+                flat = np.concatenate([np.full(pad + off, -777.0, dt), a.ravel(order="F"), np.full(pad, -777.0, dt)])
+                bufs.append(knet.KnetArray(flat))
+            es = dt().itemsize
+            ptr = lambda b: b.ptr + (pad + off) * es
+            fn["logsoftmaxback_%s_stream" % S](m, n, ptr(bufs[0]), ptr(bufs[1]), ptr(bufs[2]), lib.stream)
+            out = knet.Array(bufs[2])
+            got = out[pad + off: pad + off + m * n].reshape(m, n, order="F")
+            scale = np.maximum(np.abs(dy.astype(np.float64)), np.exp(y.astype(np.float64)) * np.abs(dy.astype(np.float64)).sum(axis=0, keepdims=True))
+            assert (np.abs(got.astype(np.float64) - want) / scale).max() <= rtol, (m, off)
+            assert np.all(out[:pad + off] == dt(-777.0)) and np.all(out[pad + off + m * n:] == dt(-777.0)), (m, off)
+    lib.check()
+
+
 def test_random_column_shapes(knet, oracle):
     """Seeded sweep over (m, n): every team size / capacity / vector-scalar combination of the column kernels, plus labels that are
     first, last and skipped."""
