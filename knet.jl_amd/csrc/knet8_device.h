@@ -33,6 +33,13 @@ template <> struct Vec16<int> {
 template <typename V> __device__ __forceinline__ V ld_stream(const V* p) { return __builtin_nontemporal_load(p); }
 template <typename V> __device__ __forceinline__ void st_stream(V* p, V v) { __builtin_nontemporal_store(v, p); }
 
+// A 16-byte store written through to the device-coherent level (sc1) instead of staying dirty in this XCD's L2.  The compiler has no form of
+// it for vectors; the inline instruction is an ordinary vector store (the "memory" clobber keeps later loads of the same address behind it).
+template <typename V> __device__ __forceinline__ void st_through(V* p, V v) {
+  static_assert(sizeof(V) == 16, "st_through: 16-byte vectors");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+
 template <typename T> __host__ __device__ __forceinline__ bool aligned16(const T* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }

@@ -140,7 +140,10 @@ __global__ __launch_bounds__(BT) void actback_biasgrad_kernel(const T* dy, const
           V r;
 #pragma unroll
           for (int e = 0; e < NV; e++) { r[e] = f(d[q][e], o[q][e]); g[q][e] = jj < j1 ? r[e] : T(0); }
-          if (jj < j1) st_stream(reinterpret_cast<V*>(dz + jj * m + a0), r);
+          // written through (sc1), not merely streamed: what a kernel leaves dirty in the L2s is written back after its last workgroup has ended,
+          // before the next launch may start; written through, dz drains while the partial sums are still being combined
+          // ((4096,2048) fp32 cold: 19.3 -> 18.4 us; nt sc1 19.9-20.0, sc0 sc1 18.6, plain 19.3)
+          if (jj < j1) st_through(reinterpret_cast<V*>(dz + jj * m + a0), r);
         }
       } else {
 #pragma unroll
