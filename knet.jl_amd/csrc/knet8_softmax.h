@@ -1038,7 +1038,8 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   }
   // Columns of 128 to 256 KB: two 512-lane workgroups per compute unit with part of the column in LDS (see softmax_col_body).
   // Measured on (32000,512) fp64, cold: logsoftmax 59.7 -> 44.5 us, softmax 59.8 -> 47.5, fused nll 52.2 -> 42.5; logsoftmaxback, whose output pass
-  // reads a second operand, gains nothing (70.8 -> 71.6) and keeps its registers-only kernel.
+  // reads a second operand, gains nothing (70.8 -> 71.6; 70.8 -> 73.4 with that pass fetching two vectors ahead, all that 128 registers leave room for) and keeps
+  // its registers-only kernel.
   // The same 512-lane kernels serve fp32 columns of 32 769 to 65 536 rows (vocabularies of 50257 entries): forward kernels 44.5 -> 41.6 and 46.4 -> 40.7 us
   // on (50257,512); the fused fp32 nll kernel is as fast from registers alone (42.4 against 45.8) and keeps them.
   if constexpr (Algo::kInputs == 1 && (!Algo::kNll || sizeof(T) == 8)) {
