@@ -1058,7 +1058,9 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   constexpr bool kStreamsA = Algo::kInputs == 2 && !Algo::kHoldA;
   constexpr bool kWideSingle = sizeof(T) == 8 && Algo::kInputs == 1;
   if (m <= 64 * 4) KNET8_SM(64, 4);
-  else if (m <= 64 * 16) KNET8_SM(64, 16);
+  // (fp64 logsoftmaxback on columns of 769 to 1024 rows: 256 lanes with two vectors each, the second operand streamed, beat one wave holding both
+  //  operands -- 1000 rows x 4096 columns, cold: 19.0 -> 18.1 us; every other kernel and width is 3 to 50 % slower that way, and so is this one below 768 rows)
+  else if (m <= 64 * 16) { if (kStreamsA && sizeof(T) == 8 && m > 768) KNET8_SM(256, 4); else KNET8_SM(64, 16); }
   else if (m <= 256 * 16) { if (kStreamsA && m > 2048) KNET8_SM(1024, 8); else KNET8_SM(256, 16); }
   else if (m <= 1024 * 8) { if constexpr (kWideSingle) KNET8_SM(256, 32); else KNET8_SM(1024, 8); }
   else if (m <= 1024 * 16) { if constexpr (kWideSingle) KNET8_SM(256, 64); else KNET8_SM(1024, 16); }

@@ -6,7 +6,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-MS = [1, 2, 3, 63, 64, 65, 250, 256, 257, 1000, 1001, 1024, 4096, 4100, 9999, 16384, 16388, 32000, 32769, 65536, 70001]
+MS = [1, 2, 3, 63, 64, 65, 250, 256, 257, 768, 769, 1000, 1001, 1024, 4096, 4100, 9999, 16384, 16388, 32000, 32769, 65536, 70001]
 
 
 def close(got, want, rtol=1e-5):
