@@ -491,15 +491,22 @@ constexpr int kShortRows = 128;
 // slower: 17 us against 12.4 us at m = 32: the column pass is the one that counts.)
 __device__ __forceinline__ int short_pad(int i) { return i + (i >> 5); }
 
-// R: elements of a column per lane (TL*R >= m).  Slots past the column's end are computed and thrown away, so the host picks, among R = 2, 3, 4, 6, 8,
-// the pair that wastes fewest: ten classes run as 4 lanes x 3, not 2 x 8.
+// Vectors per lane of a stretch.  One input: four (16 KB per workgroup).  Two inputs: one (fp32) or two (fp64) -- 4 / 8 KB per operand: with 16 KB
+// each a compute unit holds four workgroups instead of eight, and all of them are in the same phase (all reading, then all in their column pass, then
+// all writing), so the column pass is not hidden behind other workgroups' memory traffic.  Measured over m = 8 ... 100, 2^23 elements per operand, cold:
+// logsoftmaxback fp32 19.8-24.0 us with 16 KB, 18.1-19.5 with 8 KB, 17.8-19.3 with 4 KB; fp64 36.6-39.2 / 33.6-35.8 / 33.2-38.7.  The one-input kernels lose
+// with shorter stretches (fp32 logsoftmax m = 32: 12.4 / 14.3 / 15.9 us).
+template <typename T, typename Algo> constexpr int short_stretch_vectors() { return Algo::kInputs == 2 ? (sizeof(T) == 4 ? 1 : 2) : 4; }
+
+// R: elements of a column per lane (TL*R >= m).  Slots past the column's end are computed and thrown away, so the host picks, among R = 2 ... 8
+// (and 10, 12, 16 for the one-input fp32 kernels), the pair that wastes fewest: ten classes run as one lane x 10, 21 as 2 lanes x 12.
 template <typename T, typename Algo, bool VEC, int R>
 __global__ __launch_bounds__(256) void softmax_short_kernel(int m, long n, int G, int TL, const T* a, const T* b, T* out, const int* labels, T scale,
                                                             T* loss) {
   constexpr bool kTwo = Algo::kInputs == 2;
   constexpr int NV = VEC ? Vec16<T>::N : 1;
-  constexpr int Q = 4;
-  constexpr int CAP = 256 * Q * Vec16<T>::N;     // elements of a stretch: 16 KB
+  constexpr int Q = short_stretch_vectors<T, Algo>();
+  constexpr int CAP = 256 * Q * Vec16<T>::N;     // elements of a stretch
   typedef typename Vec16<T>::type V;
   __shared__ T la[CAP + CAP / 32];
   __shared__ T lb[kTwo ? CAP + CAP / 32 : 1];
@@ -987,7 +994,7 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
 #define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
   if (m <= kShortRows && n >= 64 && !(resident_cap > 0 && m > resident_cap)) {
     // stretches of whole columns (see softmax_short_kernel): G columns per workgroup, starting on 16-byte boundaries on the vector path
-    constexpr int cap = 256 * 4 * N;
+    constexpr int cap = 256 * short_stretch_vectors<T, Algo>() * N;
     const bool v16 = ma == 0 && mo == 0 && mb == 0;
     long G = cap / m;
     if (v16) {
@@ -997,14 +1004,19 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
       G = G / step * step;
     }
     // (a matrix too small for sixteen workgroups stays with one wave per column: one launch is 2.8 us there against 3.5 us through LDS)
-    if (G >= 1 && n >= 16 * G) {
+    if (G >= 1 && n * m >= 16L * 256 * 4 * N) {
       // lanes per column and elements per lane: cheapest passes over the workgroup's G columns, a pass costing its R slots plus about six slots' worth
-      // of reductions and bookkeeping (measured: ten classes are faster as 2 lanes x 8 in four passes than as 4 x 3 in seven)
-      // The stretch is cut to a whole number of passes when that costs less per column than a last pass with idle teams.
+      // of reductions and bookkeeping (measured: ten classes are faster as 2 lanes x 8 in four passes than as 4 x 3 in seven, and faster still as
+      // one lane x 10 in one).  The stretch is cut to a whole number of passes when that costs less per column than a last pass with idle teams.
+      // More than eight slots per lane pay only in the one-input fp32 kernels (fp32 logsoftmax, 2^23 elements, cold: m = 10 16.9 -> 14.6 us, 21 17.8 ->
+      // 15.0, 40 18.4 -> 14.8, 100 17.9 -> 15.7; fp64, whose slots take two registers each, and the two-input kernels with their short stretches gain
+      // nothing or lose); sixteen slots lose where eight cover the column exactly (m = 16, 32, 64, 128: 11.9-12.9 us with eight, 14.4-15.3 with sixteen).
+      constexpr bool kManySlots = sizeof(T) == 4 && Algo::kInputs == 1;
       int bestR = 8, bestTL = kWave;
       long bestG = G;
       double best = -1;
-      for (int R : {8, 6, 4, 3, 2}) {
+      for (int R : {16, 12, 10, 8, 7, 6, 5, 4, 3, 2}) {
+        if (R > 8 && (!kManySlots || (R == 16 && (m & (m - 1)) == 0))) continue;
         int TL = 1;
         while (TL < kWave && (long)TL * R < m) TL <<= 1;
         if ((long)TL * R < m) continue;
@@ -1019,8 +1031,16 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
       const dim3 grid((unsigned)((n + G - 1) / G));
 #define KNET8_SHORT(VEC, R) hipLaunchKernelGGL((softmax_short_kernel<T, Algo, VEC, R>), grid, dim3(256), 0, stream, (int)m, n, (int)G, bestTL, a, b, out, labels, scale, loss)
       if (v16) {
-        switch (bestR) { case 2: KNET8_SHORT(true, 2); break; case 3: KNET8_SHORT(true, 3); break; case 4: KNET8_SHORT(true, 4); break;
-                         case 6: KNET8_SHORT(true, 6); break; default: KNET8_SHORT(true, 8); }
+        bool launched = false;
+        if constexpr (kManySlots) {
+          launched = true;
+          switch (bestR) { case 10: KNET8_SHORT(true, 10); break; case 12: KNET8_SHORT(true, 12); break; case 16: KNET8_SHORT(true, 16); break;
+                           default: launched = false; }
+        }
+        if (!launched)
+          switch (bestR) { case 2: KNET8_SHORT(true, 2); break; case 3: KNET8_SHORT(true, 3); break; case 4: KNET8_SHORT(true, 4); break;
+                           case 5: KNET8_SHORT(true, 5); break; case 6: KNET8_SHORT(true, 6); break; case 7: KNET8_SHORT(true, 7); break;
+                           default: KNET8_SHORT(true, 8); }
       } else {
         int TL = 1;   // operands that are not all on 16-byte boundaries: the one general variant
         while (TL < kWave && TL * 8 < m) TL <<= 1;
