@@ -486,6 +486,10 @@ __global__ __launch_bounds__(TEAM) __attribute__((amdgpu_waves_per_eu(4, 4))) vo
 // and puts the results back in place.  The same Algo table as the register-resident kernels; the fused nll variant uses the plain two-reduction
 // form (max, then sum of exp), one exp per element.
 constexpr int kShortRows = 128;
+// The fused nll kernel goes this way up to 192 rows: beyond 128 rows one wave per column leaves half its lanes idle in a kernel with two reductions
+// (2^23 elements, cold, wave per column -> stretches: fp32 130 rows 26.5 -> 19.0 us, 160 21.5 -> 17.1, 192 19.1 -> 16.5, 256 15.9 -> 15.2, 300 16.9 -> 17.7;
+// fp64 130 rows 58 -> 45, 192 40 -> 36, 256 32 -> 34).  The other kernels are as fast or faster with a wave per column from 160 rows on.
+constexpr int kShortRowsNll = 192;
 // LDS layout: one padding word after every 32 entries, so that the teams of a wave, whose columns start m entries apart, do not meet in one bank
 // when m is a power of two.  (Four padding words, which would keep a 16-byte vector whole and aligned for the stretch's way in and out, measured
 // slower: 17 us against 12.4 us at m = 32: the column pass is the one that counts.)
@@ -992,7 +996,7 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   const bool vec_stream = (m % N == 0) && ma == 0 && mo == 0 && mb == 0;
   const long resident_cap = tuning(kTuneSoftmaxResidentRows);  // 0: no limit below the register capacity (tests lower it to reach the streaming kernel with short columns)
 #define KNET8_SM(TEAM, E) launch_softmax_cfg<T, Algo, TEAM, E>(stream, vec, (int)m, n, a, b, out, labels, scale, loss)
-  if (m <= kShortRows && n >= 64 && !(resident_cap > 0 && m > resident_cap)) {
+  if (m <= (Algo::kNll ? kShortRowsNll : kShortRows) && n >= 64 && !(resident_cap > 0 && m > resident_cap)) {
     // stretches of whole columns (see softmax_short_kernel): G columns per workgroup, starting on 16-byte boundaries on the vector path
     constexpr int cap = 256 * short_stretch_vectors<T, Algo>() * N;
     const bool v16 = ma == 0 && mo == 0 && mb == 0;

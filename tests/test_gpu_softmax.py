@@ -91,7 +91,7 @@ def test_columns_held_partly_in_lds(knet, oracle):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_many_short_columns(knet, oracle, dt):
-    """Columns of at most 128 rows, enough of them for sixteen workgroups: workgroups take stretches of whole columns through LDS.  Column lengths around every
+    """Columns of at most 128 rows (192 for the fused nll), enough of them for sixteen workgroups: workgroups take stretches of whole columns through LDS.  Column lengths around every
     lanes-per-column choice, a last stretch that is not full, column counts that leave one column over, and operands off the 16-byte grid (the
     general variant); every function of the family, the fused nll with a skipped instance."""
     from gpu_util import misaligned
@@ -99,7 +99,7 @@ def test_many_short_columns(knet, oracle, dt):
     rtol = 1e-5 if dt == np.float32 else 1e-12
     # (sixteen stretches of 16 KB and more: smaller matrices stay with one wave per column, which the other tests cover)
     for m, n in ((1, 70000), (2, 40001), (3, 24000), (5, 14000), (8, 9000), (10, 7001), (16, 4500), (21, 3300), (32, 2100), (33, 2100), (64, 1100),
-                 (100, 700), (127, 600), (128, 513), (10, 100)):
+                 (100, 700), (127, 600), (128, 513), (10, 100), (129, 600), (160, 450), (191, 400), (192, 401), (193, 400)):
         x = (rng.standard_normal((m, n)) * 2).astype(dt)
         dy = rng.standard_normal((m, n)).astype(dt)
         for off in (0, 1):
