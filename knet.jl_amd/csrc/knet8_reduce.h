@@ -235,7 +235,8 @@ __global__ __launch_bounds__(BT) void reduce_strided_kernel(const T* __restrict_
 template <typename T, typename Op, int NV, int U, int O>
 __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __restrict__ x, int sy, int g_full, long nout, int R, int TL, long group_stride,
                                                                   long iter_stride, long iters, long iters_per_part, long limit, unsigned P,
-                                                                  T* __restrict__ y, T* partial, unsigned* counters) {
+                                                                  T* __restrict__ y, T* partial, unsigned* counters KNET8_TL_PARAM) {
+  KNET8_TL_BEGIN
   constexpr int CAP = kRedBlock * U * NV;
   __shared__ T lds[CAP + CAP / 32];
   __shared__ unsigned flag;
@@ -286,6 +287,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
 #pragma unroll
         for (int e = 0; e < NV; e++) acc[q][e] = Op::merge(acc[q][e], v[o][q][e]);
   }
+  KNET8_TL_MID
   // one padding word per 32 entries: a team walks entries TL apart, neighbouring teams start sy apart
 #pragma unroll
   for (int q = 0; q < U; q++)
@@ -301,19 +303,27 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
   for (int jb = 0; jb < g; jb += nteams) {   // the same trip count for every lane of a wave: the shuffles below need all of them
     const int jl = jb + team;
     T r = Op::init();
-    if (jl < g)
-      for (int c = tl; c < entries; c += TL) {
-        const int i = R == 1 ? jl * sy + c : ((c / sy) * g + jl) * sy + c % sy;   // (one slab per stretch: no division per entry)
-        r = Op::merge(r, lds[i + (i >> 5)]);
+    if (jl < g) {
+      if (sy == 1) {   // (slabs of single elements, the strided view: entry c of output jl is element c*g + jl)
+        for (int c = tl; c < entries; c += TL) {
+          const int i = c * g + jl;
+          r = Op::merge(r, lds[i + (i >> 5)]);
+        }
+      } else {
+        for (int c = tl; c < entries; c += TL) {
+          const int i = R == 1 ? jl * sy + c : ((c / sy) * g + jl) * sy + c % sy;   // (one slab per stretch: no division per entry)
+          r = Op::merge(r, lds[i + (i >> 5)]);
+        }
       }
+    }
     for (int o = TL >> 1; o > 0; o >>= 1) r = Op::merge(r, __shfl_xor(r, o));
     if (jl < g && tl == 0) {
       if (P > 1) st_coherent(mine + jl, r);
       else mine[jl] = r;
     }
   }
-  if (P == 1) return;
-  if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) return;
+  if (P == 1) { KNET8_TL_END return; }
+  if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) { KNET8_TL_END return; }
   // Combine: 256/gp lanes per output share the P partials (one lane alone would wait for P memory round trips in a row), eight loads in flight each;
   // their sums meet in LDS in fixed order.
   int gp = 1;
@@ -344,6 +354,7 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
     }
   }
   if (threadIdx.x == 0) st_coherent(counters + group * kTicketStride, 0u);
+  KNET8_TL_END
 }
 
 // ---- host-side planning ----------------------------------------------------------------------------
@@ -411,10 +422,14 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   const long entries = (long)R * sy;
   int TL = 1;
   while (TL < kWave && TL * 8 < entries) TL <<= 1;
-  // parts: about four workgroups per compute unit (measured best of 2, 4, 8, 16), at least eight stretches each, and the combining pass reads g*P partials
+  // parts: about two workgroups per compute unit, at least eight stretches each, and the combining pass reads g*P partials.  Every workgroup is resident
+  // from the start and all finish their stretches at about the same time; what follows (partial results written through, ticket, the last one's
+  // combining pass) are memory round trips behind everybody else's last loads, and they get longer with the number of workgroups.  Stamps on
+  // (8, 4M) and (32, 1M) summed over the long axis, cold: two per CU have their sums after 15-21 us and are done after 27-29 us, four per CU after 12-26 us
+  // and 32-36 us; back to back (2..32 rows) x 2^25 elements: 33.5 / 31.6 / 44.0 / 32.6 us with one per CU, 30.1 / 28.0 / 34.9 / 30.1 with two, 33.1 / 33.0 / 36.6 / 37.4 with four.
   const long ncu = tuning(kTuneNumCUs);
   long P = 1;
-  if (groups < 4 * ncu) P = 4 * ncu / groups;
+  if (groups < 2 * ncu) P = 2 * ncu / groups;
   if (P > iters / 8) P = iters / 8;
   if (P * g > 65536) P = 65536 / g;
   if (P < 1 || !scratch_fits(scratch, sizeof(T) * (size_t)groups * P * g, (size_t)groups * kTicketStride)) P = 1;   // a provider of fixed size: no split beyond it
@@ -428,7 +443,7 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   const dim3 grid((unsigned)(groups * P));
 #define KNET8_STRETCH(NV, U, O) \
   hipLaunchKernelGGL((reduce_stretch_kernel<T, Op, NV, U, O>), grid, dim3(kRedBlock), 0, stream, x, (int)sy, g, whole ? nb * ny : ny, R, TL, group_stride, \
-                     iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters)
+                     iter_stride, iters, ipp, limit, (unsigned)P, y, static_cast<T*>(ws.partial), ws.counters KNET8_TL_ARG)
   if (single) { if (vec) KNET8_STRETCH(N, SV, 1); else KNET8_STRETCH(1, S1, 1); }
   else        { if (vec) KNET8_STRETCH(N, UV, 4); else KNET8_STRETCH(1, U1, 4); }
 #undef KNET8_STRETCH
