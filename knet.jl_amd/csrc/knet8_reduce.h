@@ -322,9 +322,10 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
       else mine[jl] = r;
     }
   }
-  if (P == 1) { KNET8_TL_END return; }
+  if (P == 1 || O == 1) { KNET8_TL_END return; }   // (O == 1: launches of one stretch per workgroup are never split; their registers stay what the walk needs)
   if (!last_block_ticket(counters + group * kTicketStride, P, &flag)) { KNET8_TL_END return; }
-  // Combine: 256/gp lanes per output share the P partials (one lane alone would wait for P memory round trips in a row), eight loads in flight each;
+  // Combine: 256/gp lanes per output share the P partials (one lane alone would wait for P memory round trips in a row), 32 loads in flight each
+  // (512 parts of 64 outputs are 128 partials per lane: four round trips instead of sixteen; (64, 512K) summed over the long axis 32.5 -> 29.4 us);
   // their sums meet in LDS in fixed order.
   int gp = 1;
   while (gp < g && gp < kRedBlock) gp <<= 1;
@@ -335,6 +336,14 @@ __global__ __launch_bounds__(kRedBlock) void reduce_stretch_kernel(const T* __re
     if (jl < g) {
       const T* pj = partial + group * P * g_full + jl;
       unsigned q = threadIdx.x / gp;
+      constexpr int B = 32;
+      for (; q + (B - 1) * tlc < P; q += B * tlc) {
+        T v[B];
+#pragma unroll
+        for (int k = 0; k < B; k++) v[k] = ld_coherent(pj + (long)(q + k * tlc) * g_full);
+#pragma unroll
+        for (int k = 0; k < B; k++) r = Op::merge(r, v[k]);
+      }
       for (; q + 7 * tlc < P; q += 8 * tlc) {
         T v[8];
 #pragma unroll
@@ -518,7 +527,10 @@ inline bool launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   constexpr int N = Vec16<T>::N;
   // a short contiguous axis: lanes along `a` alone would idle most of a wave; whole (s1 x R) slabs per stretch instead
   bool launched = true;
-  if (s1 < kWave && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch, &launched)) return launched;
+  // (up to 72 elements in fp32, where a row of 64 to 72 elements still leaves three quarters of a wave's 16-byte lanes idle: 2^25 elements, cold, strided kernel ->
+  //  stretches: 64 rows 44.6 -> 29.4 us, 68 43.1 -> 39.5, 72 41.4 -> 34.9; from 80 rows on, and in fp64 from 64 on, the strided kernel is faster)
+  const long short_axis = sizeof(T) == 4 ? 72 : kWave - 1;
+  if (s1 <= short_axis && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch, &launched)) return launched;
   const bool vec = aligned16(x) && (s1 % N == 0);
   // rows that do not start on 16-byte boundaries: the same tile width from N interleaved 4- or 8-byte loads per lane
   const long tile = (long)kWave * N;
