@@ -115,7 +115,8 @@ def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
         # (a contiguous axis of up to 72 elements goes this way in fp32, of up to 63 in fp64: lengths on both sides of both limits, with enough rows for a split
         #  whose combining pass has more than 32 partial results per lane, and for one with fewer)
         for (s1, d, nb) in [(2, 1000001, 1), (32, 65536, 1), (63, 1000, 1), (5, 1000, 7), (3, 999, 4), (1, 100000, 3), (16, 3, 2), (7, 300000, 1),
-                            (64, 40000, 1), (65, 9000, 1), (72, 30011, 1), (73, 3000, 1), (48, 70000, 1), (72, 50, 3)]:
+                            (64, 40000, 1), (65, 9000, 1), (72, 30011, 1), (73, 3000, 1), (48, 70000, 1), (72, 50, 3),
+                            (100, 40000, 1), (128, 33001, 1), (132, 33000, 1)]:   # (rows of at most 512 bytes, long enough for the 1024-lane kernel: four rows in flight per wave)
             x = rng.integers(-4, 5, size=(s1, d, nb)).astype(dt)
             for off in (0, 1):
                 xd = misaligned(knet, x, off)
