@@ -99,7 +99,8 @@ def test_many_short_columns(knet, oracle, dt):
     rtol = 1e-5 if dt == np.float32 else 1e-12
     # (sixteen stretches of 16 KB and more: smaller matrices stay with one wave per column, which the other tests cover)
     for m, n in ((1, 70000), (2, 40001), (3, 24000), (5, 14000), (8, 9000), (10, 7001), (16, 4500), (21, 3300), (32, 2100), (33, 2100), (64, 1100),
-                 (100, 700), (127, 600), (128, 513), (10, 100), (129, 600), (160, 450), (191, 400), (192, 401), (193, 400)):
+                 (100, 700), (127, 600), (128, 513), (10, 100), (129, 600), (160, 450), (191, 400), (192, 401), (193, 400),
+                 (7, 10000), (12, 6000), (20, 4000), (24, 3000), (40, 2000), (50, 1400), (56, 1300), (80, 900)):   # (every slots-per-lane variant the planner can pick)
         x = (rng.standard_normal((m, n)) * 2).astype(dt)
         dy = rng.standard_normal((m, n)).astype(dt)
         for off in (0, 1):
