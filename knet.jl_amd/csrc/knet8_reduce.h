@@ -497,8 +497,15 @@ inline bool launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   // neighbouring runs instead.  Many slabs (the bias gradient of a 7x7 feature map, x(49, 2048, N)): the slabs are first added onto each other as
   // rows of sy*ny contiguous elements by the strided-view kernel, into scratch, then the sy*ny sums are reduced as one slab; the sy*ny extra
   // elements written and read are nothing next to the no slabs.  (Measured, 134 MB fp32: (4,1000,8388) 158 -> 26.5 us, (49,2048,334) 43.7 -> 28.5 us, (16,16,131072) 35.9 -> 29.0 us.)
+  // Neither pays below a size that grows with the run length: the two passes cost 8.5-9.5 us before the first byte (two launches, the first one split) and 0.13 us per MB
+  // after it, the run kernel below 3.5 us and 2.3 / 1.5 / 0.6 / 0.45 / 0.34 us per MB at runs of 2 / 4 / 8 / 12 / 16 and more elements -- and the bias gradient of a
+  // convolution layer is a few MB.  Measured crossovers (fp32, 512 outputs): runs of 2: 2.5 MB, 4: 4 MB, 8: 11 MB, 12: 15 MB, 16 to 63: 22-48 MB.  Below 1.25 MB per
+  // element of the run (at most 24 MB) the array goes to the run kernel: x(16,512,128) 9.0 -> 3.8 us, x(49,512,64) 9.0 -> 6.3, x(4,512,61) 7.0 -> 3.7, x(8,512,122) 9.4 -> 4.0.
+  const size_t total_bytes = sizeof(T) * (size_t)sy * (size_t)ny * (size_t)no;
+  const size_t two_pass_from = sy < 20 ? (size_t)sy * 1310720 : (size_t(24) << 20);
+  const bool small_total = no > 1 && sy < kWave && total_bytes < two_pass_from;
   const size_t front = (sizeof(T) * (size_t)(sy * ny) + 255) / 256 * 256;
-  if (ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave && front <= kTwoPassMaxBytes && scratch_fits(scratch, 2 * front, 0)) {
+  if (!small_total && ny > 1 && sy < kWave && no >= 8 && sy * ny >= kWave && front <= kTwoPassMaxBytes && scratch_fits(scratch, 2 * front, 0)) {
     Workspace tw = take_scratch(scratch, stream, front, 0);
     if (tw.partial == nullptr) { record_error("reduction: no scratch memory for the slab sums"); return false; }
     T* tmp = static_cast<T*>(tw.partial);
@@ -511,7 +518,7 @@ inline bool launch_reduce_run(hipStream_t stream, const T* x, long sy, long ny, 
   constexpr int NR = Vec16<T>::N;
   const bool short_one_slab = no == 1 && (sy <= 256 || (sy <= kStretchMaxRun && (sy % NR != 0 || !aligned16(x))));
   bool launched = true;
-  if (ny > 1 && (sy <= 8 || short_one_slab) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch, &launched)) return launched;
+  if (!small_total && ny > 1 && (sy <= 8 || short_one_slab) && launch_reduce_stretch<T, Op>(stream, x, sy, ny, no, 1, 0, y, scratch, &launched)) return launched;
   constexpr int N = Vec16<T>::N;
   const bool vec = aligned16(x) && (sy % N == 0);
   const int nv = vec ? N : 1;

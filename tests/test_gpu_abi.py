@@ -377,7 +377,7 @@ def test_split_launch_without_scratch_is_refused_on_the_host(knet):
         dz = knet.KnetArray(dtype=np.float32, dims=(256, 4096))
         fn["reluback_biasgrad_32_stream"](256, 4096, dyd.ptr, yd.ptr, dz.ptr, out.ptr, lib.stream)
 
-    x3 = rng.integers(-3, 4, size=(4, 1000, 50)).astype(np.float32)      # many slabs of short runs: two passes, the slab sums in scratch
+    x3 = rng.integers(-3, 4, size=(4, 1000, 400)).astype(np.float32)     # many slabs of short runs, 6.4 MB (smaller arrays go to the run kernel): two passes, the slab sums in scratch
     x3d = knet.KnetArray(x3)
 
     def sum_two_pass(out):

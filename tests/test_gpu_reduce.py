@@ -100,7 +100,10 @@ def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
     for dt, S in ((np.float32, "32"), (np.float64, "64")):
         runs = [(2, 100001, 1), (8, 4096, 1), (10, 100000, 1), (128, 777, 1), (3, 5, 1), (100, 3355, 1), (127, 40, 1), (64, 2049, 1),
                 (4, 1000, 50), (8, 3, 1000), (2, 2, 100000), (7, 5, 333), (1, 3, 70000), (5, 600, 41), (8, 1, 5), (6, 100000, 3),
-                (129, 300, 1), (256, 100, 1), (257, 101, 1), (513, 50, 1), (1001, 21, 1), (1023, 9, 1), (1024, 9, 1)]
+                (129, 300, 1), (256, 100, 1), (257, 101, 1), (513, 50, 1), (1001, 21, 1), (1023, 9, 1), (1024, 9, 1),
+                # (arrays of less than 1.25 MB per element of the run go to the run kernel whatever the run length: larger ones for the two-pass route and the stretches over
+                #  several slabs, and one on either side of the limit)
+                (4, 1000, 500), (6, 100000, 4), (2, 2, 1000000), (16, 512, 700), (9, 300, 1000), (9, 300, 1300), (49, 512, 300)]
         for (sy, ny, no) in runs:
             x = rng.integers(-4, 5, size=(sy, ny, no)).astype(dt)
             x[x == 0] = 1 if x.size < 2000 else 0
