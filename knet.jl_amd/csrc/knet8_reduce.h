@@ -453,7 +453,7 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   const long entries = (long)R * sy;
   int TL = 1;
   while (TL < kWave && TL * 8 < entries) TL <<= 1;
-  // parts: about two workgroups per compute unit, at least eight stretches each, and the combining pass reads g*P partials.  Every workgroup is resident
+  // parts: about two workgroups per compute unit, a minimum of stretches each (below), and the combining pass reads g*P partials.  Every workgroup is resident
   // from the start and all finish their stretches at about the same time; what follows (partial results written through, ticket, the last one's
   // combining pass) are memory round trips behind everybody else's last loads, and they get longer with the number of workgroups.  Stamps on
   // (8, 4M) and (32, 1M) summed over the long axis, cold: two per CU have their sums after 15-21 us and are done after 27-29 us, four per CU after 12-26 us
@@ -461,7 +461,10 @@ inline bool launch_reduce_stretch(hipStream_t stream, const T* x, long sy, long 
   const long ncu = tuning(kTuneNumCUs);
   long P = 1;
   if (groups < 2 * ncu) P = 2 * ncu / groups;
-  if (P > iters / 8) P = iters / 8;
+  // (at least eight stretches per part; two in arrays of less than 8 MB, where the parts' walks are the longest thing in the launch: (10, 25000) 8.9 -> 7.5 us,
+  //  (32, 1953) 8.0 -> 6.3, (2, 125000) 9.7 -> 7.9; from 16 MB on eight are faster, 12.4 against 14.6-15.6)
+  const long per_part = sizeof(T) * (size_t)iters * (size_t)iter_stride * (size_t)groups < (size_t(8) << 20) ? 2 : 8;
+  if (P > iters / per_part) P = iters / per_part;
   if (P * g > 65536) P = 65536 / g;
   if (P < 1 || !scratch_fits(scratch, sizeof(T) * (size_t)groups * P * g, (size_t)groups * kTicketStride)) P = 1;   // a provider of fixed size: no split beyond it
   long ipp = ceil_div(iters, P);
