@@ -411,7 +411,7 @@ def test_two_pass_reduction_whose_first_pass_is_refused_leaves_the_output_alone(
     lib = knet.libknet8()
     fn = lib.fn
     rng = np.random.default_rng(57)
-    x = rng.integers(-3, 4, size=(4, 2000, 4000)).astype(np.float32)     # first pass: 32 row tiles x 62 parts = 2 MB of partial results
+    x = rng.integers(-3, 4, size=(4, 2000, 4000)).astype(np.float32)     # first pass: 32 row tiles x 64 parts = 2 MB of partial results
     xd = knet.KnetArray(x)
     out = knet.KnetArray(np.full(2000, -777.0, np.float32))
     old = fn["knet8_tune"](0, 1 << 20)

@@ -87,12 +87,12 @@ def test_no_alloc_sum_refuses_a_split_beyond_its_array(knet):
     lib = knet.libknet8()
     fn = lib.fn
     rng = np.random.default_rng(78)
-    x = rng.standard_normal((4096, 8192)).astype(np.float32)
+    x = rng.standard_normal((8192, 8192)).astype(np.float32)
     xd = knet.KnetArray(x)
-    out = knet.KnetArray(np.full(4096, -555.0, np.float32))
-    old = fn["knet8_tune"](0, 1 << 20)       # a planner told of 2^20 compute units cuts the columns into 128 parts per row tile: 2 MiB of partials
+    out = knet.KnetArray(np.full(8192, -555.0, np.float32))
+    old = fn["knet8_tune"](0, 1 << 20)       # a planner told of 2^20 compute units cuts the columns of each of the 32 row tiles into 64 parts: 2 MiB of partials
     try:
-        fn["sum_32_21_noalloc"](x.size, xd.ptr, 1, 4096, out.ptr, lib.stream)
+        fn["sum_32_21_noalloc"](x.size, xd.ptr, 1, 8192, out.ptr, lib.stream)
         assert fn["knet8_synchronize"](lib.stream) == 0
         msg = fn["knet8_last_error"]()
     finally:
@@ -100,7 +100,7 @@ def test_no_alloc_sum_refuses_a_split_beyond_its_array(knet):
     assert msg is not None and b"sum_32_21_noalloc" in msg and b"fixed scratch" in msg, msg
     assert np.all(knet.Array(out) == np.float32(-555.0))
     # and the next call is fine
-    fn["sum_32_21_noalloc"](x.size, xd.ptr, 1, 4096, out.ptr, lib.stream)
+    fn["sum_32_21_noalloc"](x.size, xd.ptr, 1, 8192, out.ptr, lib.stream)
     knet.synchronize()
     lib.check()
     assert np.all(np.abs(knet.Array(out) - x.astype(np.float64).sum(axis=1)) <= 1e-5 * np.abs(x).astype(np.float64).sum(axis=1))
