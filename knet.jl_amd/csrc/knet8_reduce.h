@@ -407,6 +407,27 @@ inline unsigned plan_parts(long groups, long units_per_group, long min_units_per
   return (unsigned)P;
 }
 
+// Parts of a split along an axis of d rows (or columns) per group, chosen by counting dependent memory round trips: a part's waves walk `per_trip` rows
+// per trip (sixteen waves with two rows in flight, or four with eight), the ticket costs two trips, and the workgroup that combines reads 128 partial rows
+// per trip when it has sixteen waves (parts of at least `big_from` rows) and 32 with four.  At most one workgroup per compute unit, parts of at least 16 rows.
+inline unsigned plan_parts_by_trips(long groups, long d, long per_trip, long big_from) {
+  const long ncu = tuning(kTuneNumCUs);
+  long pmax = groups * 2 <= ncu ? ncu / groups : 1;
+  if (pmax > d / 16) pmax = d / 16;
+  if (pmax > 65535) pmax = 65535;
+  auto trips = [&](long p) {
+    const long rows = ceil_div(d, p);
+    return ceil_div(rows, per_trip) + (p > 1 ? ceil_div(p, rows >= big_from ? 128 : 32) + 2 : 0);
+  };
+  long best = trips(1);
+  unsigned P = 1;
+  for (long p = 2; p <= pmax; p = (p * 2 <= pmax || p == pmax) ? p * 2 : pmax) {
+    const long t = trips(p);
+    if (t < best) { best = t; P = (unsigned)p; }
+  }
+  return P;
+}
+
 constexpr long kStretchMaxRun = 1024;   // longest run the stretch kernel takes
 
 // Stretch kernel for x(sy, ny, no) -> y(ny) per batch (nb batches, `batch_stride` elements apart, outputs ny apart); sy*ny small enough for
@@ -568,26 +589,10 @@ inline bool launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   const long tile = (long)kWave * N;
   const long atiles = ceil_div(s1, tile);
   const long groups = atiles * nb;
-  // Parts per tile, counted in memory round trips: a part's waves walk 32 rows per trip (sixteen waves with two rows in flight, or four with eight), the
-  // ticket costs two, and the workgroup that combines reads 128 partial rows per trip (32 with four waves).  Few parts of long walks and many parts with a
-  // long combining pass both lose: (256, 8192) 8.6 us with 128 parts, 7.0 with 64, 11.8 with 256; (1000, 128) 5.3 us with 2 parts, 4.6 with 4, 4.8 with 1;
-  // (4096, 512) 5.9 -> 5.4.  Large arrays end up where the bound of one workgroup per compute unit puts them, as before.
-  unsigned P = 1;
-  {
-    const long ncu = tuning(kTuneNumCUs);
-    long pmax = groups * 2 <= ncu ? ncu / groups : 1;
-    if (pmax > d / 16) pmax = d / 16;
-    if (pmax > 65535) pmax = 65535;
-    auto trips = [&](long p) {
-      const long rows = ceil_div(d, p);
-      return ceil_div(rows, 32) + (p > 1 ? ceil_div(p, rows >= 128 ? 128 : 32) + 2 : 0);
-    };
-    long best = trips(1);
-    for (long p = 2; p <= pmax; p = (p * 2 <= pmax || p == pmax) ? p * 2 : pmax) {
-      const long t = trips(p);
-      if (t < best) { best = t; P = (unsigned)p; }
-    }
-  }
+  // Parts per tile, counted in memory round trips (plan_parts_by_trips): few parts of long walks and many parts with a long combining pass both lose:
+  // (256, 8192) 8.6 us with 128 parts, 7.0 with 64, 11.8 with 256; (1000, 128) 5.3 us with 2 parts, 4.6 with 4, 4.8 with 1; (4096, 512) 5.9 -> 5.4.
+  // Large arrays end up where the bound of one workgroup per compute unit puts them, as before.
+  unsigned P = plan_parts_by_trips(groups, d, 32, 128);
   long kchunk = ceil_div(d, P);
   P = (unsigned)ceil_div(d, kchunk > 0 ? kchunk : 1);
   if (P < 1) P = 1;
