@@ -580,10 +580,13 @@ inline bool launch_reduce_strided(hipStream_t stream, const T* x, long s1, long 
   constexpr int N = Vec16<T>::N;
   // a short contiguous axis: lanes along `a` alone would idle most of a wave; whole (s1 x R) slabs per stretch instead
   bool launched = true;
-  // (up to 72 elements in fp32, where a row of 64 to 72 elements still leaves three quarters of a wave's 16-byte lanes idle: 2^25 elements, cold, strided kernel ->
-  //  stretches: 64 rows 44.6 -> 29.4 us, 68 43.1 -> 39.5, 72 41.4 -> 34.9; from 80 rows on, and in fp64 from 64 on, the strided kernel is faster)
-  const long short_axis = sizeof(T) == 4 ? 72 : kWave - 1;
-  if (s1 <= short_axis && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch, &launched)) return launched;
+  // By the bytes of a row: up to 128 always; up to 192 (256) in arrays of at least 48 (96) MB -- in smaller ones, and for longer rows, the strided kernel below with its
+  // parts planned by round trips is faster.  Measured, stretches / strided kernel, fp32: 32 columns x 4 MB 9.1 / 8.2 us, x 16 MB 12.3 / 13.6, x 134 MB 27.9 / 52.7;
+  // 48 x 4 MB 9.1 / 7.5, x 64 MB 22.1 / 23.2, x 134 MB 31.8 / 39.1; 64 x 16 MB 13.2 / 11.4, x 64 MB 21.1 / 20.1, x 134 MB 29.2 / 32.3; 72 x 134 MB 34.1 / 30.5;
+  // fp64: 16 x 16 MB 12.1 / 13.7; 24 x 16 MB 12.4 / 12.0, x 64 MB 21.6 / 23.1; 32 x 64 MB 21.3 / 20.1, x 134 MB 28.8 / 32.3; 48 x 134 MB 33.2 / 26.8.
+  const size_t row_bytes = (size_t)s1 * sizeof(T), array_bytes = row_bytes * (size_t)d * (size_t)nb;
+  const bool short_axis = row_bytes <= 128 || (row_bytes <= 192 && array_bytes >= (size_t(48) << 20)) || (row_bytes <= 256 && array_bytes >= (size_t(96) << 20));
+  if (short_axis && launch_reduce_stretch<T, Op>(stream, x, 1, s1, d, nb, s1 * d, y, scratch, &launched)) return launched;
   const bool vec = aligned16(x) && (s1 % N == 0);
   // rows that do not start on 16-byte boundaries: the same tile width from N interleaved 4- or 8-byte loads per lane
   const long tile = (long)kWave * N;

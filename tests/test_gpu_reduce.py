@@ -92,8 +92,8 @@ def test_raw_21_and_22_entry_points_on_odd_shapes_and_misaligned_views(knet, ora
 
 
 def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
-    """Shapes that go to the stretch kernel: runs of at most 256 elements with one slab (1024 when they do not start on 16-byte boundaries), runs of at most 8 with many, a contiguous axis shorter than
-    a wave (fp32: of up to 72 elements).  Groups with a tail, whole slabs with a last partial stretch, sizes that are and are not multiples of a 16-byte vector, batches, split
+    """Shapes that go to the stretch kernel: runs of at most 256 elements with one slab (1024 when they do not start on 16-byte boundaries), runs of at most 8 with many, a contiguous axis of at most
+    128 bytes (256 in large arrays).  Groups with a tail, whole slabs with a last partial stretch, sizes that are and are not multiples of a 16-byte vector, batches, split
     launches (enough stretches for several parts), base pointers off the 16-byte grid; every operator, exact on integer-valued data."""
     from gpu_util import misaligned
     rng = np.random.default_rng(26)
@@ -115,11 +115,11 @@ def test_stretches_of_short_runs_and_short_contiguous_axes(knet, oracle):
                     knet.knet8("%s_%s_21" % (op, S), x.size, xd.ptr, sy, ny, y.ptr)
                     want = oracle.reduce(op, x, dims=(1, 3)).ravel()
                     assert np.array_equal(knet.Array(y), want), (op, sy, ny, no, off)
-        # (a contiguous axis of up to 72 elements goes this way in fp32, of up to 63 in fp64: lengths on both sides of both limits, with enough rows for a split
-        #  whose combining pass has more than 32 partial results per lane, and for one with fewer)
+        # (a contiguous axis goes this way by the bytes of a row: up to 128 always, up to 192 in arrays of at least 48 MB, up to 256 in arrays of at least 96 MB: lengths and
+        #  sizes on both sides of the limits, with enough rows for a split whose combining pass has more than 32 partial results per lane, and for one with fewer)
         for (s1, d, nb) in [(2, 1000001, 1), (32, 65536, 1), (63, 1000, 1), (5, 1000, 7), (3, 999, 4), (1, 100000, 3), (16, 3, 2), (7, 300000, 1),
                             (64, 40000, 1), (65, 9000, 1), (72, 30011, 1), (73, 3000, 1), (48, 70000, 1), (72, 50, 3),
-                            (100, 40000, 1), (128, 33001, 1), (132, 33000, 1)]:   # (rows of at most 512 bytes, long enough for the 1024-lane kernel: four rows in flight per wave)
+                            (100, 40000, 1), (128, 33001, 1), (132, 33000, 1), (48, 262145, 1), (64, 400000, 1), (24, 300000, 1), (33, 100000, 1)]:   # (rows of at most 512 bytes, long enough for the 1024-lane kernel: four rows in flight per wave)
             x = rng.integers(-4, 5, size=(s1, d, nb)).astype(dt)
             for off in (0, 1):
                 xd = misaligned(knet, x, off)
