@@ -86,6 +86,23 @@ def test_index_bounds_and_shape_errors(knet):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_embedding_gradient_at_scale(knet, dt):
+    """addcols at the size of a language model's embedding gradient: 768-row columns of a 20000-word vocabulary, 8192 tokens drawn from a Zipf distribution (a quarter of them
+    the same word), and a number of rows that is not a multiple of anything; integer-valued data, so the sum is exact whatever order the atomics arrive in."""
+    rng = np.random.default_rng(66)
+    for rows, vocab, ntok in ((768, 20000, 8192), (301, 7000, 5000)):
+        idx = np.minimum(rng.zipf(1.3, size=ntok), vocab).astype(np.int64)
+        y = rng.integers(-3, 4, size=(rows, ntok)).astype(dt)
+        x = rng.integers(-9, 10, size=(rows, vocab)).astype(dt)
+        acc = knet.KnetArray(x)
+        knet.addcols_(acc, knet.KnetArray(y), idx)
+        want = x.copy()
+        np.add.at(want.T, idx - 1, y.T)
+        assert bits_equal(knet.Array(acc), want), (rows, vocab, ntok)
+    knet.libknet8().check()
+
+
 def test_embedding_lookup_gradient_through_the_tape(knet):
     rng = np.random.default_rng(62)
     w = rng.integers(-4, 5, size=(16, 50)).astype(np.float32)
