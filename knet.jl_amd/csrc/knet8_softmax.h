@@ -1086,9 +1086,15 @@ inline void launch_softmax(hipStream_t stream, long m, long n, const T* a, const
   //  operands -- 1000 rows x 4096 columns, cold: 19.0 -> 18.1 us; every other kernel and width is 3 to 50 % slower that way, and so is this one below 768 rows)
   else if (m <= 64 * 16) { if (kStreamsA && sizeof(T) == 8 && m > 768) KNET8_SM(256, 4); else KNET8_SM(64, 16); }
   else if (m <= 256 * 16) { if (kStreamsA && m > 2048) KNET8_SM(1024, 8); else KNET8_SM(256, 16); }
-  else if (m <= 1024 * 8) { if constexpr (kWideSingle) KNET8_SM(256, 32); else KNET8_SM(1024, 8); }
-  else if (m <= 1024 * 16) { if constexpr (kWideSingle) KNET8_SM(256, 64); else KNET8_SM(1024, 16); }
-  else if (kWideNll && m <= 256 * 128) { if constexpr (kWideNll) KNET8_SM(256, 128); }
+  // (the 256-lane fp64 teams only with more than 512 columns: with fewer, a column per 1024 lanes keeps more of the chip busy -- (16384, 64) logsoftmax 12.6 -> 11.2 us,
+  //  softmax 14.3 -> 12.0, fused nll 12.3 -> 10.5; (12000, 256) 14.8 -> 13.8 / 14.4 -> 13.5 / 14.4 -> 12.7; at 512 columns the two are level, at 1024 columns of 8192 rows
+  //  the small teams lead 24.1 to 29.7)
+  else if (m <= 1024 * 8) { if (kWideSingle && n > 512) { if constexpr (kWideSingle) KNET8_SM(256, 32); } else KNET8_SM(1024, 8); }
+  else if (m <= 1024 * 16) { if (kWideSingle && n > 512) { if constexpr (kWideSingle) KNET8_SM(256, 64); } else KNET8_SM(1024, 16); }
+  // (the 256-lane fused nll kernel only where it was found: more than 24 K rows and 257 to 512 columns, i.e. a launch between one and two workgroups per compute
+  //  unit.  Everywhere else around it the 1024-lane team is faster: (32000, 32) 9.4 -> 7.2 us, (32000, 128) 10.1 -> 8.0, (32000, 256) 13.9 -> 12.5, (32000, 640) 31.7 -> 29.0,
+  //  (32000, 1024) 48.5 -> 46.5, (17000, 576) 20.8 -> 17.3; against it (32000, 384) 17.9 / 20.2, (28000, 448) 17.7 / 19.0, (32000, 512) 22.3-23.5 / 22.4-22.8)
+  else if (kWideNll && m <= 256 * 128 && m > 24 * 1024 && n > 256 && n <= 512) { if constexpr (kWideNll) KNET8_SM(256, 128); }
   else if (m <= 1024 * (kBig1024 / 2)) KNET8_SM(1024, kBig1024 / 2);
   else KNET8_SM(1024, kBig1024);
 #undef KNET8_SM

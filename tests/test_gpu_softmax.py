@@ -38,6 +38,25 @@ def test_forward_and_backward_over_column_lengths(knet, oracle, dt):
     knet.libknet8().check()
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_mid_length_columns_many_of_them(knet, oracle, dt):
+    """Columns of 4097 to 16384 rows in matrices of more than 512 columns: the team a column gets depends on the number of columns as well (fp64 one-input kernels:
+    256 lanes with more than 512 columns, 1024 lanes with fewer, which the sweep over column lengths above covers with its five columns)."""
+    rng = np.random.default_rng(38)
+    rtol = 1e-5 if dt == np.float32 else 1e-12
+    for m, n in ((6000, 520), (12000, 515)):
+        x = (rng.standard_normal((m, n)) * 2).astype(dt)
+        dy = rng.standard_normal((m, n)).astype(dt)
+        xd, dyd = knet.KnetArray(x), knet.KnetArray(dy)
+        want = oracle.logsoftmax(x, dims=1)
+        assert np.abs(knet.Array(knet.logsoftmax(xd, dims=1)) - want).max() <= rtol * np.abs(want).max(), m
+        y = oracle.softmax(x, dims=1)
+        assert close(knet.Array(knet.softmax(xd, dims=1)), y, rtol), m
+        assert close(knet.Array(knet.logsoftmaxback(knet.KnetArray(want), dyd, dims=1)), oracle.logsoftmaxback(want, dy, dims=1), rtol), m
+        assert close(knet.Array(knet.softmaxback(knet.KnetArray(y), dyd, dims=1)), oracle.softmaxback(y, dy, dims=1), rtol), m
+    knet.libknet8().check()
+
+
 def test_columns_held_partly_in_lds(knet, oracle):
     """fp64 columns of 16385 to 32768 rows: the single-input kernels (logsoftmax, softmax, fused nll) keep 9 of each lane's 32 vectors in LDS.
     Column lengths at both ends of the range, odd lengths (columns start on and off 16-byte boundaries in turn), a skipped instance; checked
@@ -188,7 +207,7 @@ def test_gather_scatter_bit_exact(knet, oracle):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-@pytest.mark.parametrize("C,N", [(10, 100), (3, 2), (1000, 257), (4100, 9), (32000, 6), (70001, 2)])
+@pytest.mark.parametrize("C,N", [(10, 100), (3, 2), (1000, 257), (4100, 9), (32000, 6), (70001, 2), (6000, 600), (12000, 520), (28000, 300), (20000, 300)])
 def test_nll_value_and_gradient_both_paths(knet, oracle, dt, C, N):
     rng = np.random.default_rng(34)
     rtol = 1e-5 if dt == np.float32 else 1e-12
